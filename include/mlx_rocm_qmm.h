@@ -1,0 +1,252 @@
+/*
+ * mlx_rocm_qmm.h -- C ABI of the MI355X (gfx950) implementation of MLX's affine
+ * group-wise quantized matmul path.
+ *
+ * This is the thin layer the C++ `eval_gpu` bodies of a `mlx/backend/rocm` tree
+ * call: plain pointers and sizes, a HIP stream handle, an int status.  Nothing
+ * here allocates or frees device memory except the mlxrocm_malloc family.
+ *
+ * Conventions
+ *   - All data pointers are DEVICE pointers (or host-visible pinned memory).
+ *   - `dtype` is the element type shared by x, scales, biases and out
+ *     (MLX promotes them to one type before the primitive, mlx/ops.cpp:4816-4818).
+ *   - Packed weights are uint32 words; code e of a row occupies bits
+ *     [e*bits, (e+1)*bits) of the row's little-endian bit stream.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Every
+ *     compute entry point only enqueues work and returns.
+ *   - Return value: MLXROCM_OK, or a negative mlxrocm_status; the message of the
+ *     last failure on the calling thread is returned by mlxrocm_last_error().
+ *     No exception crosses this boundary.
+ */
+#ifndef MLX_ROCM_QMM_H
+#define MLX_ROCM_QMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLXROCM_ABI_VERSION 1
+
+typedef enum {
+  MLXROCM_OK = 0,
+  MLXROCM_INVALID_ARGUMENT = -1, /* std::invalid_argument on the C++ side */
+  MLXROCM_UNSUPPORTED = -2,      /* "no ROCm implementation" runtime_error */
+  MLXROCM_HIP_ERROR = -3,        /* a HIP runtime call failed */
+  MLXROCM_OUT_OF_MEMORY = -4
+} mlxrocm_status;
+
+typedef enum {
+  MLXROCM_FLOAT32 = 0,
+  MLXROCM_FLOAT16 = 1,
+  MLXROCM_BFLOAT16 = 2
+} mlxrocm_dtype;
+
+typedef void* mlxrocm_stream_t; /* hipStream_t */
+typedef void* mlxrocm_event_t;  /* hipEvent_t  */
+
+int mlxrocm_abi_version(void);
+const char* mlxrocm_last_error(void);
+
+/* ------------------------------------------------------------------------ */
+/* Quantize / dequantize                                                     */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Replaces fast::Quantize::eval_gpu with dequantize_ == false
+ * (mlx/fast_primitives.h:355-356; CPU body mlx/backend/cpu/quantized.cpp:1229-1280,
+ * algorithm quantize<T,U> :1148-1211).  w holds n_elems = rows*K elements,
+ * row-contiguous, K % group_size == 0.  Outputs: wq n_elems*bits/32 words,
+ * scales and biases n_elems/group_size elements of `dtype`.  Results are
+ * bit-identical to the CPU backend's.
+ */
+int mlxrocm_affine_quantize(
+    const void* w,
+    uint32_t* wq,
+    void* scales,
+    void* biases,
+    size_t n_elems,
+    int group_size,
+    int bits,
+    int dtype,
+    mlxrocm_stream_t stream);
+
+/*
+ * Replaces fast::Quantize::eval_gpu with dequantize_ == true
+ * (created by affine_dequantize for Device::gpu, mlx/ops.cpp:5327-5338).
+ * out[e] = T(T(code_e) * scale) + bias, two roundings as in the op graph the
+ * CPU runs (mlx/ops.cpp:5320-5324).  out holds n_elems elements.
+ */
+int mlxrocm_affine_dequantize(
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    void* out,
+    size_t n_elems,
+    int group_size,
+    int bits,
+    int dtype,
+    mlxrocm_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Quantized matmul                                                          */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Replaces QuantizedMatmul::eval_gpu (mlx/primitives.h:1631; CPU body
+ * mlx/backend/cpu/quantized.cpp:924-964, batch loop :383-419).
+ *
+ *   transpose != 0: out[l] = x[l] @ dequant(w[l]).T   w [N, K*bits/32]
+ *   transpose == 0: out[l] = x[l] @ dequant(w[l])     w [K, N*bits/32]
+ *
+ * x is [L, M, K] with batch stride x_batch_stride (elements); out is a dense
+ * [L, M, N].  w_batch_stride (uint32 words) and sb_batch_stride (elements) are
+ * 0 when one weight matrix is shared by every batch (w.ndim() == 2 in MLX).
+ * The kernel is picked from M, N, K, bits, group_size and dtype.
+ */
+int mlxrocm_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t sb_batch_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    mlxrocm_stream_t stream);
+
+/*
+ * Replaces GatherQMM::eval_gpu (mlx/primitives.h:1698; CPU body
+ * mlx/backend/cpu/quantized.cpp:966-1047, loop :700-747):
+ *
+ *   out[i] = qmm(x[lhs_indices[i]], w[rhs_indices[i]])   for i < n_indices
+ *
+ * Indices are flat batch indices (uint32, dense vectors of length n_indices).
+ * x has x_batches matrices [M, K] x_batch_stride elements apart; the weights are
+ * n_experts matrices w_expert_stride words (sb_expert_stride elements) apart, so
+ * a sliced expert stack needs no copy.  out is a dense [n_indices, M, N].
+ * rhs_sorted != 0 promises rhs_indices is non-decreasing (right_sorted_).
+ * workspace must hold mlxrocm_gather_qmm_workspace_size(...) bytes (may be NULL
+ * when that is 0).  Index values are range-checked on the device; an
+ * out-of-range pair produces zeros instead of a wild access.
+ */
+int mlxrocm_gather_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    const uint32_t* lhs_indices,
+    const uint32_t* rhs_indices,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int64_t x_batch_stride,
+    int64_t w_expert_stride,
+    int64_t sb_expert_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    int rhs_sorted,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream);
+
+size_t mlxrocm_gather_qmm_workspace_size(
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int n_experts,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    int rhs_sorted);
+
+/* Name of the kernel family the dispatcher would pick (for logs and tests):
+ * "qmv", "qmm_t", "qmm_generic", ...  Returns NULL for invalid arguments. */
+const char* mlxrocm_qmm_kernel_name(
+    int M,
+    int N,
+    int K,
+    int L,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose);
+
+/* ------------------------------------------------------------------------ */
+/* Device memory with explicit residency, streams, events                    */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * The allocator behind allocator::malloc / free and the memory counters of
+ * mlx/allocator.h:52-75 and mlx/memory.h for a ROCm build (model:
+ * mlx/backend/cuda/allocator.cpp:142-399).  Buffers are device-resident
+ * (hipMalloc) and recycled through a size-bucketed cache; nothing is
+ * host-visible unless copied explicitly with the memcpy calls below.
+ */
+int mlxrocm_malloc(void** ptr, size_t size);
+int mlxrocm_free(void* ptr);
+size_t mlxrocm_buffer_size(const void* ptr); /* allocated size, 0 if unknown */
+size_t mlxrocm_get_active_memory(void);
+size_t mlxrocm_get_peak_memory(void);
+void mlxrocm_reset_peak_memory(void);
+size_t mlxrocm_get_cache_memory(void);
+size_t mlxrocm_set_cache_limit(size_t limit); /* returns the previous limit */
+size_t mlxrocm_set_memory_limit(size_t limit);
+size_t mlxrocm_get_memory_limit(void);
+void mlxrocm_clear_cache(void);
+
+/* Pinned host staging memory (what Buffer::raw_ptr() hands to CPU readers). */
+int mlxrocm_host_malloc(void** ptr, size_t size);
+int mlxrocm_host_free(void* ptr);
+
+int mlxrocm_memcpy_h2d(void* dst, const void* src, size_t n, mlxrocm_stream_t s);
+int mlxrocm_memcpy_d2h(void* dst, const void* src, size_t n, mlxrocm_stream_t s);
+int mlxrocm_memcpy_d2d(void* dst, const void* src, size_t n, mlxrocm_stream_t s);
+
+/* Stream plumbing behind mlx::core::Stream (gpu::new_stream / synchronize,
+ * mlx/backend/gpu/eval.h:11-18).  Streams are created at default priority. */
+int mlxrocm_stream_create(mlxrocm_stream_t* stream);
+int mlxrocm_stream_destroy(mlxrocm_stream_t stream);
+int mlxrocm_stream_synchronize(mlxrocm_stream_t stream);
+
+/* Event plumbing behind mlx::core::Event (mlx/event.h; model
+ * mlx/backend/cuda/event.cu:330-420). */
+int mlxrocm_event_create(mlxrocm_event_t* event);
+int mlxrocm_event_destroy(mlxrocm_event_t event);
+int mlxrocm_event_record(mlxrocm_event_t event, mlxrocm_stream_t stream);
+int mlxrocm_event_wait(mlxrocm_event_t event, mlxrocm_stream_t stream);
+int mlxrocm_event_synchronize(mlxrocm_event_t event);
+int mlxrocm_event_query(mlxrocm_event_t event); /* 1 done, 0 pending, <0 error */
+int mlxrocm_event_elapsed_ms(float* ms, mlxrocm_event_t start, mlxrocm_event_t stop);
+
+int mlxrocm_device_count(void);
+/* name: >= 256 bytes.  Any out pointer may be NULL. */
+int mlxrocm_device_info(
+    int device,
+    char* name,
+    int* compute_units,
+    size_t* total_memory,
+    int* clock_khz);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLX_ROCM_QMM_H */

@@ -1,0 +1,7 @@
+"""mlx_amd -- MLX's affine group-wise quantized matmul path for AMD MI355X
+(gfx950): ``quantize`` / ``dequantize`` / ``quantized_matmul`` / ``gather_qmm``
+with the reference's operator names and semantics, backed by hand-written HIP
+kernels through the C ABI declared in ``include/mlx_rocm_qmm.h``."""
+from .ops import dequantize, gather_qmm, quantize, quantized_matmul
+
+__all__ = ["quantize", "dequantize", "quantized_matmul", "gather_qmm"]

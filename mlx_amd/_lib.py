@@ -1,0 +1,112 @@
+"""ctypes binding of ``libmlx_rocm_qmm.so`` (the C ABI in
+``include/mlx_rocm_qmm.h``).  There is no CPU fallback: if the library is not
+built, importing an operator raises."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libmlx_rocm_qmm.so")
+
+OK = 0
+INVALID_ARGUMENT = -1
+UNSUPPORTED = -2
+HIP_ERROR = -3
+OUT_OF_MEMORY = -4
+
+FLOAT32, FLOAT16, BFLOAT16 = 0, 1, 2
+
+_i = ctypes.c_int
+_i64 = ctypes.c_int64
+_sz = ctypes.c_size_t
+_p = ctypes.c_void_p
+
+# name -> (restype, argtypes); the list the symbol-export test walks.
+SIGNATURES = {
+    "mlxrocm_abi_version": (_i, []),
+    "mlxrocm_last_error": (ctypes.c_char_p, []),
+    "mlxrocm_affine_quantize": (_i, [_p, _p, _p, _p, _sz, _i, _i, _i, _p]),
+    "mlxrocm_affine_dequantize": (_i, [_p, _p, _p, _p, _sz, _i, _i, _i, _p]),
+    "mlxrocm_qmm": (
+        _i,
+        [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p],
+    ),
+    "mlxrocm_gather_qmm": (
+        _i,
+        [_p] * 7 + [_i] * 6 + [_i64] * 3 + [_i] * 5 + [_p, _sz, _p],
+    ),
+    "mlxrocm_gather_qmm_workspace_size": (_sz, [_i] * 10),
+    "mlxrocm_qmm_kernel_name": (ctypes.c_char_p, [_i] * 8),
+    "mlxrocm_malloc": (_i, [ctypes.POINTER(_p), _sz]),
+    "mlxrocm_free": (_i, [_p]),
+    "mlxrocm_buffer_size": (_sz, [_p]),
+    "mlxrocm_get_active_memory": (_sz, []),
+    "mlxrocm_get_peak_memory": (_sz, []),
+    "mlxrocm_reset_peak_memory": (None, []),
+    "mlxrocm_get_cache_memory": (_sz, []),
+    "mlxrocm_set_cache_limit": (_sz, [_sz]),
+    "mlxrocm_set_memory_limit": (_sz, [_sz]),
+    "mlxrocm_get_memory_limit": (_sz, []),
+    "mlxrocm_clear_cache": (None, []),
+    "mlxrocm_host_malloc": (_i, [ctypes.POINTER(_p), _sz]),
+    "mlxrocm_host_free": (_i, [_p]),
+    "mlxrocm_memcpy_h2d": (_i, [_p, _p, _sz, _p]),
+    "mlxrocm_memcpy_d2h": (_i, [_p, _p, _sz, _p]),
+    "mlxrocm_memcpy_d2d": (_i, [_p, _p, _sz, _p]),
+    "mlxrocm_stream_create": (_i, [ctypes.POINTER(_p)]),
+    "mlxrocm_stream_destroy": (_i, [_p]),
+    "mlxrocm_stream_synchronize": (_i, [_p]),
+    "mlxrocm_event_create": (_i, [ctypes.POINTER(_p)]),
+    "mlxrocm_event_destroy": (_i, [_p]),
+    "mlxrocm_event_record": (_i, [_p, _p]),
+    "mlxrocm_event_wait": (_i, [_p, _p]),
+    "mlxrocm_event_synchronize": (_i, [_p]),
+    "mlxrocm_event_query": (_i, [_p]),
+    "mlxrocm_event_elapsed_ms": (_i, [ctypes.POINTER(ctypes.c_float), _p, _p]),
+    "mlxrocm_device_count": (_i, []),
+    "mlxrocm_device_info": (
+        _i,
+        [_i, ctypes.c_char_p, ctypes.POINTER(_i), ctypes.POINTER(_sz), ctypes.POINTER(_i)],
+    ),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.isfile(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: build it with `python -m mlx_amd._build` "
+            "(hipcc, gfx950).  mlx_amd has no CPU fallback."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.mlxrocm_abi_version() != 1:
+        raise ImportError("libmlx_rocm_qmm.so ABI version mismatch")
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().mlxrocm_last_error().decode("utf-8", "replace")
+
+
+def check(status: int) -> None:
+    """Turn a status into the exception MLX's C++ glue would throw:
+    std::invalid_argument -> ValueError, runtime_error -> RuntimeError."""
+    if status == OK:
+        return
+    msg = last_error()
+    if status == INVALID_ARGUMENT:
+        raise ValueError(msg)
+    if status == OUT_OF_MEMORY:
+        raise MemoryError(msg)
+    raise RuntimeError(msg)

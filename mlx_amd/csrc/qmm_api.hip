@@ -1,0 +1,295 @@
+// qmm_api.hip -- C entry points of quantized_matmul / gather_qmm: argument
+// checks, kernel choice, launch.
+#include "qmm_args.h"
+
+namespace mlxrocm {
+
+namespace {
+
+enum class Family { Qmv, QmmNaive };
+
+// M below which the transpose=true path is a row-streaming GEMV: every packed
+// weight row is read once and reused across the few rows of x.
+constexpr int kQmvMaxM = 16;
+
+Family choose_family(int M, int /*N*/, int /*K*/, int /*L*/, bool transpose) {
+  if (transpose && M <= kQmvMaxM) {
+    return Family::Qmv;
+  }
+  return Family::QmmNaive;
+}
+
+const char* family_name(Family f) {
+  switch (f) {
+    case Family::Qmv:
+      return "qmv";
+    case Family::QmmNaive:
+      return "qmm_generic";
+  }
+  return nullptr;
+}
+
+int check_shape(
+    const char* who,
+    int M,
+    int N,
+    int K,
+    int L,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose) {
+  if (!valid_bits(bits)) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[%s] the requested number of bits %d is not supported; "
+        "supported bits are 2, 3, 4, 5, 6 and 8",
+        who,
+        bits);
+  }
+  if (!valid_group(group_size)) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[%s] the requested group size %d is not supported; "
+        "supported group sizes are 32, 64 and 128",
+        who,
+        group_size);
+  }
+  if (!valid_dtype(dtype)) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[%s] unknown dtype %d", who, dtype);
+  }
+  if (M < 0 || N < 0 || K < 0 || L < 0) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[%s] negative dimension", who);
+  }
+  // The quantized axis (K when transposed, N otherwise) is made of whole groups.
+  const int quantized_axis = transpose ? K : N;
+  if (quantized_axis % group_size != 0) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[%s] the quantized dimension %d is not a multiple of group_size=%d "
+        "(transpose=%d)",
+        who,
+        quantized_axis,
+        group_size,
+        transpose);
+  }
+  return MLXROCM_OK;
+}
+
+bool aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+int check_alignment(const char* who, const QmmArgs& a, int dtype) {
+  if (!aligned16(a.x) || !aligned16(a.w) || !aligned16(a.scales) ||
+      !aligned16(a.biases) || !aligned16(a.out)) {
+    return fail(
+        MLXROCM_UNSUPPORTED,
+        "[%s] operand pointers must be 16-byte aligned",
+        who);
+  }
+  const int64_t x_vec = 16 / static_cast<int64_t>(dtype_size(dtype));
+  if (a.x_batch_stride % x_vec != 0 || a.w_batch_stride % 4 != 0) {
+    return fail(
+        MLXROCM_UNSUPPORTED,
+        "[%s] batch strides must keep 16-byte alignment (x stride %lld, w "
+        "stride %lld)",
+        who,
+        static_cast<long long>(a.x_batch_stride),
+        static_cast<long long>(a.w_batch_stride));
+  }
+  return MLXROCM_OK;
+}
+
+int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
+  switch (choose_family(a.M, a.N, a.K, a.L, transpose)) {
+    case Family::Qmv:
+      return launch_qmv_generic(a, gs, bits, dtype, s);
+    case Family::QmmNaive:
+      return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
+  }
+  return fail(MLXROCM_UNSUPPORTED, "no kernel");
+}
+
+} // namespace
+
+} // namespace mlxrocm
+
+using namespace mlxrocm;
+
+extern "C" const char* mlxrocm_qmm_kernel_name(
+    int M,
+    int N,
+    int K,
+    int L,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose) {
+  if (check_shape("qmm", M, N, K, L, group_size, bits, dtype, transpose) !=
+      MLXROCM_OK) {
+    return nullptr;
+  }
+  return family_name(choose_family(M, N, K, L, transpose != 0));
+}
+
+extern "C" int mlxrocm_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t sb_batch_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    mlxrocm_stream_t stream) {
+  int rc = check_shape(
+      "quantized_matmul", M, N, K, L, group_size, bits, dtype, transpose);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (static_cast<int64_t>(M) * N * L == 0) {
+    return MLXROCM_OK; // empty output
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (K == 0) {
+    return launch_zero_fill(
+        out, static_cast<size_t>(M) * N * L * dtype_size(dtype), s);
+  }
+  if (!x || !wq || !scales || !biases || !out) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] null device pointer");
+  }
+  if (x_batch_stride < 0 || w_batch_stride < 0 || sb_batch_stride < 0) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] negative stride");
+  }
+  QmmArgs a{};
+  a.x = x;
+  a.w = wq;
+  a.scales = scales;
+  a.biases = biases;
+  a.out = out;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.L = L;
+  a.x_batch_stride = x_batch_stride;
+  a.w_batch_stride = w_batch_stride;
+  a.sb_batch_stride = sb_batch_stride;
+  a.lhs_indices = nullptr;
+  a.rhs_indices = nullptr;
+  a.x_batches = L;
+  a.n_experts = L;
+  rc = check_alignment("quantized_matmul", a, dtype);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  return run(a, group_size, bits, dtype, transpose != 0, s);
+}
+
+extern "C" size_t mlxrocm_gather_qmm_workspace_size(
+    int /*M*/,
+    int /*N*/,
+    int /*K*/,
+    int /*n_indices*/,
+    int /*n_experts*/,
+    int /*group_size*/,
+    int /*bits*/,
+    int /*dtype*/,
+    int /*transpose*/,
+    int /*rhs_sorted*/) {
+  return 0;
+}
+
+extern "C" int mlxrocm_gather_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    const uint32_t* lhs_indices,
+    const uint32_t* rhs_indices,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int64_t x_batch_stride,
+    int64_t w_expert_stride,
+    int64_t sb_expert_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    int /*rhs_sorted*/,
+    void* /*workspace*/,
+    size_t /*workspace_bytes*/,
+    mlxrocm_stream_t stream) {
+  int rc = check_shape(
+      "gather_qmm", M, N, K, n_indices, group_size, bits, dtype, transpose);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (static_cast<int64_t>(M) * N * n_indices == 0) {
+    return MLXROCM_OK;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (K == 0) {
+    return launch_zero_fill(
+        out, static_cast<size_t>(M) * N * n_indices * dtype_size(dtype), s);
+  }
+  if (!x || !wq || !scales || !biases || !out || !lhs_indices ||
+      !rhs_indices) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qmm] null device pointer");
+  }
+  if (x_batches <= 0 || n_experts <= 0 || x_batch_stride < 0 ||
+      w_expert_stride < 0 || sb_expert_stride < 0) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT, "[gather_qmm] invalid batch description");
+  }
+  QmmArgs a{};
+  a.x = x;
+  a.w = wq;
+  a.scales = scales;
+  a.biases = biases;
+  a.out = out;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.L = n_indices;
+  a.x_batch_stride = x_batch_stride;
+  a.w_batch_stride = w_expert_stride;
+  a.sb_batch_stride = sb_expert_stride;
+  a.lhs_indices = lhs_indices;
+  a.rhs_indices = rhs_indices;
+  a.x_batches = x_batches;
+  a.n_experts = n_experts;
+  rc = check_alignment("gather_qmm", a, dtype);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  // One grid z-slot per index pair; large index lists go in slices.
+  constexpr int kMaxZ = 65535;
+  for (int first = 0; first < n_indices; first += kMaxZ) {
+    QmmArgs part = a;
+    part.L = (n_indices - first < kMaxZ) ? n_indices - first : kMaxZ;
+    part.lhs_indices = lhs_indices + first;
+    part.rhs_indices = rhs_indices + first;
+    part.out = static_cast<char*>(out) +
+        static_cast<size_t>(first) * M * N * dtype_size(dtype);
+    rc = run(part, group_size, bits, dtype, transpose != 0, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+  }
+  return MLXROCM_OK;
+}

@@ -1,0 +1,79 @@
+// qmm_args.h -- problem descriptor shared by the quantized-matmul kernels.
+#pragma once
+
+#include "common.h"
+
+namespace mlxrocm {
+
+// One launch covers L problems.  Without index arrays problem l reads x batch l
+// and weight batch l (stride 0 = one shared weight); with them it reads
+// x[lhs[l]] and w[rhs[l]] (GatherQMM).
+struct QmmArgs {
+  const void* x;
+  const uint32_t* w;
+  const void* scales;
+  const void* biases;
+  void* out;
+  int M;
+  int N;
+  int K;
+  int L;
+  int64_t x_batch_stride;  // elements
+  int64_t w_batch_stride;  // uint32 words
+  int64_t sb_batch_stride; // elements
+  const uint32_t* lhs_indices;
+  const uint32_t* rhs_indices;
+  int x_batches; // bounds for gathered indices
+  int n_experts;
+};
+
+// Resolved operand pointers of problem l.  `valid` is false when a gathered
+// index is out of range; the problem's output is then zero-filled.
+template <typename T>
+struct QmmProblem {
+  const T* x;
+  const uint8_t* w;
+  const T* scales;
+  const T* biases;
+  T* out;
+  bool valid;
+};
+
+template <typename T>
+__device__ __forceinline__ QmmProblem<T> resolve_problem(
+    const QmmArgs& a,
+    int l) {
+  QmmProblem<T> p;
+  int64_t xb = l;
+  int64_t wb = l;
+  p.valid = true;
+  if (a.lhs_indices != nullptr) {
+    const uint32_t xi = a.lhs_indices[l];
+    const uint32_t wi = a.rhs_indices[l];
+    p.valid = xi < static_cast<uint32_t>(a.x_batches) &&
+        wi < static_cast<uint32_t>(a.n_experts);
+    xb = p.valid ? xi : 0;
+    wb = p.valid ? wi : 0;
+  }
+  p.x = static_cast<const T*>(a.x) + xb * a.x_batch_stride;
+  p.w = reinterpret_cast<const uint8_t*>(a.w + wb * a.w_batch_stride);
+  p.scales = static_cast<const T*>(a.scales) + wb * a.sb_batch_stride;
+  p.biases = static_cast<const T*>(a.biases) + wb * a.sb_batch_stride;
+  p.out = static_cast<T*>(a.out) +
+      static_cast<int64_t>(l) * a.M * static_cast<int64_t>(a.N);
+  return p;
+}
+
+// Launchers implemented per kernel family; each returns an mlxrocm_status.
+int launch_qmv_generic(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+int launch_qmm_naive(
+    const QmmArgs& a,
+    int gs,
+    int bits,
+    int dtype,
+    bool transpose,
+    hipStream_t s);
+
+int launch_zero_fill(void* p, size_t bytes, hipStream_t s);
+
+} // namespace mlxrocm

@@ -1,0 +1,423 @@
+"""Host-side mirror of MLX's affine quantization operators for MI355X.
+
+Same names, argument meaning, defaults and error behaviour as
+``mx.quantize`` / ``mx.dequantize`` / ``mx.quantized_matmul`` /
+``mx.gather_qmm`` (reference: ``mlx/ops.cpp:4784-4834, 5035-5099, 5208-5246,
+5465-5517, 5553-5629``; Python binding ``python/src/ops.cpp:4622-4866``).
+Tensors are torch tensors resident on the GPU; torch only supplies device
+memory and the current HIP stream -- every computation is done by the HIP
+kernels behind the C ABI of ``include/mlx_rocm_qmm.h``.  Invalid arguments
+raise ``ValueError`` exactly where the reference throws
+``std::invalid_argument``.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {
+    torch.float32: _lib.FLOAT32,
+    torch.float16: _lib.FLOAT16,
+    torch.bfloat16: _lib.BFLOAT16,
+}
+_FLOATING = tuple(_DTYPE_CODE)
+_MODES = ("affine", "mxfp4", "mxfp8", "nvfp4")
+_INTEGER = (
+    torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64,
+    torch.uint16, torch.uint32, torch.uint64,
+)
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(tag: str, *tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                f"[{tag}] mlx_amd runs on the GPU only; got a tensor on {t.device}"
+            )
+
+
+def _mode(tag: str, mode: str) -> str:
+    # string_to_quantization_mode, mlx/primitives.cpp
+    if mode not in _MODES:
+        raise ValueError(f"[{tag}] Invalid quantization mode '{mode}'.")
+    return mode
+
+
+def _params_from_mode(mode: str, group_size, bits) -> Tuple[int, int]:
+    # quantization_params_from_mode, mlx/ops.cpp:4675-4702
+    defaults = {"affine": (64, 4), "nvfp4": (16, 4), "mxfp4": (32, 4), "mxfp8": (32, 8)}
+    dg, db = defaults[mode]
+    return (dg if group_size is None else int(group_size),
+            db if bits is None else int(bits))
+
+
+def _affine_only(tag: str, mode: str) -> None:
+    if mode != "affine":
+        raise RuntimeError(
+            f"[{tag}] quantization mode '{mode}' has no ROCm implementation; "
+            "only 'affine' is supported."
+        )
+
+
+def _validate_mode_with_type(tag, scales, biases, out_type, mode):
+    # mlx/ops.cpp:4704-4754
+    mode = _mode(tag, mode)
+    if out_type is not None and out_type not in _FLOATING:
+        raise ValueError(
+            f"[{tag}] Only real floating types are supported but output dtype == {out_type}."
+        )
+    _affine_only(tag, mode)
+    if biases is None:
+        raise ValueError(f"[{tag}] Biases must be provided for affine quantization.")
+    dtype = torch.promote_types(scales.dtype, biases.dtype)
+    if dtype not in _FLOATING:
+        raise ValueError(
+            f"[{tag}] Only real floating types are supported but scales.dtype() == "
+            f"{scales.dtype} and biases.dtype() == {biases.dtype}."
+        )
+    return (out_type if out_type is not None else dtype), mode
+
+
+def _validate_quantized_input(tag, w, scales, group_size, bits, biases):
+    # mlx/ops.cpp:110-150
+    if w.dtype != torch.uint32:
+        raise ValueError(
+            f"[{tag}] The weight matrix should be uint32 but received {w.dtype}"
+        )
+    if biases is not None and scales.shape != biases.shape:
+        raise ValueError(
+            f"[{tag}] Scales and biases should have the same shape. Received scales "
+            f"with shape {tuple(scales.shape)} and biases with {tuple(biases.shape)}"
+        )
+    if w.dim() < 2 or scales.dim() < 2 or tuple(w.shape[:-2]) != tuple(
+        scales.shape[: w.dim() - 2]
+    ):
+        raise ValueError(
+            f"[{tag}] Weight and scales should have the same batch shape. Received "
+            f"weight with shape {tuple(w.shape)}, scales with {tuple(scales.shape)}."
+        )
+    if w.shape[-1] * 32 // bits != scales.shape[-1] * group_size:
+        raise ValueError(
+            f"[{tag}] The shapes of the weight and scales are incompatible based on "
+            f"bits and group_size. w.shape() == {tuple(w.shape)} and scales.shape() "
+            f"== {tuple(scales.shape)} with group_size={group_size} and bits={bits}"
+        )
+
+
+def _extract_dims(tag, x, w, scales, biases, transpose, group_size, bits):
+    # extract_quantized_matmul_dims, mlx/ops.cpp:152-181
+    _validate_quantized_input(tag, w, scales, group_size, bits, biases)
+    if x.dim() < 1:
+        raise ValueError(f"[{tag}] x must have at least one dimension")
+    x_inner = x.shape[-1]
+    w_inner = w.shape[-1] * 32 // bits if transpose else w.shape[-2]
+    w_outer = w.shape[-2] if transpose else w.shape[-1] * 32 // bits
+    if w_inner != x_inner:
+        raise ValueError(
+            f"[{tag}] Last dimension of first input with shape (..., {x_inner}) does "
+            f"not match the expanded quantized matrix ({w_inner}, {w_outer}) computed "
+            f"from shape {tuple(w.shape)} with group_size={group_size}, bits={bits} "
+            f"and transpose={str(bool(transpose)).lower()}"
+        )
+    return w_inner, w_outer
+
+
+def _check_affine_params(tag: str, group_size: int, bits: int) -> None:
+    # affine_quantize, mlx/ops.cpp:5038-5050
+    if group_size not in (32, 64, 128):
+        raise ValueError(
+            f"[{tag}] The requested group size {group_size} is not supported. "
+            "The supported group sizes are 32, 64, and 128."
+        )
+    if bits < 2 or bits > 8 or bits == 7:
+        raise ValueError(
+            f"[{tag}] The requested number of bits {bits} is not supported. "
+            "The supported bits are 2, 3, 4, 5, 6 and 8."
+        )
+
+
+def _last_two_dense(t: torch.Tensor) -> bool:
+    """Rows of the trailing matrix are contiguous (what the CPU backend
+    requires of w / scales / biases, mlx/backend/cpu/quantized.cpp:974-990)."""
+    return t.stride(-1) == 1 and t.stride(-2) == t.shape[-1]
+
+
+# --------------------------------------------------------------------------
+def quantize(
+    w: torch.Tensor,
+    group_size: Optional[int] = None,
+    bits: Optional[int] = None,
+    mode: str = "affine",
+):
+    """``mx.quantize``: returns ``(w_q uint32, scales, biases)``
+    (mlx/ops.cpp:5208-5246 -> affine_quantize :5035-5099)."""
+    mode = _mode("quantize", mode)
+    group_size, bits = _params_from_mode(mode, group_size, bits)
+    if w.dtype not in _FLOATING:
+        raise ValueError(
+            f"[quantize] Only real floating types can be quantized but w has type {w.dtype}."
+        )
+    if w.dim() < 2:
+        raise ValueError(
+            "[quantize] The matrix to be quantized must have at least 2 dimension "
+            f"but it has only {w.dim()}."
+        )
+    if w.shape[-1] % group_size != 0:
+        raise ValueError(
+            "[quantize] The last dimension of the matrix needs to be divisible by the "
+            f"quantization group size {group_size}. However the provided  matrix has "
+            f"shape {tuple(w.shape)}"
+        )
+    _affine_only("quantize", mode)
+    _check_affine_params("quantize", group_size, bits)
+    _require_gpu("quantize", w)
+    lib = _lib.load()
+    w = w.contiguous()  # ensure_row_contiguous, cpu/quantized.cpp:1233
+    lead = tuple(w.shape[:-1])
+    K = w.shape[-1]
+    wq = torch.empty(lead + (K * bits // 32,), dtype=torch.uint32, device=w.device)
+    scales = torch.empty(lead + (K // group_size,), dtype=w.dtype, device=w.device)
+    biases = torch.empty_like(scales)
+    _lib.check(
+        lib.mlxrocm_affine_quantize(
+            w.data_ptr(), wq.data_ptr(), scales.data_ptr(), biases.data_ptr(),
+            w.numel(), group_size, bits, _DTYPE_CODE[w.dtype], _stream_ptr(w),
+        )
+    )
+    return wq, scales, biases
+
+
+def dequantize(
+    w: torch.Tensor,
+    scales: torch.Tensor,
+    biases: Optional[torch.Tensor] = None,
+    group_size: Optional[int] = None,
+    bits: Optional[int] = None,
+    mode: str = "affine",
+    dtype: Optional[torch.dtype] = None,
+):
+    """``mx.dequantize`` (mlx/ops.cpp:5465-5517 -> affine_dequantize :5248-5340)."""
+    out_type, mode = _validate_mode_with_type("dequantize", scales, biases, dtype, mode)
+    group_size, bits = _params_from_mode(mode, group_size, bits)
+    if bits <= 0:
+        raise ValueError(f"[dequantize] Invalid value for bits: {bits}")
+    if group_size <= 0:
+        raise ValueError(f"[dequantize] Invalid value for group_size: {group_size}")
+    if w.dtype != torch.uint32:
+        raise ValueError("[dequantize] The matrix should be given as a uint32")
+    if w.dim() < 2:
+        raise ValueError(
+            "[dequantize] The matrix to be dequantized must have at least 2 dimension "
+            f"but it has only {w.dim()}."
+        )
+    if (
+        w.dim() != scales.dim()
+        or w.dim() != biases.dim()
+        or tuple(w.shape[:-1]) != tuple(scales.shape[:-1])
+        or tuple(w.shape[:-1]) != tuple(biases.shape[:-1])
+    ):
+        raise ValueError(
+            "[dequantize] Shape of scales and biases does not match the matrix"
+        )
+    out_size = w.shape[-1] * 32 // bits
+    if out_size != scales.shape[-1] * group_size or scales.shape != biases.shape:
+        raise ValueError(
+            "[dequantize] Shape of scales and biases does not match the matrix given "
+            f"the quantization parameters. Provided matrix of shape {tuple(w.shape)} "
+            f"and scales/biases of shape {tuple(scales.shape)} with "
+            f"group_size={group_size} and bits={bits}."
+        )
+    _check_affine_params("dequantize", group_size, bits)
+    _require_gpu("dequantize", w, scales, biases)
+    lib = _lib.load()
+    # The affine step runs in scales' dtype (mlx/ops.cpp:5322-5323); biases are
+    # promoted to it the way the Add primitive would.
+    sdt = torch.promote_types(scales.dtype, biases.dtype)
+    w = w.contiguous()
+    scales = scales.to(sdt).contiguous()
+    biases = biases.to(sdt).contiguous()
+    out = torch.empty(tuple(w.shape[:-1]) + (out_size,), dtype=sdt, device=w.device)
+    _lib.check(
+        lib.mlxrocm_affine_dequantize(
+            w.data_ptr(), scales.data_ptr(), biases.data_ptr(), out.data_ptr(),
+            out.numel(), group_size, bits, _DTYPE_CODE[sdt], _stream_ptr(w),
+        )
+    )
+    return out if out_type == sdt else out.to(out_type)  # astype, :5502-5505
+
+
+def _dense_batches(t: torch.Tensor, batch_shape: Tuple[int, ...]):
+    """Expand the leading dims of ``t`` to ``batch_shape``; returns the tensor
+    and its batch stride in elements (0 when one matrix serves every batch)."""
+    if t.dim() == 2:
+        return (t if _last_two_dense(t) else t.contiguous()), 0
+    t = t.expand(*batch_shape, *t.shape[-2:])
+    if not t.is_contiguous():
+        t = t.contiguous()
+    return t, t.shape[-1] * t.shape[-2]
+
+
+def quantized_matmul(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    scales: torch.Tensor,
+    biases: Optional[torch.Tensor] = None,
+    transpose: bool = True,
+    group_size: Optional[int] = None,
+    bits: Optional[int] = None,
+    mode: str = "affine",
+):
+    """``mx.quantized_matmul`` (mlx/ops.cpp:4784-4834)."""
+    dtype, mode = _validate_mode_with_type("quantized_matmul", scales, biases, None, mode)
+    group_size, bits = _params_from_mode(mode, group_size, bits)
+    _, w_outer = _extract_dims(
+        "quantized_matmul", x, w, scales, biases, transpose, group_size, bits
+    )
+    dtype = torch.promote_types(x.dtype, dtype)
+    if dtype not in _FLOATING:
+        raise ValueError(
+            "[quantized_matmul] Only real floating types are supported but "
+            f"x.dtype() == {x.dtype}."
+        )
+    _check_affine_params("quantized_matmul", group_size, bits)
+    _require_gpu("quantized_matmul", x, w, scales, biases)
+    lib = _lib.load()
+
+    x = x.to(dtype)
+    scales = scales.to(dtype)
+    biases = biases.to(dtype)
+    K = x.shape[-1]
+    M = x.shape[-2] if x.dim() > 1 else 1
+    x_batch = tuple(x.shape[:-2]) if x.dim() > 2 else ()
+    if x.dim() > 2 and w.dim() > 2:
+        # broadcast_arrays(inputs, {-2, -1}), :4823-4825
+        batch_shape = tuple(torch.broadcast_shapes(x_batch, tuple(w.shape[:-2])))
+    else:
+        batch_shape = x_batch
+        if w.dim() > 2:
+            raise ValueError(
+                "[quantized_matmul] a batched weight needs a batched first input"
+            )
+    out_shape = (tuple(x.shape[:-1]) if x.dim() <= 2 else batch_shape + (M,)) + (w_outer,)
+    L = 1
+    for d in batch_shape:
+        L *= d
+    xb = x.reshape(1, M, K) if x.dim() <= 2 else x.expand(*batch_shape, M, K)
+    xb = xb.contiguous()
+    wb, w_stride = _dense_batches(w, batch_shape)
+    sb, sb_stride = _dense_batches(scales, batch_shape)
+    bb, _ = _dense_batches(biases, batch_shape)
+    out = torch.empty(out_shape, dtype=dtype, device=x.device)
+    _lib.check(
+        lib.mlxrocm_qmm(
+            xb.data_ptr(), wb.data_ptr(), sb.data_ptr(), bb.data_ptr(), out.data_ptr(),
+            M, w_outer, K, L, M * K, w_stride, sb_stride, group_size, bits,
+            _DTYPE_CODE[dtype], int(bool(transpose)), _stream_ptr(x),
+        )
+    )
+    return out
+
+
+def _indices_or_default(tag, indices, t):
+    # mlx/ops.cpp:79-108
+    if t.dim() < 2:
+        raise ValueError(
+            f"{tag} Input must have at least two dimensions but got input with shape "
+            f"{tuple(t.shape)}."
+        )
+    if indices is not None:
+        if indices.dtype not in _INTEGER:
+            raise ValueError(
+                f"{tag} Got indices with invalid dtype. Indices must be integral."
+            )
+        return indices.to(torch.int64)
+    shape = tuple(t.shape[:-2])
+    total = 1
+    for d in shape:
+        total *= d
+    return torch.arange(total, dtype=torch.int64, device=t.device).reshape(shape)
+
+
+def gather_qmm(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    scales: torch.Tensor,
+    biases: Optional[torch.Tensor] = None,
+    lhs_indices: Optional[torch.Tensor] = None,
+    rhs_indices: Optional[torch.Tensor] = None,
+    transpose: bool = True,
+    group_size: Optional[int] = None,
+    bits: Optional[int] = None,
+    mode: str = "affine",
+    sorted_indices: bool = False,
+):
+    """``mx.gather_qmm`` (mlx/ops.cpp:5553-5629)."""
+    if lhs_indices is None and rhs_indices is None:
+        return quantized_matmul(x, w, scales, biases, transpose, group_size, bits, mode)
+    out_type, mode = _validate_mode_with_type("gather_qmm", scales, biases, None, mode)
+    group_size, bits = _params_from_mode(mode, group_size, bits)
+    _, w_outer = _extract_dims(
+        "gather_qmm", x, w, scales, biases, transpose, group_size, bits
+    )
+    out_type = torch.promote_types(x.dtype, out_type)
+    if out_type not in _FLOATING:
+        raise ValueError(
+            f"[gather_qmm] Only real floating types are supported but x.dtype() == {x.dtype}."
+        )
+    lhs = _indices_or_default("[gather_qmm]", lhs_indices, x)
+    rhs = _indices_or_default("[gather_qmm]", rhs_indices, w)
+    _check_affine_params("gather_qmm", group_size, bits)
+    _require_gpu("gather_qmm", x, w, scales, biases, lhs, rhs)
+    lib = _lib.load()
+    lhs, rhs = torch.broadcast_tensors(lhs, rhs)
+    right_sorted = bool(sorted_indices) and lhs_indices is None
+
+    x = x.to(out_type)
+    scales = scales.to(out_type)
+    biases = biases.to(out_type)
+    M, K = x.shape[-2], x.shape[-1]
+    xb = x.contiguous().reshape(-1, M, K)
+    # Only the trailing matrices must be dense; a sliced expert stack keeps its
+    # stride (python/tests/test_quantized.py:1567-1593).
+    def experts(t):
+        if t.dim() == 3 and _last_two_dense(t):
+            return t, t.stride(0)
+        t = t.contiguous().reshape(-1, *t.shape[-2:])
+        return t, t.shape[-1] * t.shape[-2]
+    wb, w_stride = experts(w)
+    sb, sb_stride = experts(scales)
+    bb, bb_stride = experts(biases)
+    if bb_stride != sb_stride:
+        bb = bb.contiguous()
+        sb = sb.contiguous()
+        sb_stride = sb.shape[-1] * sb.shape[-2]
+    n_idx = lhs.numel()
+    lhs_u = lhs.reshape(-1).to(torch.uint32).contiguous() if n_idx else lhs.reshape(-1)
+    rhs_u = rhs.reshape(-1).to(torch.uint32).contiguous() if n_idx else rhs.reshape(-1)
+    out = torch.empty(tuple(lhs.shape) + (M, w_outer), dtype=out_type, device=x.device)
+    code = _DTYPE_CODE[out_type]
+    ws_bytes = lib.mlxrocm_gather_qmm_workspace_size(
+        M, w_outer, K, n_idx, wb.shape[0], group_size, bits, code,
+        int(bool(transpose)), int(right_sorted),
+    )
+    ws = (
+        torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    )
+    _lib.check(
+        lib.mlxrocm_gather_qmm(
+            xb.data_ptr(), wb.data_ptr(), sb.data_ptr(), bb.data_ptr(),
+            lhs_u.data_ptr() if n_idx else None, rhs_u.data_ptr() if n_idx else None,
+            out.data_ptr(), M, w_outer, K, n_idx, xb.shape[0], wb.shape[0],
+            M * K, w_stride, sb_stride, group_size, bits, code,
+            int(bool(transpose)), int(right_sorted),
+            ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x),
+        )
+    )
+    return out

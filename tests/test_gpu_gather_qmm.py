@@ -1,0 +1,125 @@
+"""GPU parity of gather_qmm (expert-routed quantized matmul)."""
+import pytest
+import torch
+
+import mlx_amd
+from tests.util import (
+    activations, exact_affine_weights, exact_tolerance, matmul_tolerance,
+    normal_weights,
+)
+
+pytestmark = pytest.mark.gpu
+
+
+def _to(gpu, *ts):
+    return [None if t is None else t.to(gpu) for t in ts]
+
+
+def _gather_case(oracle, gpu, M, N, K, batch_A, batch_B, lhs, rhs, transpose,
+                 gs=64, bits=4, dtype=torch.float32):
+    x = activations(batch_A + (M, K), dtype)
+    w = normal_weights(batch_B + ((N, K) if transpose else (K, N)), dtype, std=1.0)
+    wq, s, b = oracle.quantize(w, gs, bits)
+    lhs_t = None if lhs is None else torch.tensor(lhs, dtype=torch.int64)
+    rhs_t = None if rhs is None else torch.tensor(rhs, dtype=torch.int64)
+    gx, gwq, gs_, gb, glhs, grhs = _to(gpu, x, wq, s, b, lhs_t, rhs_t)
+    got = mlx_amd.gather_qmm(gx, gwq, gs_, gb, glhs, grhs, transpose, gs, bits).cpu()
+    # expected: per-pair oracle qmm on broadcast indices (cpu/quantized.cpp:727-746)
+    nA = 1
+    for d in batch_A:
+        nA *= d
+    nB = 1
+    for d in batch_B:
+        nB *= d
+    li = torch.arange(nA).reshape(batch_A) if lhs_t is None else lhs_t
+    ri = torch.arange(nB).reshape(batch_B) if rhs_t is None else rhs_t
+    li, ri = torch.broadcast_tensors(li, ri)
+    ref = oracle.gather_qmm(
+        x.reshape(-1, M, K), wq.reshape(-1, *wq.shape[-2:]),
+        s.reshape(-1, *s.shape[-2:]), b.reshape(-1, *b.shape[-2:]),
+        li, ri, transpose, gs, bits,
+    ).reshape(tuple(li.shape) + (M, N))
+    assert got.shape == ref.shape
+    w_hat = exact_affine_weights(wq, s, b, gs, bits)
+    tol = matmul_tolerance(dtype, K, x, w_hat)
+    assert float((got.double() - ref.double()).abs().max()) <= tol
+
+
+CASES = (
+    dict(batch_A=(1,), lhs=(0,), batch_B=(3,), rhs=(2, 1)),
+    dict(batch_A=(1,), lhs=None, batch_B=(3,), rhs=(2, 1)),
+    dict(batch_A=(2,), lhs=None, batch_B=(3,), rhs=(2, 1)),
+    dict(batch_A=(3,), lhs=(0, 2), batch_B=(1,), rhs=(0,)),
+    dict(batch_A=(5,), lhs=(0, 2), batch_B=(3,), rhs=(2, 1)),
+    dict(batch_A=(4, 2), lhs=((7, 6), (5, 4), (1, 2)), batch_B=(4, 1),
+         rhs=((2,), (0,), (1,))),
+)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_gather_qmm_index_broadcasting(oracle, gpu, case):
+    # python/tests/test_quantized.py:1127-1266
+    for M, N, K, transpose in (
+        (1, 32, 128, True), (32, 32, 256, True), (1, 32, 512, True),
+        (32, 256, 32, False), (1, 512, 32, False),
+    ):
+        _gather_case(oracle, gpu, M, N, K, transpose=transpose, **case)
+
+
+@pytest.mark.parametrize("dtype", (torch.float32, torch.float16, torch.bfloat16))
+def test_gather_qmm_sorted_moe(oracle, gpu, dtype):
+    """L tokens x top-2 of 4 experts, sorted vs unsorted
+    (python/tests/test_quantized.py:1451-1565)."""
+    E, N, K, T = 4, 96, 128, 40
+    gs, bits = 64, 4
+    w = normal_weights((E, N, K), dtype, std=0.5)
+    wq, s, b = oracle.quantize(w, gs, bits)
+    x = activations((T, 1, 1, K), dtype)
+    g = torch.Generator().manual_seed(0)
+    idx = torch.randint(0, E, (T, 2), generator=g)
+    gx, gwq, gsc, gb, gidx = _to(gpu, x, wq, s, b, idx)
+    unsorted = mlx_amd.gather_qmm(gx, gwq, gsc, gb, rhs_indices=gidx,
+                                  transpose=True, group_size=gs, bits=bits)
+    assert unsorted.shape == (T, 2, 1, N)
+    # sorted: gather tokens by expert, run with sorted_indices, un-permute
+    flat = gidx.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    inv = torch.argsort(order)
+    xs = gx.reshape(T, 1, K)[order // 2]
+    ys = mlx_amd.gather_qmm(xs, gwq, gsc, gb, rhs_indices=flat[order], transpose=True,
+                            group_size=gs, bits=bits, sorted_indices=True)
+    assert ys.shape == (2 * T, 1, N)
+    resorted = ys[inv].reshape(T, 2, 1, N)
+    ref = oracle.gather_qmm(
+        x.reshape(T, 1, K), wq, s, b,
+        torch.arange(T).repeat_interleave(2), idx.reshape(-1), True, gs, bits,
+    ).reshape(T, 2, 1, N)
+    w_hat = exact_affine_weights(wq, s, b, gs, bits)
+    tol = matmul_tolerance(dtype, K, x, w_hat)
+    assert float((unsorted.cpu().double() - ref.double()).abs().max()) <= tol
+    assert float((resorted.cpu().double() - ref.double()).abs().max()) <= tol
+
+
+def test_gather_qmm_sliced_expert_stack(oracle, gpu):
+    """Non-contiguous expert stacks need no copy
+    (python/tests/test_quantized.py:1567-1593)."""
+    E, N, K = 6, 64, 128
+    w = normal_weights((E, N, K), torch.float32, std=0.5)
+    wq, s, b = oracle.quantize(w, 64, 4)
+    x = activations((8, 1, K), torch.float32)
+    idx = torch.tensor([0, 1, 2, 0, 1, 2, 2, 1])
+    gx, gwq, gs_, gb, gidx = _to(gpu, x, wq, s, b, idx)
+    got = mlx_amd.gather_qmm(gx, gwq[::2], gs_[::2], gb[::2], rhs_indices=gidx)
+    ref = oracle.gather_qmm(x, wq[::2].contiguous(), s[::2].contiguous(),
+                            b[::2].contiguous(), torch.arange(8), idx, True, 64, 4)
+    assert float((got.cpu() - ref).abs().max()) < 1e-4
+
+
+def test_gather_qmm_out_of_range_index_is_contained(gpu):
+    w = normal_weights((2, 32, 64), torch.float32).to(gpu)
+    wq, s, b = mlx_amd.quantize(w)
+    x = activations((1, 1, 64), torch.float32).to(gpu)
+    idx = torch.tensor([1, 7], device=gpu)  # 7 is not an expert
+    out = mlx_amd.gather_qmm(x, wq, s, b, rhs_indices=idx)
+    torch.cuda.synchronize()
+    assert bool((out[1] == 0).all()) and bool(out[0].abs().sum() > 0)

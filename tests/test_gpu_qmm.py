@@ -1,0 +1,137 @@
+"""GPU parity of quantized_matmul against the CPU oracle and the fp64 product."""
+import pytest
+import torch
+
+import mlx_amd
+from tests.util import (
+    ALL_BITS, ALL_GROUPS, DTYPES, activations, exact_affine_weights,
+    exact_tolerance, matmul_tolerance, normal_weights,
+)
+
+pytestmark = pytest.mark.gpu
+
+
+def _check_qmm(oracle, gpu, x, w, gs, bits, transpose=True, rows=None, quantized=None):
+    """x [M, K]; w dense weights (quantized on the CPU by the oracle) or a
+    ready (wq, s, b) triple.  `rows`: subset of x rows given to the oracle."""
+    wq, s, b = quantized if quantized is not None else oracle.quantize(w, gs, bits)
+    got = mlx_amd.quantized_matmul(
+        x.to(gpu), wq.to(gpu), s.to(gpu), b.to(gpu), transpose, gs, bits
+    )
+    torch.cuda.synchronize()
+    got = got.cpu()
+    sel = slice(None) if rows is None else rows
+    xs = x[sel]
+    ref = oracle.qmm(xs, wq, s, b, transpose, gs, bits)
+    w_hat = exact_affine_weights(wq, s, b, gs, bits)
+    K = x.shape[-1]
+    exact = xs.double() @ (w_hat.T if transpose else w_hat)
+    assert got.shape[-1] == exact.shape[-1] and got.dtype == x.dtype
+    g = got[sel].double()
+    err_ref = float((g - ref.double()).abs().max())
+    err_exact = float((g - exact).abs().max())
+    tol_ref = matmul_tolerance(x.dtype, K, x, w_hat)
+    tol_exact = exact_tolerance(x.dtype, K, x, w_hat, exact)
+    assert err_ref <= tol_ref, f"vs oracle: {err_ref} > {tol_ref}"
+    assert err_exact <= tol_exact, f"vs fp64: {err_exact} > {tol_exact}"
+    return got
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits", ALL_BITS)
+@pytest.mark.parametrize("gs", ALL_GROUPS)
+def test_qmv_all_widths(oracle, gpu, dtype, bits, gs):
+    # python/tests/test_quantized.py:565-590 (N = 67 is not a tile multiple)
+    for M, N, K in ((1, 67, 512), (3, 128, 256)):
+        w = normal_weights((N, K), dtype, seed=bits + gs)
+        x = activations((M, K), dtype)
+        _check_qmm(oracle, gpu, x, w, gs, bits)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits", ALL_BITS)
+@pytest.mark.parametrize("gs", ALL_GROUPS)
+@pytest.mark.parametrize("transpose", (True, False))
+def test_qmm_all_widths(oracle, gpu, dtype, bits, gs, transpose):
+    # python/tests/test_quantized.py:288-323: M in {8, 32, 33, 64}
+    for M in (33, 64):
+        N, K = 256, 384
+        w = normal_weights((N, K) if transpose else (K, N), dtype, seed=bits * gs)
+        x = activations((M, K), dtype)
+        _check_qmm(oracle, gpu, x, w, gs, bits, transpose)
+
+
+def test_qmv_config1_fp32(oracle, gpu):
+    w = normal_weights((4096, 4096), torch.float32, seed=0)
+    x = activations((1, 4096), torch.float32, seed=0)
+    _check_qmm(oracle, gpu, x, w, 64, 4)
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 64), (8, 128)])
+@pytest.mark.parametrize("B", (1, 4, 8))
+def test_qmv_decode_shapes_bf16(oracle, gpu, bits, gs, B):
+    for N, K in ((14336, 4096), (4096, 14336)):
+        w = normal_weights((N, K), torch.bfloat16, seed=0)
+        x = activations((B, K), torch.bfloat16)
+        _check_qmm(oracle, gpu, x, w, gs, bits)
+
+
+@pytest.mark.parametrize("bits", (4, 8))
+@pytest.mark.parametrize("gs", (64, 128))
+def test_qmm_t_prefill_shapes_bf16(oracle, gpu, bits, gs):
+    """Full prefill shapes on the GPU; the oracle sees 4 sampled rows of x
+    (each output row depends only on its own x row)."""
+    for N, K in ((4096, 4096), (14336, 4096), (4096, 14336)):
+        w = normal_weights((N, K), torch.bfloat16, seed=0)
+        q = oracle.quantize(w, gs, bits)
+        for M in (512, 2048):
+            x = activations((M, K), torch.bfloat16)
+            rows = torch.tensor([0, M // 3, M // 2 + 1, M - 1])
+            _check_qmm(oracle, gpu, x, None, gs, bits, rows=rows, quantized=q)
+
+
+@pytest.mark.parametrize("bits", (2, 3, 5, 6))
+@pytest.mark.parametrize("dtype", (torch.float32, torch.bfloat16))
+def test_odd_width_stress_matmul(oracle, gpu, dtype, bits):
+    for N, K in ((11008, 4096), (4096, 11008)):
+        w = normal_weights((N, K), dtype, seed=bits)
+        q = oracle.quantize(w, 32, bits)
+        _check_qmm(oracle, gpu, activations((1, K), dtype), None, 32, bits, quantized=q)
+        x = activations((1024, K), dtype)
+        rows = torch.tensor([0, 511, 1023])
+        _check_qmm(oracle, gpu, x, None, 32, bits, rows=rows, quantized=q)
+
+
+def test_qmm_batched_shapes(oracle, gpu):
+    # python/tests/test_quantized.py:540-563
+    gs, bits = 64, 4
+    w = normal_weights((32, 256), torch.float32)
+    wq, s, b = oracle.quantize(w, gs, bits)
+    x = activations((3, 5, 256), torch.float32)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq.to(gpu), s.to(gpu), b.to(gpu), True, gs, bits)
+    assert got.shape == (3, 5, 32)
+    ref = oracle.qmm_batched(x, wq, s, b, True, gs, bits)
+    assert float((got.cpu() - ref).abs().max()) < 1e-4
+    # batched weights
+    w3 = normal_weights((3, 32, 256), torch.float32, seed=5)
+    wq3, s3, b3 = oracle.quantize(w3, gs, bits)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq3.to(gpu), s3.to(gpu), b3.to(gpu), True, gs, bits)
+    ref = oracle.qmm_batched(x, wq3, s3, b3, True, gs, bits)
+    assert float((got.cpu() - ref).abs().max()) < 1e-4
+    # 1-D x
+    x1 = activations((256,), torch.float32)
+    got = mlx_amd.quantized_matmul(x1.to(gpu), wq.to(gpu), s.to(gpu), b.to(gpu))
+    assert got.shape == (32,)
+    ref = oracle.qmm(x1.reshape(1, -1), wq, s, b, True, gs, bits)[0]
+    assert float((got.cpu() - ref).abs().max()) < 1e-4
+
+
+def test_qmm_type_promotion(gpu):
+    """x, scales, biases are cast to the promoted type (mlx/ops.cpp:4816-4818)."""
+    w = normal_weights((64, 128), torch.bfloat16).to(gpu)
+    wq, s, b = mlx_amd.quantize(w)
+    x = activations((2, 128), torch.float32).to(gpu)
+    out = mlx_amd.quantized_matmul(x, wq, s, b)
+    assert out.dtype == torch.float32
+    out16 = mlx_amd.quantized_matmul(x.to(torch.float16), wq, s, b)
+    assert out16.dtype == torch.float32  # float16 x bfloat16 -> float32
