@@ -96,6 +96,11 @@ def test_gather_qmm_sorted_moe(oracle, gpu, dtype):
     ).reshape(T, 2, 1, N)
     w_hat = exact_affine_weights(wq, s, b, gs, bits)
     tol = matmul_tolerance(dtype, K, x, w_hat)
+    exact = torch.einsum(
+        "tk,tjnk->tjn", x.reshape(T, K).double(), w_hat[idx]
+    ).reshape(T, 2, 1, N)
+    assert float((unsorted.cpu().double() - exact).abs().max()) <= exact_tolerance(
+        dtype, K, x, w_hat, exact)
     assert float((unsorted.cpu().double() - ref.double()).abs().max()) <= tol
     assert float((resorted.cpu().double() - ref.double()).abs().max()) <= tol
 

@@ -31,6 +31,12 @@ def _check_qmm(oracle, gpu, x, w, gs, bits, transpose=True, rows=None, quantized
     err_ref = float((g - ref.double()).abs().max())
     err_exact = float((g - exact).abs().max())
     tol_ref = matmul_tolerance(x.dtype, K, x, w_hat)
+    if x.dtype != torch.float32:
+        # The x86 CPU reference accumulates 16-bit types in the element type
+        # (cpu/quantized.cpp:177-206); at K >= 4096 its own distance from the
+        # exact product already exceeds the bound, so that measured distance is
+        # discounted.  The fp64 check below is the strict one.
+        tol_ref += float((ref.double() - exact).abs().max())
     tol_exact = exact_tolerance(x.dtype, K, x, w_hat, exact)
     assert err_ref <= tol_ref, f"vs oracle: {err_ref} > {tol_ref}"
     assert err_exact <= tol_exact, f"vs fp64: {err_exact} > {tol_exact}"
