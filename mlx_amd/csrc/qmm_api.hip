@@ -104,6 +104,9 @@ int check_alignment(const char* who, const QmmArgs& a, int dtype) {
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
   switch (choose_family(a.M, a.N, a.K, a.L, transpose)) {
     case Family::Qmv:
+      if (qmv_mfma_supported(a, gs, bits, dtype)) {
+        return launch_qmv_mfma(a, gs, bits, dtype, s);
+      }
       return launch_qmv_generic(a, gs, bits, dtype, s);
     case Family::QmmNaive:
       return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
