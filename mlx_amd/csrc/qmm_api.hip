@@ -104,6 +104,9 @@ int check_alignment(const char* who, const QmmArgs& a, int dtype) {
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
   switch (choose_family(a.M, a.N, a.K, a.L, transpose)) {
     case Family::Qmv:
+      if (qmv_stream_supported(a, gs, bits, dtype)) {
+        return launch_qmv_stream(a, gs, bits, dtype, s);
+      }
       if (qmv_mfma_supported(a, gs, bits, dtype)) {
         return launch_qmv_mfma(a, gs, bits, dtype, s);
       }
