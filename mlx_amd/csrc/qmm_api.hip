@@ -6,15 +6,18 @@ namespace mlxrocm {
 
 namespace {
 
-enum class Family { Qmv, QmmNaive };
+enum class Family { Qmv, QmmT, QmmNaive };
 
-// M below which the transpose=true path is a row-streaming GEMV: every packed
+// M up to which the transpose=true path is a row-streaming GEMV: every packed
 // weight row is read once and reused across the few rows of x.
-constexpr int kQmvMaxM = 16;
+constexpr int kQmvMaxM = 8;
 
-Family choose_family(int M, int /*N*/, int /*K*/, int /*L*/, bool transpose) {
+Family choose_family(int M, int /*N*/, int K, int /*L*/, int dtype, bool transpose) {
   if (transpose && M <= kQmvMaxM) {
     return Family::Qmv;
+  }
+  if (transpose && dtype != MLXROCM_FLOAT32 && K % 64 == 0 && K >= 64) {
+    return Family::QmmT;
   }
   return Family::QmmNaive;
 }
@@ -23,6 +26,8 @@ const char* family_name(Family f) {
   switch (f) {
     case Family::Qmv:
       return "qmv";
+    case Family::QmmT:
+      return "qmm_t";
     case Family::QmmNaive:
       return "qmm_generic";
   }
@@ -102,7 +107,12 @@ int check_alignment(const char* who, const QmmArgs& a, int dtype) {
 }
 
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
-  switch (choose_family(a.M, a.N, a.K, a.L, transpose)) {
+  switch (choose_family(a.M, a.N, a.K, a.L, dtype, transpose)) {
+    case Family::QmmT:
+      if (qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
+        return launch_qmm_mfma(a, gs, bits, dtype, s);
+      }
+      return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
     case Family::Qmv:
       if (qmv_stream_supported(a, gs, bits, dtype)) {
         return launch_qmv_stream(a, gs, bits, dtype, s);
@@ -136,7 +146,7 @@ extern "C" const char* mlxrocm_qmm_kernel_name(
       MLXROCM_OK) {
     return nullptr;
   }
-  return family_name(choose_family(M, N, K, L, transpose != 0));
+  return family_name(choose_family(M, N, K, L, dtype, transpose != 0));
 }
 
 extern "C" int mlxrocm_qmm(

@@ -78,6 +78,8 @@ bool qmv_stream_supported(const QmmArgs& a, int gs, int bits, int dtype);
 int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 bool qmv_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype);
 int launch_qmv_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
+int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 int launch_zero_fill(void* p, size_t bytes, hipStream_t s);
 
 } // namespace mlxrocm
