@@ -3,14 +3,16 @@
 //
 //   y[M, N] = x[M, K] * dequant(W)[N, K]^T
 //
-// A workgroup of 256 threads (2 x 2 wavefronts) owns a 256 (M) x 128 (N) tile of
-// y and walks K in steps of 64.  Per step:
-//   * the x tile (256 x 64) and the packed W tile (128 rows x 64 codes) are
-//     fetched into registers while the previous step's MFMAs run;
+// A workgroup of 512 threads (8 wavefronts: 2 along M x 4 along N) owns a
+// 256 (M) x 256 (N) tile of y and walks K in steps of 64 through two LDS stages
+// (2 x 72 KiB).  Per step:
+//   * the x tile (256 x 64) and the packed W tile (256 rows x 64 codes) of the
+//     step after next are fetched into registers;
 //   * W is dequantized exactly once per workgroup -- thread (n, h) expands the
 //     32 codes [32h, 32h+32) of row n with one scale/bias pair (a K-step never
 //     holds more than one group per 32 codes) as fp32 fma(s, code, b), rounds to
-//     T and stores them to LDS, so the 256 rows of x reuse every weight;
+//     T and stores them to the idle LDS stage while the matrix cores work on
+//     the other one, so the 256 rows of x reuse every weight;
 //   * each wavefront computes a 64 (N) x 128 (M) block of y^T with
 //     v_mfma_f32_32x32x16: A operand = W rows, B operand = x rows, so that a lane
 //     ends up with 4 consecutive n of one m -- an 8-byte store of y.
@@ -27,10 +29,10 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kBM = 256;
-constexpr int kBN = 128;
+constexpr int kBN = 256;
 constexpr int kBK = 64;
 constexpr int kLdsStride = kBK + 8; // elements per LDS row
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 
 template <typename T>
 __device__ __forceinline__ floatx16 mfma32(const uint4& a, const uint4& b, const floatx16& c);
@@ -115,14 +117,18 @@ __device__ __forceinline__ void dequant32(
 
 template <typename T, int BITS, int GS>
 __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
-  __shared__ __attribute__((aligned(16))) T xs[kBM * kLdsStride];
-  __shared__ __attribute__((aligned(16))) T ws[kBN * kLdsStride];
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // two stages, each an x tile followed by a W tile
+  constexpr int kXTile = kBM * kLdsStride; // elements
+  constexpr int kWTile = kBN * kLdsStride;
+  constexpr int kStage = kXTile + kWTile;
+  T* lds = reinterpret_cast<T*>(smem);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wn = wave & 1;  // which 64 columns (n) of the tile
-  const int wm = wave >> 1; // which 128 rows (m) of the tile
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 3;  // which 64 columns (n) of the tile
+  const int wm = wave >> 2; // which 128 rows (m) of the tile
   const int M = a.M;
   const int N = a.N;
   const int K = a.K;
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
   const int row_words = K / 32 * BITS;
 
   // ---- loader roles ----
-  // x: thread covers 16-byte chunk (tid % 8) of rows tid/8 + 32 i, i < 8.
+  // x: thread covers 16-byte chunk (tid % 8) of rows tid/8 + 64 i, i < 4.
   const int xc = tid & 7;
   const int xr = tid >> 3;
   // W: thread (wr, wh) covers codes [32 wh, 32 wh + 32) of tile row wr.
@@ -145,43 +151,56 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
       static_cast<size_t>(w_row) * row_words + wh * BITS;
   const T* ssrc = p.scales + static_cast<size_t>(w_row) * groups;
   const T* bsrc = p.biases + static_cast<size_t>(w_row) * groups;
+  // Rows of x past M are never stored, so they may read any valid row: the
+  // loads then need no predicate.  32-bit element offsets from p.x.
+  uint32_t xoff0, xoff1, xoff2, xoff3;
+  {
+    auto row_off = [&](int i) {
+      const int m = m0 + xr + 64 * i;
+      return static_cast<uint32_t>(m < M ? m : M - 1) * static_cast<uint32_t>(K) + xc * 8;
+    };
+    xoff0 = row_off(0);
+    xoff1 = row_off(1);
+    xoff2 = row_off(2);
+    xoff3 = row_off(3);
+  }
 
-  uint4 xreg[8];
+  // registers of the tile in flight
+  uint4 xq0, xq1, xq2, xq3;
   uint32_t wreg[BITS];
-  float sreg, breg;
+  T sreg, breg; // converted when used, so the loads are not waited for early
 
-  auto load_tile = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int m = m0 + xr + 32 * i;
-      xreg[i] = make_uint4(0, 0, 0, 0);
-      if (m < M) {
-        xreg[i] = *reinterpret_cast<const uint4*>(p.x + static_cast<size_t>(m) * K + k0 + xc * 8);
-      }
-    }
-    const uint32_t* wp = wsrc + (k0 / 32) * BITS;
-#pragma unroll
-    for (int j = 0; j < BITS; ++j) {
-      wreg[j] = wp[j];
-    }
-    const int g = (k0 + 32 * wh) / GS;
-    sreg = to_f32(ssrc[g]);
-    breg = to_f32(bsrc[g]);
-  };
+#define QMM_LOAD_TILE(k0)                                                        \
+  do {                                                                           \
+    xq0 = *reinterpret_cast<const uint4*>(p.x + xoff0 + (k0));                   \
+    xq1 = *reinterpret_cast<const uint4*>(p.x + xoff1 + (k0));                   \
+    xq2 = *reinterpret_cast<const uint4*>(p.x + xoff2 + (k0));                   \
+    xq3 = *reinterpret_cast<const uint4*>(p.x + xoff3 + (k0));                   \
+    const uint32_t* wp__ = wsrc + ((k0) / 32) * BITS;                            \
+    _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
+      wreg[j__] = wp__[j__];                                                     \
+    }                                                                            \
+    const int g__ = ((k0) + 32 * wh) / GS;                                       \
+    sreg = ssrc[g__];                                                            \
+    breg = bsrc[g__];                                                            \
+  } while (0)
 
-  auto store_tile = [&]() {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      *reinterpret_cast<uint4*>(&xs[(xr + 32 * i) * kLdsStride + xc * 8]) = xreg[i];
-    }
-    uint32_t dq[16];
-    dequant32<T, BITS>(wreg, sreg, breg, dq);
-    uint4* dst = reinterpret_cast<uint4*>(&ws[wr * kLdsStride + wh * 32]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      dst[j] = make_uint4(dq[4 * j], dq[4 * j + 1], dq[4 * j + 2], dq[4 * j + 3]);
-    }
-  };
+#define QMM_STORE_TILE(stage)                                                    \
+  do {                                                                           \
+    T* xs__ = lds + (stage) * kStage;                                            \
+    T* ws__ = xs__ + kXTile;                                                     \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 0) * kLdsStride + xc * 8]) = xq0;      \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 64) * kLdsStride + xc * 8]) = xq1;     \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 128) * kLdsStride + xc * 8]) = xq2;    \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 192) * kLdsStride + xc * 8]) = xq3;    \
+    uint32_t dq__[16];                                                           \
+    dequant32<T, BITS>(wreg, to_f32(sreg), to_f32(breg), dq__);                  \
+    uint4* dst__ = reinterpret_cast<uint4*>(&ws__[wr * kLdsStride + wh * 32]);   \
+    _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                        \
+      dst__[j__] = make_uint4(                                                   \
+          dq__[4 * j__], dq__[4 * j__ + 1], dq__[4 * j__ + 2], dq__[4 * j__ + 3]); \
+    }                                                                            \
+  } while (0)
 
   // ---- accumulators: 2 (n) x 4 (m) tiles of 32 x 32 ----
   floatx16 acc[2][4];
@@ -198,17 +217,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
 
   const int fr = lane & 31; // fragment row inside a 32-row MFMA tile
   const int fk = lane >> 5; // which 8 of the 16 k of an MFMA step
-  const T* wfrag = &ws[(wn * 64 + fr) * kLdsStride + fk * 8];
-  const T* xfrag = &xs[(wm * 128 + fr) * kLdsStride + fk * 8];
+  const int xfrag_off = (wm * 128 + fr) * kLdsStride + fk * 8;
+  const int wfrag_off = kXTile + (wn * 64 + fr) * kLdsStride + fk * 8;
 
-  load_tile(0);
-  for (int k0 = 0; k0 < K; k0 += kBK) {
-    __syncthreads(); // the previous step's fragment reads are done
-    store_tile();
-    __syncthreads();
-    if (k0 + kBK < K) {
-      load_tile(k0 + kBK);
-    }
+  auto mfma_tile = [&](int stage) {
+    const T* xfrag = lds + stage * kStage + xfrag_off;
+    const T* wfrag = lds + stage * kStage + wfrag_off;
 #pragma unroll
     for (int kk = 0; kk < kBK / 16; ++kk) {
       uint4 af[2];
@@ -229,6 +243,27 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
         }
       }
     }
+  };
+
+  // ---- software pipeline: registers hold tile t+1 while LDS stage t%2 feeds
+  // the matrix cores; one barrier per K-step ----
+  const int nk = K / kBK;
+  QMM_LOAD_TILE(0);
+  QMM_STORE_TILE(0);
+  if (nk > 1) {
+    QMM_LOAD_TILE(kBK);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) {
+      QMM_STORE_TILE(cur ^ 1); // tile kt+1: dequantize + write the idle stage
+    }
+    if (kt + 2 < nk) {
+      QMM_LOAD_TILE((kt + 2) * kBK); // in flight during this step's MFMAs
+    }
+    mfma_tile(cur);
+    __syncthreads();
   }
 
   // ---- epilogue: D[n][m] tiles; register r of lane (col, half) holds
@@ -271,6 +306,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
   }
 }
 
+#undef QMM_LOAD_TILE
+#undef QMM_STORE_TILE
+
+constexpr size_t kQmmSmemBytes =
+    static_cast<size_t>(2) * (kBM + kBN) * kLdsStride * 2; // two stages, 16-bit
+
 } // namespace
 
 bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose) {
@@ -293,7 +334,16 @@ int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
       return dispatch_group(gs, [&](auto gval) {
         constexpr int B = decltype(bval)::value;
         constexpr int G = decltype(gval)::value;
-        qmm_t_mfma_kernel<T, B, G><<<grid, kThreads, 0, s>>>(a);
+        auto kern = qmm_t_mfma_kernel<T, B, G>;
+        static bool configured = false; // per instantiation
+        if (!configured) {
+          MLXROCM_HIP_TRY(hipFuncSetAttribute(
+              reinterpret_cast<const void*>(kern),
+              hipFuncAttributeMaxDynamicSharedMemorySize,
+              static_cast<int>(kQmmSmemBytes)));
+          configured = true;
+        }
+        kern<<<grid, kThreads, kQmmSmemBytes, s>>>(a);
         MLXROCM_HIP_TRY(hipGetLastError());
         return static_cast<int>(MLXROCM_OK);
       });
