@@ -1,0 +1,81 @@
+"""Argument validation of the Python operator mirror: same conditions and the
+same exception type (std::invalid_argument -> ValueError) as the reference's
+ops, python/tests/test_quantized.py:877-956.  Runs on the CPU: every check
+comes before the first device call."""
+import pytest
+import torch
+
+import mlx_amd
+
+
+def _triple(N=64, K=512, gs=64, bits=4, dtype=torch.float32):
+    wq = torch.zeros((N, K * bits // 32), dtype=torch.uint32)
+    s = torch.ones((N, K // gs), dtype=dtype)
+    return wq, s, torch.zeros_like(s)
+
+
+def test_quantize_errors():
+    with pytest.raises(ValueError, match="floating"):
+        mlx_amd.quantize(torch.zeros((4, 64), dtype=torch.int32))
+    with pytest.raises(ValueError, match="at least 2"):
+        mlx_amd.quantize(torch.zeros(64))
+    with pytest.raises(ValueError, match="divisible"):
+        mlx_amd.quantize(torch.zeros((4, 65)))
+    with pytest.raises(ValueError, match="group size"):
+        mlx_amd.quantize(torch.zeros((4, 96)), group_size=48)
+    with pytest.raises(ValueError, match="bits"):
+        mlx_amd.quantize(torch.zeros((4, 64)), bits=7)
+    with pytest.raises(ValueError, match="mode"):
+        mlx_amd.quantize(torch.zeros((4, 64)), mode="bogus")
+    with pytest.raises(RuntimeError, match="ROCm"):
+        mlx_amd.quantize(torch.zeros((4, 64)), mode="mxfp4")
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.quantize(torch.zeros((4, 64)))  # valid, but not on the device
+
+
+def test_quantized_matmul_errors():
+    wq, s, b = _triple()
+    x = torch.zeros((2, 512))
+    with pytest.raises(ValueError, match="Biases must be provided"):
+        mlx_amd.quantized_matmul(x, wq, s, None)
+    with pytest.raises(ValueError, match="uint32"):
+        mlx_amd.quantized_matmul(x, wq.view(torch.int32), s, b)
+    with pytest.raises(ValueError, match="same shape"):
+        mlx_amd.quantized_matmul(x, wq, s, b[:, :4])
+    with pytest.raises(ValueError, match="incompatible"):
+        mlx_amd.quantized_matmul(x, wq, s, b, group_size=32)
+    with pytest.raises(ValueError, match="does not match"):
+        mlx_amd.quantized_matmul(torch.zeros((2, 256)), wq, s, b)
+    with pytest.raises(ValueError, match="does not match"):
+        mlx_amd.quantized_matmul(x, wq, s, b, transpose=False)
+    with pytest.raises(ValueError, match="floating"):
+        mlx_amd.quantized_matmul(x, wq, s.to(torch.int32), b.to(torch.int32))
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.quantized_matmul(x, wq, s, b)
+
+
+def test_dequantize_errors():
+    wq, s, b = _triple()
+    with pytest.raises(ValueError, match="uint32"):
+        mlx_amd.dequantize(wq.view(torch.int32), s, b)
+    with pytest.raises(ValueError, match="does not match"):
+        mlx_amd.dequantize(wq, s[:32], b[:32])
+    with pytest.raises(ValueError, match="does not match"):
+        mlx_amd.dequantize(wq, s, b, group_size=128)
+    with pytest.raises(ValueError, match="floating"):
+        mlx_amd.dequantize(wq, s, b, dtype=torch.int32)
+    with pytest.raises(ValueError, match="at least 2"):
+        mlx_amd.dequantize(wq[0], s[0], b[0])
+
+
+def test_gather_qmm_errors_and_defaults():
+    wq, s, b = _triple()
+    wq3, s3, b3 = wq.reshape(1, 64, 64), s.reshape(1, 64, 8), b.reshape(1, 64, 8)
+    x = torch.zeros((3, 1, 512))
+    with pytest.raises(ValueError, match="integral"):
+        mlx_amd.gather_qmm(x, wq3, s3, b3, rhs_indices=torch.zeros(3))
+    with pytest.raises(ValueError, match="at least two"):
+        mlx_amd.gather_qmm(torch.zeros(512), wq3, s3, b3, rhs_indices=torch.zeros(3, dtype=torch.int64))
+    # without indices it is quantized_matmul (mlx/ops.cpp:5566-5569)
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.gather_qmm(x, wq, s, b)
