@@ -25,6 +25,11 @@ import time
 
 HBM_PEAK_GBPS = 8000.0
 BF16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes, scaled by
+# a copy of known size (profiles/qmv_stream_4bit_g64_bf16_14336x4096.md and
+# profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md).
+QMV_TRAFFIC_BYTES = 33224900
+QMM_T_TRAFFIC_BYTES = 276972000
 
 N, K = 14336, 4096
 BITS, GS = 4, 64
@@ -129,6 +134,9 @@ def main() -> int:
     ap.add_argument("--only", choices=("qmv", "qmm_t"), default=None)
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying a HIP graph")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run 20 device-to-device copies of 256 MiB: the known-size "
+                         "kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; this build has no multi-GPU path "
@@ -146,6 +154,17 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     dt = torch.bfloat16
+
+    if args.copy_probe:
+        nbytes = 256 << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        for _ in range(20):
+            _lib.check(lib.mlxrocm_memcpy_d2d(dst.data_ptr(), src.data_ptr(), nbytes, stream))
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes": nbytes, "copies": 20}))
+        return 0
 
     g = torch.Generator().manual_seed(0)
     x_cpu = torch.randn((1, K), generator=g, dtype=torch.float32).to(dt)
@@ -210,7 +229,7 @@ def main() -> int:
                 "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s",
                 "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                "traffic": None,
+                "traffic": QMV_TRAFFIC_BYTES,
                 "kernel_us": round(ev_ms * 1e3, 3),
                 "bytes_per_launch": nbytes,
                 "llc_resident_gbps": round(nbytes / (llc_ms * 1e-3) / 1e9, 2),
@@ -249,7 +268,7 @@ def main() -> int:
                 "peak": BF16_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
                 "frac": round(tflops / BF16_PEAK_TFLOPS, 4),
-                "traffic": None,
+                "traffic": QMM_T_TRAFFIC_BYTES,
             },
         }
 
