@@ -1,0 +1,260 @@
+// quantized.cpp -- eval_gpu of the affine quantization primitives for the ROCm
+// backend: QuantizedMatmul, GatherQMM and fast::Quantize
+// (mlx/primitives.h:1616-1717, mlx/fast_primitives.h:337-371).
+//
+// Each body does what the CUDA backend's does around its kernels
+// (mlx/backend/cuda/quantized/quantized.cpp:15-324): make operands dense where
+// the kernels need it, allocate the output, translate `array`s into the plain
+// pointers / sizes / strides of the C ABI, enqueue on the stream's encoder and
+// retain what the kernels read.  Every arithmetic decision (kernel choice,
+// tiling) lives behind mlxrocm_qmm / mlxrocm_gather_qmm.
+#include <sstream>
+#include <stdexcept>
+
+#include "mlx/allocator.h"
+#include "mlx/backend/gpu/copy.h"
+#include "mlx/fast_primitives.h"
+#include "mlx/primitives.h"
+#include "mlx/utils.h"
+
+#include "allocator.h"
+#include "device.h"
+
+namespace mlx::core {
+
+namespace {
+
+int dtype_code(Dtype t, const char* who) {
+  switch (t) {
+    case float32:
+      return MLXROCM_FLOAT32;
+    case float16:
+      return MLXROCM_FLOAT16;
+    case bfloat16:
+      return MLXROCM_BFLOAT16;
+    default: {
+      std::ostringstream msg;
+      msg << "[" << who << "] Only float32, float16 and bfloat16 are supported "
+          << "by the ROCm backend but got " << t << ".";
+      throw std::runtime_error(msg.str());
+    }
+  }
+}
+
+void require_affine(QuantizationMode mode, const char* who) {
+  if (mode != QuantizationMode::Affine) {
+    std::ostringstream msg;
+    msg << "[" << who << "] quantization mode '"
+        << quantization_mode_to_string(mode)
+        << "' has no ROCm implementation; only 'affine' is supported.";
+    throw std::runtime_error(msg.str());
+  }
+}
+
+array ensure_row_contiguous(
+    const array& x,
+    rocm::CommandEncoder& enc,
+    const Stream& s) {
+  // The kernels use 16-byte vector loads: a view that starts off that grid is
+  // copied like a strided one.
+  if (x.flags().row_contiguous && x.offset() % 16 == 0) {
+    return x;
+  }
+  array copy = contiguous_copy_gpu(x, s);
+  enc.add_temporary(copy);
+  return copy;
+}
+
+// Only the trailing matrix has to be dense (mlx/backend/cpu/quantized.cpp:974-990);
+// leading dims keep their strides.
+array ensure_dense_matrices(
+    const array& x,
+    rocm::CommandEncoder& enc,
+    const Stream& s) {
+  if (x.ndim() >= 2 && x.strides()[x.ndim() - 1] == 1 &&
+      x.strides()[x.ndim() - 2] == x.shape(-1) && x.offset() % 16 == 0) {
+    return x;
+  }
+  array copy = contiguous_copy_gpu(x, s);
+  enc.add_temporary(copy);
+  return copy;
+}
+
+// Stride between consecutive matrices of a stack whose leading dims are
+// either absent, a single dim, or row-contiguous.
+int64_t matrix_stride(const array& a) {
+  if (a.ndim() <= 2) {
+    return 0;
+  }
+  return a.strides()[a.ndim() - 3];
+}
+
+bool single_batch_stride(const array& a) {
+  // true when element i of the flattened leading dims sits at i * stride
+  int64_t expect = matrix_stride(a);
+  for (int d = a.ndim() - 3; d >= 0; --d) {
+    if (a.shape(d) != 1 && a.strides()[d] != expect) {
+      return false;
+    }
+    expect *= a.shape(d);
+  }
+  return true;
+}
+
+} // namespace
+
+void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
+  require_affine(mode_, "quantized_matmul");
+  auto& s = stream();
+  auto& enc = rocm::get_command_encoder(s);
+
+  array x = ensure_row_contiguous(inputs[0], enc, s);
+  array w = ensure_row_contiguous(inputs[1], enc, s);
+  array scales = ensure_row_contiguous(inputs[2], enc, s);
+  array biases = ensure_row_contiguous(inputs[3], enc, s);
+
+  out.set_data(allocator::malloc(out.nbytes()));
+
+  const int K = x.shape(-1);
+  const int M = x.ndim() > 1 ? x.shape(-2) : 1;
+  const int N = out.shape(-1);
+  const int L = (M == 0 || K == 0) ? 0 : static_cast<int>(x.size() / (size_t(K) * M));
+  // w.ndim() == 2: one weight for every batch (mlx/backend/cpu/quantized.cpp:396-397)
+  const int64_t w_stride = w.ndim() > 2 ? int64_t(w.shape(-1)) * w.shape(-2) : 0;
+  const int64_t sb_stride =
+      w.ndim() > 2 ? int64_t(scales.shape(-1)) * scales.shape(-2) : 0;
+
+  rocm::check(mlxrocm_qmm(
+      rocm::gpu_ptr<void>(x, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(w, enc.stream()),
+      rocm::gpu_ptr<void>(scales, enc.stream()),
+      rocm::gpu_ptr<void>(biases, enc.stream()),
+      rocm::gpu_ptr<void>(out, enc.stream()),
+      M,
+      N,
+      K,
+      L,
+      int64_t(M) * K,
+      w_stride,
+      sb_stride,
+      group_size_,
+      bits_,
+      dtype_code(x.dtype(), "quantized_matmul"),
+      transpose_ ? 1 : 0,
+      enc.stream()));
+}
+
+void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
+  require_affine(mode_, "gather_qmm");
+  auto& s = stream();
+  auto& enc = rocm::get_command_encoder(s);
+
+  array x = ensure_row_contiguous(inputs[0], enc, s);
+  array w = ensure_dense_matrices(inputs[1], enc, s);
+  array scales = ensure_dense_matrices(inputs[2], enc, s);
+  array biases = ensure_dense_matrices(inputs[3], enc, s);
+  // A stack the kernels can address as base + e * stride keeps its layout
+  // (sliced expert stacks); anything more exotic is made dense.
+  if (!single_batch_stride(w) || !single_batch_stride(scales) ||
+      !single_batch_stride(biases) ||
+      matrix_stride(scales) != matrix_stride(biases)) {
+    w = ensure_row_contiguous(w, enc, s);
+    scales = ensure_row_contiguous(scales, enc, s);
+    biases = ensure_row_contiguous(biases, enc, s);
+  }
+  array lhs = ensure_row_contiguous(inputs[4], enc, s);
+  array rhs = ensure_row_contiguous(inputs[5], enc, s);
+
+  out.set_data(allocator::malloc(out.nbytes()));
+
+  const int K = x.shape(-1);
+  const int M = x.shape(-2);
+  const int N = out.shape(-1);
+  const int n_idx = static_cast<int>(lhs.size());
+  const int x_batches = (M == 0 || K == 0) ? 0 : static_cast<int>(x.size() / (size_t(K) * M));
+  const int n_experts =
+      static_cast<int>(w.size() / (size_t(w.shape(-1)) * w.shape(-2)));
+  const int dt = dtype_code(x.dtype(), "gather_qmm");
+
+  const size_t ws_bytes = mlxrocm_gather_qmm_workspace_size(
+      M, N, K, n_idx, n_experts, group_size_, bits_, dt, transpose_, right_sorted_);
+  void* ws_ptr = nullptr;
+  if (ws_bytes > 0) {
+    array ws({static_cast<int>(ws_bytes)}, uint8, nullptr, {});
+    ws.set_data(allocator::malloc(ws_bytes));
+    enc.add_temporary(ws);
+    ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
+  }
+
+  rocm::check(mlxrocm_gather_qmm(
+      rocm::gpu_ptr<void>(x, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(w, enc.stream()),
+      rocm::gpu_ptr<void>(scales, enc.stream()),
+      rocm::gpu_ptr<void>(biases, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(lhs, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(rhs, enc.stream()),
+      rocm::gpu_ptr<void>(out, enc.stream()),
+      M,
+      N,
+      K,
+      n_idx,
+      x_batches,
+      n_experts,
+      int64_t(M) * K,
+      w.ndim() > 2 ? matrix_stride(w) : 0,
+      scales.ndim() > 2 ? matrix_stride(scales) : 0,
+      group_size_,
+      bits_,
+      dt,
+      transpose_ ? 1 : 0,
+      right_sorted_ ? 1 : 0,
+      ws_ptr,
+      ws_bytes,
+      enc.stream()));
+}
+
+void fast::Quantize::eval_gpu(
+    const std::vector<array>& inputs,
+    std::vector<array>& outputs) {
+  require_affine(mode_, "quantize");
+  auto& s = stream();
+  auto& enc = rocm::get_command_encoder(s);
+
+  if (dequantize_) {
+    array wq = ensure_row_contiguous(inputs[0], enc, s);
+    array scales = ensure_row_contiguous(inputs[1], enc, s);
+    array biases = ensure_row_contiguous(inputs[2], enc, s);
+    array& w = outputs[0];
+    w.set_data(allocator::malloc(w.nbytes()));
+    rocm::check(mlxrocm_affine_dequantize(
+        rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+        rocm::gpu_ptr<void>(scales, enc.stream()),
+        rocm::gpu_ptr<void>(biases, enc.stream()),
+        rocm::gpu_ptr<void>(w, enc.stream()),
+        w.size(),
+        group_size_,
+        bits_,
+        dtype_code(w.dtype(), "dequantize"),
+        enc.stream()));
+  } else {
+    array w = ensure_row_contiguous(inputs[0], enc, s);
+    array& wq = outputs[0];
+    array& scales = outputs[1];
+    array& biases = outputs[2];
+    wq.set_data(allocator::malloc(wq.nbytes()));
+    scales.set_data(allocator::malloc(scales.nbytes()));
+    biases.set_data(allocator::malloc(biases.nbytes()));
+    rocm::check(mlxrocm_affine_quantize(
+        rocm::gpu_ptr<void>(w, enc.stream()),
+        rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+        rocm::gpu_ptr<void>(scales, enc.stream()),
+        rocm::gpu_ptr<void>(biases, enc.stream()),
+        w.size(),
+        group_size_,
+        bits_,
+        dtype_code(w.dtype(), "quantize"),
+        enc.stream()));
+  }
+}
+
+} // namespace mlx::core

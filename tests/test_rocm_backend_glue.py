@@ -1,0 +1,57 @@
+"""The C++ host glue (mlx_amd/rocm_backend) type-checks against MLX's own headers.
+
+The glue is the reference-side binding of the C ABI: `eval_gpu` bodies of
+QuantizedMatmul / GatherQMM / fast::Quantize plus allocator, stream encoder and
+event over `mlxrocm_*`.  It can only be compiled where the MLX source tree is
+present; on a machine without it the test is skipped.
+"""
+import os
+import shutil
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+GLUE = ROOT / "mlx_amd" / "rocm_backend"
+MLX_TREE = Path(os.environ.get("MLX_SOURCE_DIR", "/root/reference"))
+
+SOURCES = sorted(p.name for p in GLUE.glob("*.cpp"))
+
+
+def _syntax_check(name):
+    cmd = [
+        "g++", "-std=c++20", "-fsyntax-only", "-Wall", "-Werror=return-type",
+        f"-I{MLX_TREE}", f"-I{ROOT / 'include'}", f"-I{GLUE}", str(GLUE / name),
+    ]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    return name, proc.returncode, proc.stderr
+
+
+@pytest.mark.skipif(not (MLX_TREE / "mlx" / "primitives.h").exists(),
+                    reason="MLX source tree not present")
+@pytest.mark.skipif(shutil.which("g++") is None, reason="g++ not present")
+def test_glue_compiles_against_mlx_headers():
+    assert SOURCES, "no glue sources found"
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        results = list(pool.map(_syntax_check, SOURCES))
+    failed = [(n, err) for n, rc, err in results if rc != 0]
+    assert not failed, "\n".join(f"{n}:\n{err}" for n, err in failed)
+
+
+def test_glue_defines_the_three_eval_gpu_bodies():
+    text = (GLUE / "quantized.cpp").read_text()
+    for sig in ("void QuantizedMatmul::eval_gpu(", "void GatherQMM::eval_gpu(",
+                "void fast::Quantize::eval_gpu("):
+        assert sig in text
+
+
+def test_glue_calls_only_declared_abi_symbols():
+    import re
+    header = (ROOT / "include" / "mlx_rocm_qmm.h").read_text()
+    declared = set(re.findall(r"\b(mlxrocm_[a-z0-9_]+)\s*\(", header))
+    used = set()
+    for p in list(GLUE.glob("*.cpp")) + list(GLUE.glob("*.h")):
+        used |= set(re.findall(r"\b(mlxrocm_[a-z0-9_]+)\s*\(", p.read_text()))
+    assert used <= declared, sorted(used - declared)
