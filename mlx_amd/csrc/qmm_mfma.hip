@@ -51,15 +51,15 @@ mfma32<f16_t>(const uint4& a, const uint4& b, const floatx16& c) {
       __builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+// Two floats -> two T in one dword (lo in the low half), round to nearest even;
+// the vector convert selects the packed hardware convert.
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  union {
-    T h[2];
-    uint32_t u;
-  } r;
-  r.h[0] = static_cast<T>(lo);
-  r.h[1] = static_cast<T>(hi);
-  return r.u;
+  typedef T Tx2 __attribute__((ext_vector_type(2)));
+  const floatx2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, Tx2));
 }
 
 // Code i (0..31) of the 32 codes held in BITS consecutive dwords.
@@ -86,8 +86,11 @@ __device__ __forceinline__ void dequant32(
     // nibbles -> bytes first, so that every convert is a cvt_f32_ubyteN
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const uint32_t lo = w[d] & 0x0f0f0f0fu;        // codes 0,2,4,6
-      const uint32_t hi = (w[d] >> 4) & 0x0f0f0f0fu; // codes 1,3,5,7
+      uint32_t lo = w[d] & 0x0f0f0f0fu;        // codes 0,2,4,6
+      uint32_t hi = (w[d] >> 4) & 0x0f0f0f0fu; // codes 1,3,5,7
+      // keep the byte form: otherwise the shifts are folded back into one
+      // bit-field extract per code
+      asm volatile("" : "+v"(lo), "+v"(hi));
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float c0 = static_cast<float>((lo >> (8 * j)) & 0xffu);
@@ -246,7 +249,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
   };
 
   // ---- software pipeline: registers hold tile t+1 while LDS stage t%2 feeds
-  // the matrix cores; one barrier per K-step ----
+  // the matrix cores.  The two wavefronts that share a SIMD (wm = 0 and 1)
+  // work in opposite phases: while one issues the MFMAs of tile t, the other
+  // dequantizes and stores its share of tile t+1 and fetches tile t+2, so the
+  // matrix pipe and the vector ALU of a SIMD are busy at the same time.  Tile
+  // t+1 is complete after both phases; stage (t+1)%2 was last read in step t-1.
   const int nk = K / kBK;
   QMM_LOAD_TILE(0);
   QMM_STORE_TILE(0);
@@ -254,17 +261,37 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
     QMM_LOAD_TILE(kBK);
   }
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) {
-      QMM_STORE_TILE(cur ^ 1); // tile kt+1: dequantize + write the idle stage
-    }
-    if (kt + 2 < nk) {
-      QMM_LOAD_TILE((kt + 2) * kBK); // in flight during this step's MFMAs
-    }
-    mfma_tile(cur);
+  // wm = 0: compute(t), store(t+1), compute(t+1), ...
+  // wm = 1: store(1), compute(0), store(2), compute(1), ...
+  // with a barrier after every phase; both sides execute 2 nk + 1 barriers.
+#define QMM_MEM_PHASE(ts)                                                        \
+  do {                                                                           \
+    const int ts__ = (ts);                                                       \
+    if (ts__ < nk) {                                                             \
+      QMM_STORE_TILE(ts__ & 1);                                                  \
+    }                                                                            \
+    /* unconditional: past the end the last tile is fetched again and never     \
+       stored, which keeps the loaded registers free of a select */             \
+    const int tl__ = ts__ + 1 < nk ? ts__ + 1 : nk - 1;                          \
+    QMM_LOAD_TILE(tl__ * kBK);                                                   \
+  } while (0)
+
+  if (wm == 1) {
+    QMM_MEM_PHASE(1);
     __syncthreads();
   }
+  for (int t = 0; t < nk; ++t) {
+    __builtin_amdgcn_s_setprio(1);
+    mfma_tile(t & 1);
+    __builtin_amdgcn_s_setprio(0);
+    __syncthreads();
+    QMM_MEM_PHASE(t + 1 + wm);
+    __syncthreads();
+  }
+  if (wm == 0) {
+    __syncthreads();
+  }
+#undef QMM_MEM_PHASE
 
   // ---- epilogue: D[n][m] tiles; register r of lane (col, half) holds
   // n = 8 (r / 4) + 4 half + r % 4, m = col.  Four consecutive n -> one 8-byte
