@@ -3,21 +3,29 @@
 //
 //   y[M, N] = x[M, K] * dequant(W)[N, K]^T
 //
-// A workgroup of 512 threads (8 wavefronts: 2 along M x 4 along N) owns a
-// 256 (M) x 256 (N) tile of y and walks K in steps of 64 through two LDS stages
-// (2 x 72 KiB).  Per step:
-//   * the x tile (256 x 64) and the packed W tile (256 rows x 64 codes) of the
+// A workgroup of 512 threads (8 wavefronts: 4 along M x 2 along N) owns a
+// 256 (M) x BN (N) tile of y, BN = 32 NT with NT in {6, 7, 8} chosen on the host
+// so that the tile count fills the compute units evenly, and walks K in steps
+// of 64 through two LDS stages.  Per step:
+//   * the x tile (256 x 64) and the packed W tile (BN rows x 64 codes) of the
 //     step after next are fetched into registers;
 //   * W is dequantized exactly once per workgroup -- thread (n, h) expands the
 //     32 codes [32h, 32h+32) of row n with one scale/bias pair (a K-step never
 //     holds more than one group per 32 codes) as fp32 fma(s, code, b), rounds to
-//     T and stores them to the idle LDS stage while the matrix cores work on
-//     the other one, so the 256 rows of x reuse every weight;
-//   * each wavefront computes a 64 (N) x 128 (M) block of y^T with
-//     v_mfma_f32_32x32x16: A operand = W rows, B operand = x rows, so that a lane
-//     ends up with 4 consecutive n of one m -- an 8-byte store of y.
+//     T and stores them to the idle LDS stage, so the 256 rows of x reuse every
+//     weight;
+//   * each wavefront computes a 16 NT (N) x 64 (M) block of y^T with
+//     v_mfma_f32_16x16x32: A operand = W rows, B operand = x rows, so that a lane
+//     ends up with 4 consecutive n of one m.
+// The vector-ALU, LDS and global-memory instructions of a step are placed by
+// hand in the slots between the MFMAs (one scheduling barrier per slot), so the
+// matrix pipe never waits for a block of dequantization work.
 // LDS rows are 64 elements + 8 of padding (144 bytes), which makes the 16-byte
-// fragment reads of 16 consecutive rows hit 64 distinct banks.
+// fragment reads of 16 consecutive rows hit 64 distinct banks.  The finished
+// tile is staged through LDS once more so that y is written in full 16-byte,
+// row-contiguous stores.
+#include <utility>
+
 #include "qmm_args.h"
 
 namespace mlxrocm {
@@ -26,32 +34,31 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBM = 256;
-constexpr int kBN = 256;
 constexpr int kBK = 64;
 constexpr int kLdsStride = kBK + 8; // elements per LDS row
 constexpr int kThreads = 512;
+constexpr int kOutPad = 8; // elements of padding per row of the staged y tile
 
 template <typename T>
-__device__ __forceinline__ floatx16 mfma32(const uint4& a, const uint4& b, const floatx16& c);
+__device__ __forceinline__ floatx4 mfma16(const uint4& a, const uint4& b, const floatx4& c);
 
 template <>
-__device__ __forceinline__ floatx16
-mfma32<bf16_t>(const uint4& a, const uint4& b, const floatx16& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+__device__ __forceinline__ floatx4
+mfma16<bf16_t>(const uint4& a, const uint4& b, const floatx4& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
       __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
 template <>
-__device__ __forceinline__ floatx16
-mfma32<f16_t>(const uint4& a, const uint4& b, const floatx16& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+__device__ __forceinline__ floatx4
+mfma16<f16_t>(const uint4& a, const uint4& b, const floatx4& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(
       __builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
-
-typedef float floatx2 __attribute__((ext_vector_type(2)));
 
 // Two floats -> two T in one dword (lo in the low half), round to nearest even;
 // the vector convert selects the packed hardware convert.
@@ -75,51 +82,91 @@ __device__ __forceinline__ uint32_t code32(const uint32_t (&w)[BITS], int i) {
   return v & ((1u << BITS) - 1u);
 }
 
-// 32 codes -> 32 elements of T: fma(s, code, b) in fp32, one rounding to T.
+// Dequantization of the 32 codes held in BITS consecutive dwords, two codes at
+// a time so that the work can be spread between MFMAs: pair<Q>() returns
+// elements 2Q and 2Q+1 as fma(s, code, b) in fp32, rounded once to T and packed.
+template <typename T, int BITS>
+struct PairDequant {
+  uint32_t lo, hi; // 4-bit: codes 0,2,4,6 / 1,3,5,7 of the current dword as bytes
+
+  template <int Q>
+  __device__ __forceinline__ uint32_t pair(const uint32_t (&w)[BITS], float s, float b) {
+    float c0, c1;
+    if constexpr (BITS == 4) {
+      constexpr int d = Q / 4;
+      constexpr int j = Q % 4;
+      if constexpr (j == 0) {
+        lo = w[d] & 0x0f0f0f0fu;
+        hi = (w[d] >> 4) & 0x0f0f0f0fu;
+        // keep the byte form: otherwise the shifts are folded back into one
+        // bit-field extract per code
+        asm("" : "+v"(lo));
+        asm("" : "+v"(hi));
+      }
+      c0 = static_cast<float>((lo >> (8 * j)) & 0xffu);
+      c1 = static_cast<float>((hi >> (8 * j)) & 0xffu);
+    } else if constexpr (BITS == 8) {
+      constexpr int d = Q / 2;
+      constexpr int j = Q % 2;
+      c0 = static_cast<float>((w[d] >> (16 * j)) & 0xffu);
+      c1 = static_cast<float>((w[d] >> (16 * j + 8)) & 0xffu);
+    } else {
+      c0 = static_cast<float>(code32<BITS>(w, 2 * Q));
+      c1 = static_cast<float>(code32<BITS>(w, 2 * Q + 1));
+    }
+    return pack2<T>(fmaf(s, c0, b), fmaf(s, c1, b));
+  }
+};
+
+template <typename T, int BITS, int... Q>
+__device__ __forceinline__ void dequant32_impl(
+    const uint32_t (&w)[BITS],
+    float s,
+    float b,
+    uint32_t (&out)[16],
+    std::integer_sequence<int, Q...>) {
+  PairDequant<T, BITS> dq;
+  ((out[Q] = dq.template pair<Q>(w, s, b)), ...);
+}
+
+// 32 codes -> 32 elements of T in one go (prologue).
 template <typename T, int BITS>
 __device__ __forceinline__ void dequant32(
     const uint32_t (&w)[BITS],
     float s,
     float b,
     uint32_t (&out)[16]) {
-  if constexpr (BITS == 4) {
-    // nibbles -> bytes first, so that every convert is a cvt_f32_ubyteN
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      uint32_t lo = w[d] & 0x0f0f0f0fu;        // codes 0,2,4,6
-      uint32_t hi = (w[d] >> 4) & 0x0f0f0f0fu; // codes 1,3,5,7
-      // keep the byte form: otherwise the shifts are folded back into one
-      // bit-field extract per code
-      asm volatile("" : "+v"(lo), "+v"(hi));
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float c0 = static_cast<float>((lo >> (8 * j)) & 0xffu);
-        const float c1 = static_cast<float>((hi >> (8 * j)) & 0xffu);
-        out[4 * d + j] = pack2<T>(fmaf(s, c0, b), fmaf(s, c1, b));
-      }
-    }
-  } else if constexpr (BITS == 8) {
-#pragma unroll
-    for (int d = 0; d < 8; ++d) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const float c0 = static_cast<float>((w[d] >> (16 * j)) & 0xffu);
-        const float c1 = static_cast<float>((w[d] >> (16 * j + 8)) & 0xffu);
-        out[2 * d + j] = pack2<T>(fmaf(s, c0, b), fmaf(s, c1, b));
-      }
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float c0 = static_cast<float>(code32<BITS>(w, 2 * i));
-      const float c1 = static_cast<float>(code32<BITS>(w, 2 * i + 1));
-      out[i] = pack2<T>(fmaf(s, c0, b), fmaf(s, c1, b));
-    }
-  }
+  dequant32_impl<T, BITS>(w, s, b, out, std::make_integer_sequence<int, 16>{});
 }
 
-template <typename T, int BITS, int GS>
-__global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
+// ---- placement of the side work in the MFMA slots of one K-step -------------
+// NS = 8 NT slots.  Dequantization pair q (0..15) goes to slot q NS / 16, the
+// 16-byte store of pairs 4r..4r+3 to the slot after pair 4r+3, the x store +
+// refetch of row block i to slot 4i + 1 and the packed-W fetch to slot 0.
+constexpr int pair_slot(int q, int ns) {
+  return q * ns / 16;
+}
+constexpr int pair_at(int m, int ns) {
+  for (int q = 0; q < 16; ++q) {
+    if (pair_slot(q, ns) == m) {
+      return q;
+    }
+  }
+  return -1;
+}
+constexpr int wstore_at(int m, int ns) {
+  for (int r = 0; r < 4; ++r) {
+    if (pair_slot(4 * r + 3, ns) + 1 == m) {
+      return r;
+    }
+  }
+  return -1;
+}
+
+template <typename T, int BITS, int NT>
+__global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, const int gs_shift) {
+  constexpr int kBN = 32 * NT;
+  constexpr int kNS = 8 * NT; // MFMAs per wavefront per K-step
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // two stages, each an x tile followed by a W tile
   constexpr int kXTile = kBM * kLdsStride; // elements
@@ -130,8 +177,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wn = wave & 3;  // which 64 columns (n) of the tile
-  const int wm = wave >> 2; // which 128 rows (m) of the tile
+  const int wn = wave & 1;  // which 16 NT columns (n) of the tile
+  const int wm = wave >> 1; // which 64 rows (m) of the tile
   const int M = a.M;
   const int N = a.N;
   const int K = a.K;
@@ -139,15 +186,16 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
   const int m0 = blockIdx.y * kBM;
   const QmmProblem<T> p = resolve_problem<T>(a, blockIdx.z);
 
-  const int groups = K / GS;
+  const int groups = K >> gs_shift;
   const int row_words = K / 32 * BITS;
 
   // ---- loader roles ----
   // x: thread covers 16-byte chunk (tid % 8) of rows tid/8 + 64 i, i < 4.
   const int xc = tid & 7;
   const int xr = tid >> 3;
-  // W: thread (wr, wh) covers codes [32 wh, 32 wh + 32) of tile row wr.
-  const int wr = tid >> 1;
+  // W: thread (wr, wh) covers codes [32 wh, 32 wh + 32) of tile row wr; rows
+  // past the tile (NT < 8) are clamped and land in LDS padding that is unused.
+  const int wr = (tid >> 1) < kBN ? (tid >> 1) : kBN - 1;
   const int wh = tid & 1;
   const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
   const uint32_t* wsrc = reinterpret_cast<const uint32_t*>(p.w) +
@@ -168,34 +216,52 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
     xoff3 = row_off(3);
   }
 
-  // registers of the tile in flight
+  // registers of the tiles in flight: x and the packed W of the next K-step,
+  // and the packed W of the step after that (wnext), fetched a whole step ahead
   uint4 xq0, xq1, xq2, xq3;
-  uint32_t wreg[BITS];
-  T sreg, breg; // converted when used, so the loads are not waited for early
+  uint32_t wreg[BITS], wnext[BITS];
+  T sreg, breg, snext, bnext; // converted when used, so the loads are not waited for early
 
-#define QMM_LOAD_TILE(k0)                                                        \
+#define QMM_LOAD_X(k0)                                                           \
   do {                                                                           \
     xq0 = *reinterpret_cast<const uint4*>(p.x + xoff0 + (k0));                   \
     xq1 = *reinterpret_cast<const uint4*>(p.x + xoff1 + (k0));                   \
     xq2 = *reinterpret_cast<const uint4*>(p.x + xoff2 + (k0));                   \
     xq3 = *reinterpret_cast<const uint4*>(p.x + xoff3 + (k0));                   \
-    const uint32_t* wp__ = wsrc + ((k0) / 32) * BITS;                            \
-    _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
-      wreg[j__] = wp__[j__];                                                     \
-    }                                                                            \
-    const int g__ = ((k0) + 32 * wh) / GS;                                       \
-    sreg = ssrc[g__];                                                            \
-    breg = bsrc[g__];                                                            \
   } while (0)
 
-#define QMM_STORE_TILE(stage)                                                    \
+#define QMM_LOAD_W(k0)                                                           \
+  do {                                                                           \
+    const uint32_t* wp__ = wsrc + ((k0) / 32) * BITS;                            \
+    _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
+      wnext[j__] = wp__[j__];                                                    \
+    }                                                                            \
+    const int g__ = ((k0) + 32 * wh) >> gs_shift;                                \
+    snext = ssrc[g__];                                                           \
+    bnext = bsrc[g__];                                                           \
+  } while (0)
+
+#define QMM_ROTATE_W()                                                           \
+  do {                                                                           \
+    _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
+      wreg[j__] = wnext[j__];                                                    \
+    }                                                                            \
+    sreg = snext;                                                                \
+    breg = bnext;                                                                \
+  } while (0)
+
+#define QMM_STORE_X(stage)                                                       \
   do {                                                                           \
     T* xs__ = lds + (stage) * kStage;                                            \
-    T* ws__ = xs__ + kXTile;                                                     \
     *reinterpret_cast<uint4*>(&xs__[(xr + 0) * kLdsStride + xc * 8]) = xq0;      \
     *reinterpret_cast<uint4*>(&xs__[(xr + 64) * kLdsStride + xc * 8]) = xq1;     \
     *reinterpret_cast<uint4*>(&xs__[(xr + 128) * kLdsStride + xc * 8]) = xq2;    \
     *reinterpret_cast<uint4*>(&xs__[(xr + 192) * kLdsStride + xc * 8]) = xq3;    \
+  } while (0)
+
+#define QMM_STORE_W(stage)                                                       \
+  do {                                                                           \
+    T* ws__ = lds + (stage) * kStage + kXTile;                                   \
     uint32_t dq__[16];                                                           \
     dequant32<T, BITS>(wreg, to_f32(sreg), to_f32(breg), dq__);                  \
     uint4* dst__ = reinterpret_cast<uint4*>(&ws__[wr * kLdsStride + wh * 32]);   \
@@ -205,127 +271,212 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
     }                                                                            \
   } while (0)
 
-  // ---- accumulators: 2 (n) x 4 (m) tiles of 32 x 32 ----
-  floatx16 acc[2][4];
+  // ---- accumulators: NT (n) x 4 (m) tiles of 16 x 16 ----
+  floatx4 acc[NT][4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < NT; ++i) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int r = 0; r < 4; ++r) {
         acc[i][j][r] = 0.0f;
       }
     }
   }
 
-  const int fr = lane & 31; // fragment row inside a 32-row MFMA tile
-  const int fk = lane >> 5; // which 8 of the 16 k of an MFMA step
-  const int xfrag_off = (wm * 128 + fr) * kLdsStride + fk * 8;
-  const int wfrag_off = kXTile + (wn * 64 + fr) * kLdsStride + fk * 8;
+  const int fi = lane & 15; // fragment row inside a 16-row MFMA tile
+  const int fk = lane >> 4; // which 8 of the 32 k of an MFMA step
+  const int xfrag_off = (wm * 64 + fi) * kLdsStride + fk * 8;
+  const int wfrag_off = kXTile + (wn * 16 * NT + fi) * kLdsStride + fk * 8;
 
-  auto mfma_tile = [&](int stage) {
-    const T* xfrag = lds + stage * kStage + xfrag_off;
-    const T* wfrag = lds + stage * kStage + wfrag_off;
-#pragma unroll
-    for (int kk = 0; kk < kBK / 16; ++kk) {
-      uint4 af[2];
-      uint4 bf[4];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        af[i] = *reinterpret_cast<const uint4*>(wfrag + i * 32 * kLdsStride + kk * 16);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        bf[j] = *reinterpret_cast<const uint4*>(xfrag + j * 32 * kLdsStride + kk * 16);
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
-        }
-      }
-    }
+  // MFMA operand fragments.  All four x fragments of a 32-wide k slice stay in
+  // registers (two sets, one per slice); the W fragments stream through a ring
+  // of three, each read two groups of four MFMAs before its first use.
+  uint4 bfr[2][4];
+  uint4 afr[3];
+  auto read_b = [&](int stage, int s, int b) {
+    bfr[s][b] = *reinterpret_cast<const uint4*>(
+        lds + stage * kStage + xfrag_off + b * 16 * kLdsStride + s * 32);
+  };
+  auto read_a = [&](int stage, int s, int t, int slot) {
+    afr[slot] = *reinterpret_cast<const uint4*>(
+        lds + stage * kStage + wfrag_off + t * 16 * kLdsStride + s * 32);
   };
 
-  // ---- software pipeline: registers hold tile t+1 while LDS stage t%2 feeds
-  // the matrix cores.  The two wavefronts that share a SIMD (wm = 0 and 1)
-  // work in opposite phases: while one issues the MFMAs of tile t, the other
-  // dequantizes and stores its share of tile t+1 and fetches tile t+2, so the
-  // matrix pipe and the vector ALU of a SIMD are busy at the same time.  Tile
-  // t+1 is complete after both phases; stage (t+1)%2 was last read in step t-1.
+  // ---- software pipeline, one barrier per K-step.  Step t issues 8 NT MFMAs
+  // on tile t (LDS stage t%2); the slots between them carry, in a fixed order,
+  //   * the fragment reads that the MFMAs two groups later need,
+  //   * the dequantization of this thread's 32 codes of W tile t+1 (two codes
+  //     per slot) and its four 16-byte stores to the idle stage,
+  //   * the stores of x tile t+1 (fetched during step t-1), each followed by
+  //     the fetch of the same rows of x tile t+2,
+  //   * the fetch of the packed W of tile t+2 (one step ahead of its use).
+  // Fetches past the last step are clamped to the last tile (never stored), so
+  // the loop body has no branch.
   const int nk = K / kBK;
-  QMM_LOAD_TILE(0);
-  QMM_STORE_TILE(0);
-  if (nk > 1) {
-    QMM_LOAD_TILE(kBK);
+  const int klast = (nk - 1) * kBK;
+  QMM_LOAD_X(0);
+  QMM_LOAD_W(0);
+  QMM_ROTATE_W();
+  QMM_STORE_X(0);
+  QMM_STORE_W(0);
+  {
+    const int k1 = nk > 1 ? kBK : 0;
+    QMM_LOAD_X(k1);
+    QMM_LOAD_W(k1);
+    QMM_ROTATE_W();
   }
   __syncthreads();
-  // wm = 0: compute(t), store(t+1), compute(t+1), ...
-  // wm = 1: store(1), compute(0), store(2), compute(1), ...
-  // with a barrier after every phase; both sides execute 2 nk + 1 barriers.
-#define QMM_MEM_PHASE(ts)                                                        \
-  do {                                                                           \
-    const int ts__ = (ts);                                                       \
-    if (ts__ < nk) {                                                             \
-      QMM_STORE_TILE(ts__ & 1);                                                  \
+
+  // One slot: MFMA number m of the step and the side work assigned to it.
+  // PREP = 1 in the main loop, 0 in the last step (nothing left to prepare).
+#define QMM_SLOT(m, PREP)                                                        \
+  if constexpr ((m) < kNS) {                                                     \
+    constexpr int s__ = (m) / (4 * NT);                                          \
+    constexpr int t__ = ((m) % (4 * NT)) / 4;                                    \
+    constexpr int b__ = (m) % 4;                                                 \
+    constexpr int g__ = s__ * NT + t__; /* running W-fragment number */          \
+    acc[t__][b__] = mfma16<T>(afr[g__ % 3], bfr[s__][b__], acc[t__][b__]);       \
+    if constexpr (b__ == 3 && g__ + 3 < 2 * NT) {                                \
+      /* the ring entry just retired takes fragment g + 3 */                     \
+      read_a(cur, (g__ + 3) / NT, (g__ + 3) % NT, g__ % 3);                      \
     }                                                                            \
-    /* unconditional: past the end the last tile is fetched again and never     \
-       stored, which keeps the loaded registers free of a select */             \
-    const int tl__ = ts__ + 1 < nk ? ts__ + 1 : nk - 1;                          \
-    QMM_LOAD_TILE(tl__ * kBK);                                                   \
-  } while (0)
+    if constexpr (s__ == 0 && t__ >= NT - 4 && b__ == 1) {                       \
+      read_b(cur, 1, t__ - (NT - 4));                                            \
+    }                                                                            \
+    if constexpr (PREP) {                                                        \
+      if constexpr ((m) == 0) {                                                  \
+        QMM_LOAD_W(k2);                                                          \
+      }                                                                          \
+      if constexpr (pair_at((m), kNS) >= 0) {                                    \
+        dqv[pair_at((m), kNS)] = dq.template pair<pair_at((m), kNS)>(wreg, sf, bf); \
+      }                                                                          \
+      if constexpr (wstore_at((m), kNS) >= 0) {                                  \
+        constexpr int r__ = wstore_at((m), kNS);                                 \
+        wdst[r__] = make_uint4(                                                  \
+            dqv[4 * r__], dqv[4 * r__ + 1], dqv[4 * r__ + 2], dqv[4 * r__ + 3]); \
+      }                                                                          \
+      if constexpr ((m) == 1) {                                                  \
+        *reinterpret_cast<uint4*>(&xs[(xr + 0) * kLdsStride + xc * 8]) = xq0;    \
+        xq0 = *reinterpret_cast<const uint4*>(p.x + xoff0 + k2);                 \
+      }                                                                          \
+      if constexpr ((m) == 5) {                                                  \
+        *reinterpret_cast<uint4*>(&xs[(xr + 64) * kLdsStride + xc * 8]) = xq1;   \
+        xq1 = *reinterpret_cast<const uint4*>(p.x + xoff1 + k2);                 \
+      }                                                                          \
+      if constexpr ((m) == 9) {                                                  \
+        *reinterpret_cast<uint4*>(&xs[(xr + 128) * kLdsStride + xc * 8]) = xq2;  \
+        xq2 = *reinterpret_cast<const uint4*>(p.x + xoff2 + k2);                 \
+      }                                                                          \
+      if constexpr ((m) == 13) {                                                 \
+        *reinterpret_cast<uint4*>(&xs[(xr + 192) * kLdsStride + xc * 8]) = xq3;  \
+        xq3 = *reinterpret_cast<const uint4*>(p.x + xoff3 + k2);                 \
+      }                                                                          \
+    }                                                                            \
+    __builtin_amdgcn_sched_barrier(0);                                           \
+  }
 
-  if (wm == 1) {
-    QMM_MEM_PHASE(1);
-    __syncthreads();
-  }
-  for (int t = 0; t < nk; ++t) {
-    __builtin_amdgcn_s_setprio(1);
-    mfma_tile(t & 1);
-    __builtin_amdgcn_s_setprio(0);
-    __syncthreads();
-    QMM_MEM_PHASE(t + 1 + wm);
-    __syncthreads();
-  }
-  if (wm == 0) {
-    __syncthreads();
-  }
-#undef QMM_MEM_PHASE
+#define QMM_SLOTS8(m0, PREP)                                                     \
+  QMM_SLOT((m0) + 0, PREP) QMM_SLOT((m0) + 1, PREP) QMM_SLOT((m0) + 2, PREP)     \
+  QMM_SLOT((m0) + 3, PREP) QMM_SLOT((m0) + 4, PREP) QMM_SLOT((m0) + 5, PREP)     \
+  QMM_SLOT((m0) + 6, PREP) QMM_SLOT((m0) + 7, PREP)
 
-  // ---- epilogue: D[n][m] tiles; register r of lane (col, half) holds
-  // n = 8 (r / 4) + 4 half + r % 4, m = col.  Four consecutive n -> one 8-byte
-  // store of y[m][n .. n+3].
-  const int col = lane & 31;
-  const int half = lane >> 5;
+#define QMM_STEP(PREP)                                                           \
+  read_b(cur, 0, 0);                                                             \
+  read_a(cur, 0, 0, 0);                                                          \
+  read_b(cur, 0, 1);                                                             \
+  read_b(cur, 0, 2);                                                             \
+  read_b(cur, 0, 3);                                                             \
+  read_a(cur, 0, 1, 1);                                                          \
+  read_a(cur, 0, 2, 2);                                                          \
+  __builtin_amdgcn_sched_barrier(0);                                             \
+  QMM_SLOTS8(0, PREP) QMM_SLOTS8(8, PREP) QMM_SLOTS8(16, PREP) QMM_SLOTS8(24, PREP) \
+  QMM_SLOTS8(32, PREP) QMM_SLOTS8(40, PREP) QMM_SLOTS8(48, PREP) QMM_SLOTS8(56, PREP)
+
+  for (int t = 0; t + 1 < nk; ++t) {
+    const int cur = t & 1;
+    const int k2 = (t + 2) * kBK < klast ? (t + 2) * kBK : klast;
+    T* xs = lds + (cur ^ 1) * kStage;
+    uint4* wdst = reinterpret_cast<uint4*>(&xs[kXTile + wr * kLdsStride + wh * 32]);
+    const float sf = to_f32(sreg);
+    const float bf = to_f32(breg);
+    PairDequant<T, BITS> dq;
+    uint32_t dqv[16];
+    QMM_STEP(1)
+    QMM_ROTATE_W();
+    __syncthreads();
+  }
+  {
+    // last tile: nothing left to prepare; the names below only satisfy the
+    // discarded branches of the slot macro
+    const int cur = (nk - 1) & 1;
+    constexpr int k2 = 0;
+    T* xs = nullptr;
+    uint4* wdst = nullptr;
+    constexpr float sf = 0.0f;
+    constexpr float bf = 0.0f;
+    PairDequant<T, BITS> dq;
+    uint32_t dqv[16];
+    (void)k2;
+    (void)xs;
+    (void)wdst;
+    (void)sf;
+    (void)bf;
+    (void)dq;
+    (void)dqv;
+    QMM_STEP(0)
+  }
+#undef QMM_STEP
+#undef QMM_SLOTS8
+#undef QMM_SLOT
+
+  // ---- epilogue.  D[n][m] tiles: register r of lane (col, quad) holds
+  // n = 4 quad + r, m = col.  The tile is rounded to T and staged in LDS as
+  // ys[m][n] (the K loop is done with it), then written out row by row in
+  // 16-byte pieces, 32 NT * 2 contiguous bytes per row.
+  __syncthreads();
+  constexpr int kOutStride = kBN + kOutPad;
+  T* ys = lds;
+  {
+    const int col = lane & 15;
+    const int quad = lane >> 4;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int m = m0 + wm * 128 + j * 32 + col;
-    if (m >= M) {
-      continue;
-    }
-    T* yrow = p.out + static_cast<size_t>(m) * N;
+    for (int j = 0; j < 4; ++j) {
+      T* yrow = ys + (wm * 64 + j * 16 + col) * kOutStride + wn * 16 * NT + 4 * quad;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * 64 + i * 32 + 8 * q + 4 * half;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] = p.valid ? acc[i][j][4 * q + e] : 0.0f;
+      for (int i = 0; i < NT; ++i) {
+        uint2 packed;
+        packed.x = pack2<T>(acc[i][j][0], acc[i][j][1]);
+        packed.y = pack2<T>(acc[i][j][2], acc[i][j][3]);
+        if (!p.valid) {
+          packed = make_uint2(0u, 0u);
         }
-        if (n + 3 < N && (N % 4) == 0) {
-          uint2 packed;
-          packed.x = pack2<T>(v[0], v[1]);
-          packed.y = pack2<T>(v[2], v[3]);
-          *reinterpret_cast<uint2*>(yrow + n) = packed;
+        *reinterpret_cast<uint2*>(yrow + 16 * i) = packed;
+      }
+    }
+  }
+  __syncthreads();
+  {
+    constexpr int kChunks = kBN / 8;             // 16-byte pieces per tile row
+    constexpr int kRowsPerPass = kThreads / 32;  // 32 lanes cover up to 256 columns
+    const int c = tid & 31;
+    const int r0 = tid >> 5;
+    const bool vec_ok = (N % 8) == 0; // rows of y stay 16-byte aligned
+    if (c < kChunks) {
+#pragma unroll 4
+      for (int r = r0; r < kBM; r += kRowsPerPass) {
+        const int m = m0 + r;
+        const int n = n0 + c * 8;
+        if (m >= M || n >= N) {
+          continue;
+        }
+        const T* src = ys + r * kOutStride + c * 8;
+        T* dst = p.out + static_cast<size_t>(m) * N + n;
+        if (vec_ok && n + 8 <= N) {
+          *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
         } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (n + e < N) {
-              yrow[n + e] = from_f32<T>(v[e]);
-            }
+          for (int e = 0; e < 8 && n + e < N; ++e) {
+            dst[e] = src[e];
           }
         }
       }
@@ -333,11 +484,70 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a) {
   }
 }
 
-#undef QMM_LOAD_TILE
-#undef QMM_STORE_TILE
+#undef QMM_LOAD_X
+#undef QMM_LOAD_W
+#undef QMM_ROTATE_W
+#undef QMM_STORE_X
+#undef QMM_STORE_W
 
-constexpr size_t kQmmSmemBytes =
-    static_cast<size_t>(2) * (kBM + kBN) * kLdsStride * 2; // two stages, 16-bit
+template <int NT>
+constexpr size_t qmm_smem_bytes() {
+  constexpr size_t stages = static_cast<size_t>(2) * (kBM + 32 * NT) * kLdsStride * 2;
+  constexpr size_t out = static_cast<size_t>(kBM) * (32 * NT + kOutPad) * 2;
+  return stages > out ? stages : out;
+}
+
+int compute_units() {
+  static int cus = [] {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+      return 256;
+    }
+    return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }();
+  return cus;
+}
+
+// Tile width (in units of 32 columns) that finishes first: a workgroup needs
+// time ~ NT per tile and the tiles run in ceil(tiles / CUs) rounds.
+int choose_nt(int M, int N, int L) {
+  const long cus = compute_units();
+  const long mt = (M + kBM - 1) / kBM;
+  int best = 8;
+  long best_cost = -1;
+  for (int nt = 8; nt >= 6; --nt) {
+    const long tiles = mt * ((N + 32 * nt - 1) / (32 * nt)) * L;
+    const long rounds = (tiles + cus - 1) / cus;
+    const long cost = rounds * (nt * 8 + 3); // + fixed per-tile prologue/epilogue
+    if (best_cost < 0 || cost < best_cost) {
+      best = nt;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+template <typename T, int BITS, int NT>
+int launch_variant(const QmmArgs& a, int gs_shift, hipStream_t s) {
+  constexpr size_t smem = qmm_smem_bytes<NT>();
+  const dim3 grid((a.N + 32 * NT - 1) / (32 * NT), (a.M + kBM - 1) / kBM, a.L);
+  if (grid.y > 65535u || grid.z > 65535u) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
+  }
+  auto kern = qmm_t_mfma_kernel<T, BITS, NT>;
+  static bool configured = false; // per instantiation
+  if (!configured) {
+    MLXROCM_HIP_TRY(hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern),
+        hipFuncAttributeMaxDynamicSharedMemorySize,
+        static_cast<int>(smem)));
+    configured = true;
+  }
+  kern<<<grid, kThreads, smem, s>>>(a, gs_shift);
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return static_cast<int>(MLXROCM_OK);
+}
 
 } // namespace
 
@@ -351,29 +561,20 @@ bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool tran
 }
 
 int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
-  const dim3 grid((a.N + kBN - 1) / kBN, (a.M + kBM - 1) / kBM, a.L);
-  if (grid.y > 65535u || grid.z > 65535u) {
-    return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
-  }
+  const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
+  const int nt = choose_nt(a.M, a.N, a.L);
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
-      return dispatch_group(gs, [&](auto gval) {
-        constexpr int B = decltype(bval)::value;
-        constexpr int G = decltype(gval)::value;
-        auto kern = qmm_t_mfma_kernel<T, B, G>;
-        static bool configured = false; // per instantiation
-        if (!configured) {
-          MLXROCM_HIP_TRY(hipFuncSetAttribute(
-              reinterpret_cast<const void*>(kern),
-              hipFuncAttributeMaxDynamicSharedMemorySize,
-              static_cast<int>(kQmmSmemBytes)));
-          configured = true;
-        }
-        kern<<<grid, kThreads, kQmmSmemBytes, s>>>(a);
-        MLXROCM_HIP_TRY(hipGetLastError());
-        return static_cast<int>(MLXROCM_OK);
-      });
+      constexpr int B = decltype(bval)::value;
+      switch (nt) {
+        case 6:
+          return launch_variant<T, B, 6>(a, gs_shift, s);
+        case 7:
+          return launch_variant<T, B, 7>(a, gs_shift, s);
+        default:
+          return launch_variant<T, B, 8>(a, gs_shift, s);
+      }
     });
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
