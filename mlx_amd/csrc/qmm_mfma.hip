@@ -4,7 +4,7 @@
 //   y[M, N] = x[M, K] * dequant(W)[N, K]^T
 //
 // A workgroup of 512 threads (8 wavefronts: 4 along M x 2 along N) owns a
-// 256 (M) x BN (N) tile of y, BN = 32 NT with NT in {6, 7, 8} chosen on the host
+// 256 (M) x BN (N) tile of y, BN = 32 NT with NT in {5, 6, 7} chosen on the host
 // so that the tile count fills the compute units evenly, and walks K in steps
 // of 64 through two LDS stages.  Per step:
 //   * the x tile (256 x 64) and the packed W tile (BN rows x 64 codes) of the
@@ -140,11 +140,13 @@ __device__ __forceinline__ void dequant32(
 }
 
 // ---- placement of the side work in the MFMA slots of one K-step -------------
-// NS = 8 NT slots.  Dequantization pair q (0..15) goes to slot q NS / 16, the
-// 16-byte store of pairs 4r..4r+3 to the slot after pair 4r+3, the x store +
-// refetch of row block i to slot 4i + 1 and the packed-W fetch to slot 0.
+// NS = 8 NT slots.  Everything that writes LDS has to be issued before the
+// barrier in slot NS - 14, so the 16 dequantization pairs are spread over the
+// first NS - 16 slots: pair q goes to slot q (NS - 16) / 16, the 16-byte store
+// of pairs 4r..4r+3 to the slot after pair 4r+3, the x store + refetch of row
+// block i to slot 4i + 1 and the packed-W fetch to slot 0.
 constexpr int pair_slot(int q, int ns) {
-  return q * ns / 16;
+  return q * (ns - 16) / 16;
 }
 constexpr int pair_at(int m, int ns) {
   for (int q = 0; q < 16; ++q) {
@@ -193,8 +195,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   // x: thread covers 16-byte chunk (tid % 8) of rows tid/8 + 64 i, i < 4.
   const int xc = tid & 7;
   const int xr = tid >> 3;
-  // W: thread (wr, wh) covers codes [32 wh, 32 wh + 32) of tile row wr; rows
-  // past the tile (NT < 8) are clamped and land in LDS padding that is unused.
+  // W: thread (wr, wh) covers codes [32 wh, 32 wh + 32) of tile row wr; the
+  // threads past the tile's rows repeat its last row (same values, same place).
   const int wr = (tid >> 1) < kBN ? (tid >> 1) : kBN - 1;
   const int wh = tid & 1;
   const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
@@ -218,16 +220,22 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 
   // registers of the tiles in flight: x and the packed W of the next K-step,
   // and the packed W of the step after that (wnext), fetched a whole step ahead
-  uint4 xq0, xq1, xq2, xq3;
+  // (x: two sets used by alternate steps, each fetched two steps ahead)
+  constexpr int kXSets = 2;
+  uint4 xa0, xa1, xa2, xa3; // set 0
+  uint4 xb0, xb1, xb2, xb3; // set 1
+// named registers, not an array: an array indexed through macros ends up in
+// scratch memory
+#define QMM_XQ(set, i) (*((kXSets == 2 && (set) == 1) ? &xb##i : &xa##i))
   uint32_t wreg[BITS], wnext[BITS];
   T sreg, breg, snext, bnext; // converted when used, so the loads are not waited for early
 
-#define QMM_LOAD_X(k0)                                                           \
+#define QMM_LOAD_X(set, k0)                                                      \
   do {                                                                           \
-    xq0 = *reinterpret_cast<const uint4*>(p.x + xoff0 + (k0));                   \
-    xq1 = *reinterpret_cast<const uint4*>(p.x + xoff1 + (k0));                   \
-    xq2 = *reinterpret_cast<const uint4*>(p.x + xoff2 + (k0));                   \
-    xq3 = *reinterpret_cast<const uint4*>(p.x + xoff3 + (k0));                   \
+    QMM_XQ(set, 0) = *reinterpret_cast<const uint4*>(p.x + xoff0 + (k0));        \
+    QMM_XQ(set, 1) = *reinterpret_cast<const uint4*>(p.x + xoff1 + (k0));        \
+    QMM_XQ(set, 2) = *reinterpret_cast<const uint4*>(p.x + xoff2 + (k0));        \
+    QMM_XQ(set, 3) = *reinterpret_cast<const uint4*>(p.x + xoff3 + (k0));        \
   } while (0)
 
 #define QMM_LOAD_W(k0)                                                           \
@@ -250,13 +258,13 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
     breg = bnext;                                                                \
   } while (0)
 
-#define QMM_STORE_X(stage)                                                       \
+#define QMM_STORE_X(set, stage)                                                  \
   do {                                                                           \
     T* xs__ = lds + (stage) * kStage;                                            \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 0) * kLdsStride + xc * 8]) = xq0;      \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 64) * kLdsStride + xc * 8]) = xq1;     \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 128) * kLdsStride + xc * 8]) = xq2;    \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 192) * kLdsStride + xc * 8]) = xq3;    \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 0) * kLdsStride + xc * 8]) = QMM_XQ(set, 0);   \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 64) * kLdsStride + xc * 8]) = QMM_XQ(set, 1);  \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 128) * kLdsStride + xc * 8]) = QMM_XQ(set, 2); \
+    *reinterpret_cast<uint4*>(&xs__[(xr + 192) * kLdsStride + xc * 8]) = QMM_XQ(set, 3); \
   } while (0)
 
 #define QMM_STORE_W(stage)                                                       \
@@ -291,9 +299,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 
   // MFMA operand fragments.  All four x fragments of a 32-wide k slice stay in
   // registers (two sets, one per slice); the W fragments stream through a ring
-  // of three, each read two groups of four MFMAs before its first use.
+  // of four, each read three groups of four MFMAs before its first use.  W
+  // fragment number g of a step is (slice g / NT, tile g % NT); numbers 2 NT..
+  // are the first fragments of the next step.
   uint4 bfr[2][4];
-  uint4 afr[3];
+  uint4 afr[4];
   auto read_b = [&](int stage, int s, int b) {
     bfr[s][b] = *reinterpret_cast<const uint4*>(
         lds + stage * kStage + xfrag_off + b * 16 * kLdsStride + s * 32);
@@ -305,126 +315,130 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 
   // ---- software pipeline, one barrier per K-step.  Step t issues 8 NT MFMAs
   // on tile t (LDS stage t%2); the slots between them carry, in a fixed order,
-  //   * the fragment reads that the MFMAs two groups later need,
+  //   * the fragment reads that the MFMAs three groups later need,
   //   * the dequantization of this thread's 32 codes of W tile t+1 (two codes
   //     per slot) and its four 16-byte stores to the idle stage,
-  //   * the stores of x tile t+1 (fetched during step t-1), each followed by
-  //     the fetch of the same rows of x tile t+2,
-  //   * the fetch of the packed W of tile t+2 (one step ahead of its use).
-  // Fetches past the last step are clamped to the last tile (never stored), so
-  // the loop body has no branch.
+  //   * the stores of x tile t+1, each followed by the fetch of the same rows
+  //     of a later x tile into the registers just freed,
+  //   * the fetch of the packed W of tile t+2 (one step ahead of its use),
+  //   * in slot NS - 14 the barrier: by then this wavefront has issued all its
+  //     LDS writes of tile t+1 and all its reads of tile t.  The remaining slots
+  //     already read the first fragments of tile t+1, so the next step starts
+  //     without waiting for LDS.
+  // Every step is the same code, the last one included: its fetches are clamped
+  // to the last tile and what it stores is never read.
   const int nk = K / kBK;
   const int klast = (nk - 1) * kBK;
-  QMM_LOAD_X(0);
+  auto kclamp = [&](int t) { return t * kBK < klast ? t * kBK : klast; };
+  QMM_LOAD_X(0, 0);
   QMM_LOAD_W(0);
   QMM_ROTATE_W();
-  QMM_STORE_X(0);
+  QMM_STORE_X(0, 0);
   QMM_STORE_W(0);
-  {
-    const int k1 = nk > 1 ? kBK : 0;
-    QMM_LOAD_X(k1);
-    QMM_LOAD_W(k1);
-    QMM_ROTATE_W();
+  QMM_LOAD_X(0, kclamp(1));
+  if constexpr (kXSets == 2) {
+    QMM_LOAD_X(1, kclamp(2));
   }
+  QMM_LOAD_W(kclamp(1));
+  QMM_ROTATE_W();
   __syncthreads();
+  read_b(0, 0, 0);
+  read_a(0, 0, 0, 0);
+  read_b(0, 0, 1);
+  read_b(0, 0, 2);
+  read_b(0, 0, 3);
+  read_a(0, 0, 1, 1);
+  read_a(0, 0, 2, 2);
+  read_a(0, 0, 3, 3);
 
-  // One slot: MFMA number m of the step and the side work assigned to it.
-  // PREP = 1 in the main loop, 0 in the last step (nothing left to prepare).
-#define QMM_SLOT(m, PREP)                                                        \
+  // One slot: MFMA number m of a step of parity P and the side work assigned
+  // to it.  `t` is the step, cur/nxt its LDS stages.
+#define QMM_SLOT(m, P)                                                           \
   if constexpr ((m) < kNS) {                                                     \
     constexpr int s__ = (m) / (4 * NT);                                          \
     constexpr int t__ = ((m) % (4 * NT)) / 4;                                    \
     constexpr int b__ = (m) % 4;                                                 \
-    constexpr int g__ = s__ * NT + t__; /* running W-fragment number */          \
-    acc[t__][b__] = mfma16<T>(afr[g__ % 3], bfr[s__][b__], acc[t__][b__]);       \
-    if constexpr (b__ == 3 && g__ + 3 < 2 * NT) {                                \
-      /* the ring entry just retired takes fragment g + 3 */                     \
-      read_a(cur, (g__ + 3) / NT, (g__ + 3) % NT, g__ % 3);                      \
+    constexpr int g__ = s__ * NT + t__;              /* W fragment number */     \
+    constexpr int e__ = ((P) * 2 * NT + g__) % 4;    /* its ring entry */        \
+    acc[t__][b__] = mfma16<T>(afr[e__], bfr[s__][b__], acc[t__][b__]);           \
+    if constexpr (b__ == 3) {                                                    \
+      /* the ring entry just retired takes fragment g + 4 */                     \
+      if constexpr (g__ + 4 < 2 * NT) {                                          \
+        read_a(cur, (g__ + 4) / NT, (g__ + 4) % NT, e__);                        \
+      } else {                                                                   \
+        read_a(nxt, 0, g__ + 4 - 2 * NT, e__);                                   \
+      }                                                                          \
     }                                                                            \
     if constexpr (s__ == 0 && t__ >= NT - 4 && b__ == 1) {                       \
       read_b(cur, 1, t__ - (NT - 4));                                            \
     }                                                                            \
-    if constexpr (PREP) {                                                        \
-      if constexpr ((m) == 0) {                                                  \
-        QMM_LOAD_W(k2);                                                          \
-      }                                                                          \
-      if constexpr (pair_at((m), kNS) >= 0) {                                    \
-        dqv[pair_at((m), kNS)] = dq.template pair<pair_at((m), kNS)>(wreg, sf, bf); \
-      }                                                                          \
-      if constexpr (wstore_at((m), kNS) >= 0) {                                  \
-        constexpr int r__ = wstore_at((m), kNS);                                 \
-        wdst[r__] = make_uint4(                                                  \
-            dqv[4 * r__], dqv[4 * r__ + 1], dqv[4 * r__ + 2], dqv[4 * r__ + 3]); \
-      }                                                                          \
-      if constexpr ((m) == 1) {                                                  \
-        *reinterpret_cast<uint4*>(&xs[(xr + 0) * kLdsStride + xc * 8]) = xq0;    \
-        xq0 = *reinterpret_cast<const uint4*>(p.x + xoff0 + k2);                 \
-      }                                                                          \
-      if constexpr ((m) == 5) {                                                  \
-        *reinterpret_cast<uint4*>(&xs[(xr + 64) * kLdsStride + xc * 8]) = xq1;   \
-        xq1 = *reinterpret_cast<const uint4*>(p.x + xoff1 + k2);                 \
-      }                                                                          \
-      if constexpr ((m) == 9) {                                                  \
-        *reinterpret_cast<uint4*>(&xs[(xr + 128) * kLdsStride + xc * 8]) = xq2;  \
-        xq2 = *reinterpret_cast<const uint4*>(p.x + xoff2 + k2);                 \
-      }                                                                          \
-      if constexpr ((m) == 13) {                                                 \
-        *reinterpret_cast<uint4*>(&xs[(xr + 192) * kLdsStride + xc * 8]) = xq3;  \
-        xq3 = *reinterpret_cast<const uint4*>(p.x + xoff3 + k2);                 \
-      }                                                                          \
+    if constexpr ((m) == kNS - 12 || (m) == kNS - 11 || (m) == kNS - 10 ||       \
+                  (m) == kNS - 8) {                                              \
+      read_b(nxt, 0, (m) == kNS - 8 ? 3 : (m) - (kNS - 12));                     \
+    }                                                                            \
+    if constexpr ((m) == 0) {                                                    \
+      QMM_LOAD_W(k2);                                                            \
+    }                                                                            \
+    if constexpr (pair_at((m), kNS) >= 0) {                                      \
+      dqv[pair_at((m), kNS)] = dq.template pair<pair_at((m), kNS)>(wreg, sf, bf); \
+    }                                                                            \
+    if constexpr (wstore_at((m), kNS) >= 0) {                                    \
+      constexpr int r__ = wstore_at((m), kNS);                                   \
+      wdst[r__] = make_uint4(                                                    \
+          dqv[4 * r__], dqv[4 * r__ + 1], dqv[4 * r__ + 2], dqv[4 * r__ + 3]);   \
+    }                                                                            \
+    if constexpr ((m) == 1) {                                                    \
+      *reinterpret_cast<uint4*>(&xs[(xr + 0) * kLdsStride + xc * 8]) = QMM_XQ(P, 0);   \
+      QMM_XQ(P, 0) = *reinterpret_cast<const uint4*>(p.x + xoff0 + kx);          \
+    }                                                                            \
+    if constexpr ((m) == 5) {                                                    \
+      *reinterpret_cast<uint4*>(&xs[(xr + 64) * kLdsStride + xc * 8]) = QMM_XQ(P, 1);  \
+      QMM_XQ(P, 1) = *reinterpret_cast<const uint4*>(p.x + xoff1 + kx);          \
+    }                                                                            \
+    if constexpr ((m) == 9) {                                                    \
+      *reinterpret_cast<uint4*>(&xs[(xr + 128) * kLdsStride + xc * 8]) = QMM_XQ(P, 2); \
+      QMM_XQ(P, 2) = *reinterpret_cast<const uint4*>(p.x + xoff2 + kx);          \
+    }                                                                            \
+    if constexpr ((m) == 13) {                                                   \
+      *reinterpret_cast<uint4*>(&xs[(xr + 192) * kLdsStride + xc * 8]) = QMM_XQ(P, 3); \
+      QMM_XQ(P, 3) = *reinterpret_cast<const uint4*>(p.x + xoff3 + kx);          \
+    }                                                                            \
+    if constexpr ((m) == kNS - 14) {                                             \
+      __syncthreads();                                                           \
     }                                                                            \
     __builtin_amdgcn_sched_barrier(0);                                           \
   }
 
-#define QMM_SLOTS8(m0, PREP)                                                     \
-  QMM_SLOT((m0) + 0, PREP) QMM_SLOT((m0) + 1, PREP) QMM_SLOT((m0) + 2, PREP)     \
-  QMM_SLOT((m0) + 3, PREP) QMM_SLOT((m0) + 4, PREP) QMM_SLOT((m0) + 5, PREP)     \
-  QMM_SLOT((m0) + 6, PREP) QMM_SLOT((m0) + 7, PREP)
+#define QMM_SLOTS8(m0, P)                                                        \
+  QMM_SLOT((m0) + 0, P) QMM_SLOT((m0) + 1, P) QMM_SLOT((m0) + 2, P)              \
+  QMM_SLOT((m0) + 3, P) QMM_SLOT((m0) + 4, P) QMM_SLOT((m0) + 5, P)              \
+  QMM_SLOT((m0) + 6, P) QMM_SLOT((m0) + 7, P)
 
-#define QMM_STEP(PREP)                                                           \
-  read_b(cur, 0, 0);                                                             \
-  read_a(cur, 0, 0, 0);                                                          \
-  read_b(cur, 0, 1);                                                             \
-  read_b(cur, 0, 2);                                                             \
-  read_b(cur, 0, 3);                                                             \
-  read_a(cur, 0, 1, 1);                                                          \
-  read_a(cur, 0, 2, 2);                                                          \
-  __builtin_amdgcn_sched_barrier(0);                                             \
-  QMM_SLOTS8(0, PREP) QMM_SLOTS8(8, PREP) QMM_SLOTS8(16, PREP) QMM_SLOTS8(24, PREP) \
-  QMM_SLOTS8(32, PREP) QMM_SLOTS8(40, PREP) QMM_SLOTS8(48, PREP) QMM_SLOTS8(56, PREP)
-
-  for (int t = 0; t + 1 < nk; ++t) {
-    const int cur = t & 1;
-    const int k2 = (t + 2) * kBK < klast ? (t + 2) * kBK : klast;
-    T* xs = lds + (cur ^ 1) * kStage;
-    uint4* wdst = reinterpret_cast<uint4*>(&xs[kXTile + wr * kLdsStride + wh * 32]);
-    const float sf = to_f32(sreg);
-    const float bf = to_f32(breg);
-    PairDequant<T, BITS> dq;
-    uint32_t dqv[16];
-    QMM_STEP(1)
-    QMM_ROTATE_W();
-    __syncthreads();
+#define QMM_STEP(tt, P)                                                          \
+  {                                                                              \
+    const int cur = (P);                                                         \
+    const int nxt = (P) ^ 1;                                                     \
+    const int k2 = kclamp((tt) + 2);                                             \
+    const int kx = kclamp((tt) + 1 + kXSets);                                    \
+    T* xs = lds + nxt * kStage;                                                  \
+    uint4* wdst = reinterpret_cast<uint4*>(&xs[kXTile + wr * kLdsStride + wh * 32]); \
+    const float sf = to_f32(sreg);                                               \
+    const float bf = to_f32(breg);                                               \
+    PairDequant<T, BITS> dq;                                                     \
+    uint32_t dqv[16];                                                            \
+    __builtin_amdgcn_sched_barrier(0);                                           \
+    QMM_SLOTS8(0, P) QMM_SLOTS8(8, P) QMM_SLOTS8(16, P) QMM_SLOTS8(24, P)        \
+    QMM_SLOTS8(32, P) QMM_SLOTS8(40, P) QMM_SLOTS8(48, P) QMM_SLOTS8(56, P)      \
+    QMM_ROTATE_W();                                                              \
   }
-  {
-    // last tile: nothing left to prepare; the names below only satisfy the
-    // discarded branches of the slot macro
-    const int cur = (nk - 1) & 1;
-    constexpr int k2 = 0;
-    T* xs = nullptr;
-    uint4* wdst = nullptr;
-    constexpr float sf = 0.0f;
-    constexpr float bf = 0.0f;
-    PairDequant<T, BITS> dq;
-    uint32_t dqv[16];
-    (void)k2;
-    (void)xs;
-    (void)wdst;
-    (void)sf;
-    (void)bf;
-    (void)dq;
-    (void)dqv;
-    QMM_STEP(0)
+
+  int t = 0;
+  for (; t + 1 < nk; t += 2) {
+    QMM_STEP(t, 0)
+    QMM_STEP(t + 1, 1)
+  }
+  if (t < nk) {
+    QMM_STEP(t, 0)
   }
 #undef QMM_STEP
 #undef QMM_SLOTS8
@@ -484,6 +498,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   }
 }
 
+#undef QMM_XQ
 #undef QMM_LOAD_X
 #undef QMM_LOAD_W
 #undef QMM_ROTATE_W
@@ -514,9 +529,9 @@ int compute_units() {
 int choose_nt(int M, int N, int L) {
   const long cus = compute_units();
   const long mt = (M + kBM - 1) / kBM;
-  int best = 8;
+  int best = 7;
   long best_cost = -1;
-  for (int nt = 8; nt >= 6; --nt) {
+  for (int nt = 7; nt >= 5; --nt) {
     const long tiles = mt * ((N + 32 * nt - 1) / (32 * nt)) * L;
     const long rounds = (tiles + cus - 1) / cus;
     const long cost = rounds * (nt * 8 + 3); // + fixed per-tile prologue/epilogue
@@ -568,12 +583,12 @@ int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
     return dispatch_bits(bits, [&](auto bval) {
       constexpr int B = decltype(bval)::value;
       switch (nt) {
+        case 5:
+          return launch_variant<T, B, 5>(a, gs_shift, s);
         case 6:
           return launch_variant<T, B, 6>(a, gs_shift, s);
-        case 7:
-          return launch_variant<T, B, 7>(a, gs_shift, s);
         default:
-          return launch_variant<T, B, 8>(a, gs_shift, s);
+          return launch_variant<T, B, 7>(a, gs_shift, s);
       }
     });
   };
