@@ -1,0 +1,175 @@
+// gather_group.hip -- groups the index pairs of a GatherQMM call by expert so
+// that the matrix-core GEMM reads every expert's weights once for all the rows
+// routed to it (the reference loops over the pairs one GEMV at a time,
+// mlx/backend/cpu/quantized.cpp:700-747; the Metal backend groups sorted runs,
+// mlx/backend/metal/quantized.cpp:1905-1923).
+//
+// Three small kernels fill a caller-provided workspace:
+//   count    one atomic per pair into counts[expert]; pairs with an index out of
+//            range are left out and their output rows are zero-filled here;
+//   plan     one workgroup: exclusive scan of the counts -> first sorted
+//            position of every expert, and the list of 256-row tiles
+//            {expert, first position, rows}; the tile count stays on the device;
+//   scatter  perm[position] = pair, position handed out by a per-expert cursor.
+// The order inside an expert's run is arbitrary; every output row depends on
+// its own x row only, so the result does not depend on it.
+#include "qmm_args.h"
+
+namespace mlxrocm {
+
+namespace {
+
+constexpr int kTileRows = 256;
+constexpr int kMaxExperts = 4096; // plan kernel keeps the counts in LDS
+
+template <typename T>
+__global__ __launch_bounds__(256) void group_count_kernel(
+    const uint32_t* lhs,
+    const uint32_t* rhs,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int32_t* counts,
+    T* out,
+    int N) {
+  const int l = blockIdx.x * blockDim.x + threadIdx.x;
+  if (l >= n_indices) {
+    return;
+  }
+  const uint32_t xi = lhs[l];
+  const uint32_t wi = rhs[l];
+  if (xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts)) {
+    atomicAdd(&counts[wi], 1);
+  } else {
+    T* row = out + static_cast<size_t>(l) * N;
+    for (int n = 0; n < N; ++n) {
+      row[n] = static_cast<T>(0.0f);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void group_plan_kernel(
+    int n_experts,
+    const int32_t* counts,
+    int32_t* offsets,
+    int32_t* tiles,
+    int32_t* n_tiles) {
+  __shared__ int32_t cnt[kMaxExperts];
+  __shared__ int32_t first_pos[kMaxExperts];
+  __shared__ int32_t first_tile[kMaxExperts];
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    cnt[e] = counts[e];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int pos = 0;
+    int tile = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      first_pos[e] = pos;
+      first_tile[e] = tile;
+      pos += cnt[e];
+      tile += (cnt[e] + kTileRows - 1) / kTileRows;
+    }
+    *n_tiles = tile;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    offsets[e] = first_pos[e];
+    const int c = cnt[e];
+    int t = first_tile[e];
+    for (int r = 0; r < c; r += kTileRows, ++t) {
+      tiles[3 * t + 0] = e;
+      tiles[3 * t + 1] = first_pos[e] + r;
+      tiles[3 * t + 2] = (c - r < kTileRows) ? c - r : kTileRows;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void group_scatter_kernel(
+    const uint32_t* lhs,
+    const uint32_t* rhs,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    const int32_t* offsets,
+    int32_t* cursor,
+    int32_t* perm) {
+  const int l = blockIdx.x * blockDim.x + threadIdx.x;
+  if (l >= n_indices) {
+    return;
+  }
+  const uint32_t xi = lhs[l];
+  const uint32_t wi = rhs[l];
+  if (xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts)) {
+    const int pos = offsets[wi] + atomicAdd(&cursor[wi], 1);
+    perm[pos] = l;
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* p, int n, int32_t v) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    p[i] = v;
+  }
+}
+
+size_t align_up(size_t v, size_t a) {
+  return (v + a - 1) / a * a;
+}
+
+} // namespace
+
+int gather_group_max_tiles(int n_indices, int n_experts) {
+  // every expert may end on a partial tile
+  return (n_indices + kTileRows - 1) / kTileRows + n_experts;
+}
+
+size_t gather_group_workspace_bytes(int n_indices, int n_experts) {
+  if (n_indices <= 0 || n_experts <= 0 || n_experts > kMaxExperts) {
+    return 0;
+  }
+  const size_t ints = static_cast<size_t>(3) * n_experts + 4 +
+      static_cast<size_t>(3) * gather_group_max_tiles(n_indices, n_experts) + n_indices;
+  return align_up(ints * sizeof(int32_t), 256);
+}
+
+// Fills the workspace and points the grouped-mode fields of `a` into it.
+int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s) {
+  const int E = a.n_experts;
+  const int n = a.L;
+  int32_t* ws = static_cast<int32_t*>(workspace);
+  int32_t* counts = ws;
+  int32_t* cursor = counts + E;
+  int32_t* offsets = cursor + E;
+  int32_t* n_tiles = offsets + E;
+  int32_t* tiles = n_tiles + 4;
+  int32_t* perm = tiles + 3 * gather_group_max_tiles(n, E);
+
+  // counts and cursors start at zero (a fill kernel, so that the sequence can be
+  // captured into a graph)
+  fill_i32_kernel<<<(2 * E + 255) / 256, 256, 0, s>>>(counts, 2 * E, 0);
+  MLXROCM_HIP_TRY(hipGetLastError());
+  const int blocks = (n + 255) / 256;
+  if (dtype == MLXROCM_BFLOAT16) {
+    group_count_kernel<bf16_t><<<blocks, 256, 0, s>>>(
+        a.lhs_indices, a.rhs_indices, n, a.x_batches, E, counts,
+        static_cast<bf16_t*>(a.out), a.N);
+  } else {
+    group_count_kernel<f16_t><<<blocks, 256, 0, s>>>(
+        a.lhs_indices, a.rhs_indices, n, a.x_batches, E, counts,
+        static_cast<f16_t*>(a.out), a.N);
+  }
+  MLXROCM_HIP_TRY(hipGetLastError());
+  group_plan_kernel<<<1, 256, 0, s>>>(E, counts, offsets, tiles, n_tiles);
+  MLXROCM_HIP_TRY(hipGetLastError());
+  group_scatter_kernel<<<blocks, 256, 0, s>>>(
+      a.lhs_indices, a.rhs_indices, n, a.x_batches, E, offsets, cursor, perm);
+  MLXROCM_HIP_TRY(hipGetLastError());
+
+  a.group_tiles = tiles;
+  a.group_perm = perm;
+  a.group_ntiles = n_tiles;
+  return MLXROCM_OK;
+}
+
+} // namespace mlxrocm

@@ -211,18 +211,50 @@ extern "C" int mlxrocm_qmm(
   return run(a, group_size, bits, dtype, transpose != 0, s);
 }
 
+// Grouping by expert pays when every expert's weights are shared by several
+// index pairs; it needs one row of x per pair, the matrix-core GEMM, 32-bit
+// element offsets into x and a workspace for the sorted order.
+bool group_gather(
+    int M,
+    int K,
+    int n_indices,
+    int n_experts,
+    int x_batches,
+    int64_t x_batch_stride,
+    int dtype,
+    bool transpose) {
+  if (M != 1 || !transpose || dtype == MLXROCM_FLOAT32 || K % 64 != 0 || K < 64) {
+    return false;
+  }
+  if (n_indices < 32 || static_cast<int64_t>(n_indices) < 4 * static_cast<int64_t>(n_experts)) {
+    return false;
+  }
+  if (static_cast<int64_t>(x_batches) * x_batch_stride + K >= (int64_t(1) << 32)) {
+    return false;
+  }
+  if (gather_group_max_tiles(n_indices, n_experts) > 65535) {
+    return false;
+  }
+  return gather_group_workspace_bytes(n_indices, n_experts) > 0;
+}
+
 extern "C" size_t mlxrocm_gather_qmm_workspace_size(
-    int /*M*/,
+    int M,
     int /*N*/,
-    int /*K*/,
-    int /*n_indices*/,
-    int /*n_experts*/,
+    int K,
+    int n_indices,
+    int n_experts,
     int /*group_size*/,
     int /*bits*/,
-    int /*dtype*/,
-    int /*transpose*/,
+    int dtype,
+    int transpose,
     int /*rhs_sorted*/) {
-  return 0;
+  // x_batches / stride are unknown here; mlxrocm_gather_qmm checks them and
+  // falls back to the ungrouped launch if they rule grouping out.
+  if (!group_gather(M, K, n_indices, n_experts, 1, 0, dtype, transpose != 0)) {
+    return 0;
+  }
+  return gather_group_workspace_bytes(n_indices, n_experts);
 }
 
 extern "C" int mlxrocm_gather_qmm(
@@ -247,8 +279,8 @@ extern "C" int mlxrocm_gather_qmm(
     int dtype,
     int transpose,
     int /*rhs_sorted*/,
-    void* /*workspace*/,
-    size_t /*workspace_bytes*/,
+    void* workspace,
+    size_t workspace_bytes,
     mlxrocm_stream_t stream) {
   int rc = check_shape(
       "gather_qmm", M, N, K, n_indices, group_size, bits, dtype, transpose);
@@ -292,6 +324,19 @@ extern "C" int mlxrocm_gather_qmm(
   rc = check_alignment("gather_qmm", a, dtype);
   if (rc != MLXROCM_OK) {
     return rc;
+  }
+  if (workspace != nullptr &&
+      group_gather(
+          M, K, n_indices, n_experts, x_batches, x_batch_stride, dtype, transpose != 0) &&
+      workspace_bytes >= gather_group_workspace_bytes(n_indices, n_experts)) {
+    if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) {
+      return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qmm] workspace must be 4-byte aligned");
+    }
+    rc = launch_gather_group(a, dtype, workspace, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    return launch_qmm_mfma_grouped(a, group_size, bits, dtype, s);
   }
   // One grid z-slot per index pair; large index lists go in slices.
   constexpr int kMaxZ = 65535;

@@ -25,6 +25,14 @@ struct QmmArgs {
   const uint32_t* rhs_indices;
   int x_batches; // bounds for gathered indices
   int n_experts;
+  // Grouped gather (M == 1): the index pairs sorted by expert and cut into tiles
+  // of up to 256 rows.  group_tiles holds {expert, first sorted position, rows}
+  // per tile, group_perm maps a sorted position to its index pair, group_ntiles
+  // points at the number of tiles (known on the device only).  All null
+  // otherwise.
+  const int32_t* group_tiles;
+  const int32_t* group_perm;
+  const int32_t* group_ntiles;
 };
 
 // Resolved operand pointers of problem l.  `valid` is false when a gathered
@@ -81,5 +89,12 @@ int launch_qmv_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
 bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 int launch_zero_fill(void* p, size_t bytes, hipStream_t s);
+
+// Grouping of gathered index pairs by expert (gather_group.hip) and the grouped
+// launch of the matrix-core GEMM over its tiles (qmm_mfma.hip).
+size_t gather_group_workspace_bytes(int n_indices, int n_experts);
+int gather_group_max_tiles(int n_indices, int n_experts);
+int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s);
+int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 
 } // namespace mlxrocm

@@ -165,7 +165,10 @@ constexpr int wstore_at(int m, int ns) {
   return -1;
 }
 
-template <typename T, int BITS, int NT>
+// GROUPED: blockIdx.y walks the tile list of a gather grouped by expert (M == 1
+// per index pair): the tile's rows are the x rows of up to 256 index pairs that
+// share one expert, fetched and written back through the permutation.
+template <typename T, int BITS, int NT, bool GROUPED>
 __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, const int gs_shift) {
   constexpr int kBN = 32 * NT;
   constexpr int kNS = 8 * NT; // MFMAs per wavefront per K-step
@@ -181,12 +184,31 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1;  // which 16 NT columns (n) of the tile
   const int wm = wave >> 1; // which 64 rows (m) of the tile
-  const int M = a.M;
   const int N = a.N;
   const int K = a.K;
   const int n0 = blockIdx.x * kBN;
-  const int m0 = blockIdx.y * kBM;
-  const QmmProblem<T> p = resolve_problem<T>(a, blockIdx.z);
+  int M = a.M;
+  int m0 = blockIdx.y * kBM;
+  int row0 = 0; // grouped: first sorted position of the tile
+  QmmProblem<T> p;
+  if constexpr (GROUPED) {
+    const int tile = blockIdx.y;
+    if (tile >= *a.group_ntiles) {
+      return; // the grid covers the worst-case tile count
+    }
+    const int e = a.group_tiles[3 * tile];
+    row0 = a.group_tiles[3 * tile + 1];
+    M = a.group_tiles[3 * tile + 2];
+    m0 = 0;
+    p.x = static_cast<const T*>(a.x);
+    p.w = reinterpret_cast<const uint8_t*>(a.w + static_cast<int64_t>(e) * a.w_batch_stride);
+    p.scales = static_cast<const T*>(a.scales) + static_cast<int64_t>(e) * a.sb_batch_stride;
+    p.biases = static_cast<const T*>(a.biases) + static_cast<int64_t>(e) * a.sb_batch_stride;
+    p.out = static_cast<T*>(a.out);
+    p.valid = true;
+  } else {
+    p = resolve_problem<T>(a, blockIdx.z);
+  }
 
   const int groups = K >> gs_shift;
   const int row_words = K / 32 * BITS;
@@ -210,7 +232,13 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   {
     auto row_off = [&](int i) {
       const int m = m0 + xr + 64 * i;
-      return static_cast<uint32_t>(m < M ? m : M - 1) * static_cast<uint32_t>(K) + xc * 8;
+      const int mc = m < M ? m : M - 1;
+      if constexpr (GROUPED) {
+        const uint32_t pair = static_cast<uint32_t>(a.group_perm[row0 + mc]);
+        return a.lhs_indices[pair] * static_cast<uint32_t>(a.x_batch_stride) + xc * 8;
+      } else {
+        return static_cast<uint32_t>(mc) * static_cast<uint32_t>(K) + xc * 8;
+      }
     };
     xoff0 = row_off(0);
     xoff1 = row_off(1);
@@ -485,7 +513,9 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
           continue;
         }
         const T* src = ys + r * kOutStride + c * 8;
-        T* dst = p.out + static_cast<size_t>(m) * N + n;
+        const size_t orow =
+            GROUPED ? static_cast<size_t>(a.group_perm[row0 + r]) : static_cast<size_t>(m);
+        T* dst = p.out + orow * N + n;
         if (vec_ok && n + 8 <= N) {
           *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
         } else {
@@ -543,14 +573,13 @@ int choose_nt(int M, int N, int L) {
   return best;
 }
 
-template <typename T, int BITS, int NT>
-int launch_variant(const QmmArgs& a, int gs_shift, hipStream_t s) {
+template <typename T, int BITS, int NT, bool GROUPED>
+int launch_variant(const QmmArgs& a, int gs_shift, dim3 grid, hipStream_t s) {
   constexpr size_t smem = qmm_smem_bytes<NT>();
-  const dim3 grid((a.N + 32 * NT - 1) / (32 * NT), (a.M + kBM - 1) / kBM, a.L);
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
-  auto kern = qmm_t_mfma_kernel<T, BITS, NT>;
+  auto kern = qmm_t_mfma_kernel<T, BITS, NT, GROUPED>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -562,6 +591,10 @@ int launch_variant(const QmmArgs& a, int gs_shift, hipStream_t s) {
   kern<<<grid, kThreads, smem, s>>>(a, gs_shift);
   MLXROCM_HIP_TRY(hipGetLastError());
   return static_cast<int>(MLXROCM_OK);
+}
+
+int shift_of(int gs) {
+  return gs == 32 ? 5 : (gs == 64 ? 6 : 7);
 }
 
 } // namespace
@@ -576,20 +609,38 @@ bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool tran
 }
 
 int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
-  const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
+  const int gs_shift = shift_of(gs);
   const int nt = choose_nt(a.M, a.N, a.L);
+  const dim3 grid((a.N + 32 * nt - 1) / (32 * nt), (a.M + kBM - 1) / kBM, a.L);
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
       constexpr int B = decltype(bval)::value;
       switch (nt) {
         case 5:
-          return launch_variant<T, B, 5>(a, gs_shift, s);
+          return launch_variant<T, B, 5, false>(a, gs_shift, grid, s);
         case 6:
-          return launch_variant<T, B, 6>(a, gs_shift, s);
+          return launch_variant<T, B, 6, false>(a, gs_shift, grid, s);
         default:
-          return launch_variant<T, B, 7>(a, gs_shift, s);
+          return launch_variant<T, B, 7, false>(a, gs_shift, grid, s);
       }
+    });
+  };
+  return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
+}
+
+// Gather grouped by expert: `a` carries the tile list; one grid row per
+// possible tile, rows past the device-side tile count exit at once.
+int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  constexpr int kNT = 7;
+  const int gs_shift = shift_of(gs);
+  const dim3 grid(
+      (a.N + 32 * kNT - 1) / (32 * kNT), gather_group_max_tiles(a.L, a.n_experts), 1);
+  auto run = [&](auto tval) -> int {
+    using T = decltype(tval);
+    return dispatch_bits(bits, [&](auto bval) {
+      constexpr int B = decltype(bval)::value;
+      return launch_variant<T, B, kNT, true>(a, gs_shift, grid, s);
     });
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});

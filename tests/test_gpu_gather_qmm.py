@@ -128,3 +128,66 @@ def test_gather_qmm_out_of_range_index_is_contained(gpu):
     out = mlx_amd.gather_qmm(x, wq, s, b, rhs_indices=idx)
     torch.cuda.synchronize()
     assert bool((out[1] == 0).all()) and bool(out[0].abs().sum() > 0)
+
+
+def _grouped_ws_bytes(M, N, K, n_idx, E, gs, bits, dtype_code=2):
+    from mlx_amd import _lib
+    return _lib.load().mlxrocm_gather_qmm_workspace_size(
+        M, N, K, n_idx, E, gs, bits, dtype_code, 1, 0)
+
+
+@pytest.mark.parametrize("bits,gs", ((4, 64), (8, 128), (3, 32), (6, 64)))
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_gather_qmm_grouped_by_expert(oracle, gpu, dtype, bits, gs):
+    """Many index pairs per expert take the grouped matrix-core path: a skewed
+    routing (one expert with more than one 256-row tile, one expert unused), x
+    rows reused by several pairs, N not a multiple of the tile."""
+    E, N, K, T = 5, 200, 256, 700
+    assert _grouped_ws_bytes(1, N, K, T, E, gs, bits) > 0  # the grouped path is taken
+    w = normal_weights((E, N, K), dtype, std=0.5)
+    wq, s, b = oracle.quantize(w, gs, bits)
+    X = 64
+    x = activations((X, 1, K), dtype)
+    g = torch.Generator().manual_seed(1)
+    rhs = torch.multinomial(torch.tensor([0.6, 0.0, 0.25, 0.1, 0.05]), T,
+                            replacement=True, generator=g)
+    lhs = torch.randint(0, X, (T,), generator=g)
+    assert int((rhs == 0).sum()) > 256 and int((rhs == 1).sum()) == 0
+    gx, gwq, gsc, gb, glhs, grhs = _to(gpu, x, wq, s, b, lhs, rhs)
+    got = mlx_amd.gather_qmm(gx, gwq, gsc, gb, glhs, grhs, True, gs, bits).cpu()
+    assert got.shape == (T, 1, N)
+    w_hat = exact_affine_weights(wq, s, b, gs, bits)
+    exact = torch.einsum("tk,tnk->tn", x.reshape(X, K).double()[lhs], w_hat[rhs])
+    err = float((got.reshape(T, N).double() - exact).abs().max())
+    assert err <= exact_tolerance(dtype, K, x, w_hat, exact)
+    # and against the oracle on a subsample of the pairs (the oracle is scalar)
+    sub = torch.arange(0, T, 23)
+    ref = oracle.gather_qmm(x, wq, s, b, lhs[sub], rhs[sub], True, gs, bits)
+    tol = matmul_tolerance(dtype, K, x, w_hat)
+    assert float((got[sub].double() - ref.double()).abs().max()) <= tol
+
+
+def test_gather_qmm_grouped_matches_ungrouped(gpu):
+    """The grouped launch and the one-GEMV-per-pair launch agree row for row up
+    to accumulation order (same fp32 accumulate, one rounding), also with a
+    sliced expert stack and an out-of-range expert index (zero row)."""
+    E, N, K, T = 6, 448, 512, 96
+    dtype = torch.bfloat16
+    w = normal_weights((E, N, K), dtype, std=0.5).to(gpu)
+    wq, s, b = mlx_amd.quantize(w, 64, 4)
+    x = activations((T, 1, K), dtype).to(gpu)
+    g = torch.Generator().manual_seed(2)
+    rhs = torch.randint(0, 3, (T,), generator=g).to(gpu)
+    rhs[5] = 3  # the sliced stack has three experts
+    grouped = mlx_amd.gather_qmm(x, wq[::2], s[::2], b[::2], rhs_indices=rhs)
+    # the same pairs one small call at a time: below the grouping threshold
+    parts = [
+        mlx_amd.gather_qmm(x[i:i + 8], wq[::2], s[::2], b[::2], rhs_indices=rhs[i:i + 8])
+        for i in range(0, T, 8)
+    ]
+    single = torch.cat(parts)
+    torch.cuda.synchronize()
+    assert bool((grouped[5] == 0).all())
+    diff = (grouped.float() - single.float()).abs().max()
+    scale = single.float().abs().max()
+    assert float(diff) <= 2 ** -7 * float(scale)
