@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the affine quantized-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only qmv|qmm_t]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only qmv|qmm_t] [--sweep]
 
 One "step" is one launch of the decode GEMV (qmv) of the Llama-3-8B gate/up
 projection: x bf16 [1, 4096] against W [14336, 4096] quantized to 4 bits,
@@ -125,6 +125,122 @@ def cpu_baseline(x_cpu, wq_cpu, s_cpu, b_cpu, nbytes: int) -> dict:
     }
 
 
+def sweep(torch, mlx_amd, dev) -> list:
+    """The other synthetic configurations of the path (prefill shapes, decode at
+    batch 4 and 8, 8-bit, odd code widths, fp32, expert-routed gather, quantize
+    and dequantize): one timing each, weights cycled through > 512 MB of copies
+    wherever one launch reads less than that, so that figures are HBM figures."""
+    rows = []
+    g = torch.Generator().manual_seed(0)
+
+    def timed(fn, min_ms=30.0):
+        for _ in range(2):
+            fn(0)
+        torch.cuda.synchronize()
+        reps, total = 4, 0.0
+        while True:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(reps):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            total = e0.elapsed_time(e1)
+            if total >= min_ms or reps >= 4096:
+                return total / reps
+            reps *= 4
+
+    def weights(n, k, dtype, std=0.02):
+        return (torch.randn((n, k), generator=g, dtype=torch.float32) * std).to(dtype).to(dev)
+
+    def ring_of(q, nbytes):
+        copies = max(1, min(24, int(600e6 // max(nbytes, 1)) + 1))
+        return [q] + [tuple(t.clone() for t in q) for _ in range(copies - 1)]
+
+    def add(cfg, name, ms, nbytes=None, flops=None, kernel=None):
+        row = {"config": cfg, "case": name, "us": round(ms * 1e3, 2)}
+        if nbytes is not None:
+            row["GB/s"] = round(nbytes / ms / 1e6, 1)
+        if flops is not None:
+            row["TFLOP/s"] = round(flops / ms / 1e9, 1)
+        if kernel:
+            row["kernel"] = kernel
+        rows.append(row)
+        print(json.dumps(row), file=sys.stderr, flush=True)
+
+    def kname(M, n, k, gs, bits, dtype):
+        from mlx_amd import _lib
+        code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+        return _lib.load().mlxrocm_qmm_kernel_name(M, n, k, 1, gs, bits, code, 1).decode()
+
+    def matmul_case(cfg, M, n, k, bits, gs, dtype):
+        esz = 4 if dtype == torch.float32 else 2
+        q = mlx_amd.quantize(weights(n, k, dtype), gs, bits)
+        wbytes = n * k * bits // 8 + 2 * n * (k // gs) * esz
+        ring = ring_of(q, wbytes) if M <= 64 else [q]
+        x = torch.randn((M, k), generator=g, dtype=torch.float32).to(dtype).to(dev)
+        fn = lambda i: mlx_amd.quantized_matmul(x, *ring[i % len(ring)], True, gs, bits)
+        ms = timed(fn)
+        name = f"x {str(dtype)[6:]} [{M},{k}] W [{n},{k}] b{bits} g{gs}"
+        if M <= 64:
+            add(cfg, name, ms, nbytes=qmv_bytes(M, n, k, bits, gs, esz),
+                kernel=kname(M, n, k, gs, bits, dtype))
+        else:
+            add(cfg, name, ms, flops=2.0 * M * n * k, kernel=kname(M, n, k, gs, bits, dtype))
+
+    bf16, f32 = torch.bfloat16, torch.float32
+    # Cfg1: fp32 4096 x 4096, 4-bit group 64
+    w = weights(4096, 4096, f32)
+    ms = timed(lambda i: mlx_amd.quantize(w, 64, 4))
+    qbytes = 4096 * 4096 * 4 + 4096 * 4096 // 2 + 2 * 4096 * 64 * 4
+    add("cfg1", "quantize f32 [4096,4096] b4 g64", ms, nbytes=qbytes)
+    q = mlx_amd.quantize(w, 64, 4)
+    ms = timed(lambda i: mlx_amd.dequantize(*q, 64, 4))
+    add("cfg1", "dequantize f32 [4096,4096] b4 g64", ms, nbytes=qbytes)
+    matmul_case("cfg1", 1, 4096, 4096, 4, 64, f32)
+    # Cfg2: decode, Llama-3-8B MLP shapes
+    for (n, k) in ((14336, 4096), (4096, 14336)):
+        for (bits, gs) in ((4, 64), (8, 128)):
+            for B in (1, 4, 8):
+                matmul_case("cfg2", B, n, k, bits, gs, bf16)
+    # Cfg3: prefill
+    for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336)):
+        for (bits, gs) in ((4, 64), (8, 128)):
+            for M in (512, 2048, 8192):
+                matmul_case("cfg3", M, n, k, bits, gs, bf16)
+    # Cfg4: 8 experts, top-2 routing
+    E, n, k = 8, 14336, 4096
+    wq, sc, bi = mlx_amd.quantize(
+        (torch.randn((E, n, k), generator=g, dtype=torch.float32) * 0.02).to(bf16).to(dev), 64, 4)
+    for T in (1, 64, 2048):
+        x = torch.randn((T, 1, 1, k), generator=g, dtype=torch.float32).to(bf16).to(dev)
+        idx = torch.randint(0, E, (T, 2), generator=torch.Generator().manual_seed(0)).to(dev)
+        ms = timed(lambda i: mlx_amd.gather_qmm(x, wq, sc, bi, rhs_indices=idx, transpose=True,
+                                                group_size=64, bits=4))
+        add("cfg4", f"gather T={T} top-2 of 8, unsorted", ms, flops=4.0 * T * n * k)
+        flat = idx.reshape(-1)
+        order = torch.argsort(flat, stable=True)
+        xs = x.reshape(T, 1, k)[order // 2].contiguous()
+        fs = flat[order].contiguous()
+        ms = timed(lambda i: mlx_amd.gather_qmm(xs, wq, sc, bi, rhs_indices=fs, transpose=True,
+                                                group_size=64, bits=4, sorted_indices=True))
+        add("cfg4", f"gather T={T} top-2 of 8, sorted", ms, flops=4.0 * T * n * k)
+    del wq, sc, bi
+    # Cfg5: odd code widths, group 32, Llama-2-7B MLP shapes
+    for dtype in (bf16, f32):
+        esz = 4 if dtype == f32 else 2
+        for bits in (2, 3, 5, 6):
+            w = weights(11008, 4096, dtype)
+            ms = timed(lambda i: mlx_amd.quantize(w, 32, bits))
+            nb = 11008 * 4096 * esz + 11008 * 4096 * bits // 8 + 2 * 11008 * 128 * esz
+            add("cfg5", f"quantize {str(dtype)[6:]} [11008,4096] b{bits} g32", ms, nbytes=nb)
+            matmul_case("cfg5", 1, 11008, 4096, bits, 32, dtype)
+            matmul_case("cfg5", 1024, 11008, 4096, bits, 32, dtype)
+            matmul_case("cfg5", 1, 4096, 11008, bits, 32, dtype)
+    return rows
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -134,6 +250,9 @@ def main() -> int:
     ap.add_argument("--only", choices=("qmv", "qmm_t"), default=None)
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying a HIP graph")
+    ap.add_argument("--sweep", action="store_true",
+                    help="time the other synthetic configurations of the path instead of "
+                         "the headline pair; prints one JSON line {\"sweep\": [...]}")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run 20 device-to-device copies of 256 MiB: the known-size "
                          "kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -164,6 +283,10 @@ def main() -> int:
             _lib.check(lib.mlxrocm_memcpy_d2d(dst.data_ptr(), src.data_ptr(), nbytes, stream))
         torch.cuda.synchronize()
         print(json.dumps({"copy_probe_bytes": nbytes, "copies": 20}))
+        return 0
+
+    if args.sweep:
+        print(json.dumps({"sweep": sweep(torch, mlx_amd, dev)}))
         return 0
 
     g = torch.Generator().manual_seed(0)

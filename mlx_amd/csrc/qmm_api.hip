@@ -1,5 +1,8 @@
 // qmm_api.hip -- C entry points of quantized_matmul / gather_qmm: argument
 // checks, kernel choice, launch.
+#include <mutex>
+#include <unordered_map>
+
 #include "qmm_args.h"
 
 namespace mlxrocm {
@@ -16,8 +19,8 @@ Family choose_family(int M, int /*N*/, int K, int /*L*/, int dtype, bool transpo
   if (transpose && M <= kQmvMaxM) {
     return Family::Qmv;
   }
-  if (transpose && dtype != MLXROCM_FLOAT32 && K % 64 == 0 && K >= 64) {
-    return Family::QmmT;
+  if (transpose && K % 64 == 0 && K >= 64) {
+    return Family::QmmT; // fp32 runs on the same matrix path, operands split in two
   }
   return Family::QmmNaive;
 }
@@ -106,11 +109,103 @@ int check_alignment(const char* who, const QmmArgs& a, int dtype) {
   return MLXROCM_OK;
 }
 
+// Device scratch that outlives a call: one buffer per stream, grown on demand
+// and kept until the process ends.  Work that uses it is ordered by the stream;
+// the mutex is held while that work is enqueued so that two host threads cannot
+// interleave their kernels on one buffer.
+struct StreamScratch {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_scratch_mu;
+std::unordered_map<hipStream_t, StreamScratch> g_scratch;
+
+int stream_scratch(hipStream_t s, size_t bytes, void** out) {
+  StreamScratch& sc = g_scratch[s];
+  if (sc.bytes < bytes) {
+    if (sc.ptr != nullptr) {
+      MLXROCM_HIP_TRY(hipStreamSynchronize(s)); // earlier users are done
+      MLXROCM_HIP_TRY(hipFree(sc.ptr));
+      sc.ptr = nullptr;
+      sc.bytes = 0;
+    }
+    const size_t want = (bytes + (size_t(1) << 21) - 1) >> 21 << 21;
+    hipError_t err = hipMalloc(&sc.ptr, want);
+    if (err != hipSuccess) {
+      (void)hipGetLastError();
+      sc.ptr = nullptr;
+      return fail(
+          err == hipErrorOutOfMemory ? MLXROCM_OUT_OF_MEMORY : MLXROCM_HIP_ERROR,
+          "[qmm] unable to allocate %zu bytes of scratch: %s",
+          want,
+          hipGetErrorString(err));
+    }
+    sc.bytes = want;
+  }
+  *out = sc.ptr;
+  return MLXROCM_OK;
+}
+
+// fp32 prefill: x is split into bf16 high/low parts in scratch, at most
+// kSplitScratchBytes of it at a time (row blocks of one batch entry), and each
+// block runs on the bf16 matrix path with fp32 scales, biases and output.
+constexpr size_t kSplitScratchBytes = size_t(256) << 20;
+
+int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
+  const size_t row_bytes = split_x_bytes(1, a.K);
+  int rows_per_block = static_cast<int>(kSplitScratchBytes / row_bytes / 256 * 256);
+  if (rows_per_block < 256) {
+    rows_per_block = 256;
+  }
+  if (rows_per_block > a.M) {
+    rows_per_block = a.M;
+  }
+  // the kernel addresses x with 32-bit element offsets
+  if (static_cast<uint64_t>(rows_per_block) * 3u * static_cast<uint64_t>(a.K) >= (uint64_t(1) << 32)) {
+    return launch_qmm_naive(a, gs, bits, MLXROCM_FLOAT32, true, s);
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  void* scratch = nullptr;
+  int rc = stream_scratch(s, split_x_bytes(rows_per_block, a.K), &scratch);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  for (int l = 0; l < a.L; ++l) {
+    for (int m_begin = 0; m_begin < a.M; m_begin += rows_per_block) {
+      const int rows = (a.M - m_begin < rows_per_block) ? a.M - m_begin : rows_per_block;
+      const float* x = static_cast<const float*>(a.x) + l * a.x_batch_stride +
+          static_cast<int64_t>(m_begin) * a.K;
+      rc = split_x_for_mfma(x, scratch, static_cast<size_t>(rows), a.K, s);
+      if (rc != MLXROCM_OK) {
+        return rc;
+      }
+      QmmArgs part = a;
+      part.x = scratch;
+      part.M = rows;
+      part.L = 1;
+      part.x_batch_stride = static_cast<int64_t>(rows) * 3 * a.K;
+      part.w = a.w + l * a.w_batch_stride;
+      part.scales = static_cast<const float*>(a.scales) + l * a.sb_batch_stride;
+      part.biases = static_cast<const float*>(a.biases) + l * a.sb_batch_stride;
+      part.out = static_cast<float*>(a.out) +
+          (static_cast<int64_t>(l) * a.M + m_begin) * static_cast<int64_t>(a.N);
+      rc = launch_qmm_mfma_split(part, gs, bits, s);
+      if (rc != MLXROCM_OK) {
+        return rc;
+      }
+    }
+  }
+  return MLXROCM_OK;
+}
+
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
   switch (choose_family(a.M, a.N, a.K, a.L, dtype, transpose)) {
     case Family::QmmT:
       if (qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
         return launch_qmm_mfma(a, gs, bits, dtype, s);
+      }
+      if (dtype == MLXROCM_FLOAT32 && a.lhs_indices == nullptr) {
+        return run_split_fp32(a, gs, bits, s);
       }
       return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
     case Family::Qmv:

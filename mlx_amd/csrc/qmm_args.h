@@ -95,6 +95,12 @@ int launch_zero_fill(void* p, size_t bytes, hipStream_t s);
 size_t gather_group_workspace_bytes(int n_indices, int n_experts);
 int gather_group_max_tiles(int n_indices, int n_experts);
 int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s);
+// fp32 operands on the bf16 matrix path: x is first split into bf16 high and
+// low parts (split_x_for_mfma into a buffer of split_x_bytes), then
+// launch_qmm_mfma_split runs with a.x pointing at that buffer.
+size_t split_x_bytes(size_t rows, int K);
+int split_x_for_mfma(const void* x, void* xs, size_t rows, int K, hipStream_t s);
+int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s);
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 
 } // namespace mlxrocm

@@ -20,10 +20,17 @@
 // The vector-ALU, LDS and global-memory instructions of a step are placed by
 // hand in the slots between the MFMAs (one scheduling barrier per slot), so the
 // matrix pipe never waits for a block of dequantization work.
+// fp32 operands run on the same bf16 matrix path at three times the K length:
+// a pre-pass splits x into a high and a low bf16 part, laid out per 64-wide k
+// block as [hi | lo | hi]; the kernel pairs those blocks with the weights'
+// [hi | hi | lo] parts (dequantized in fp32, split on the fly), which sums to
+// x_hi w_hi + x_lo w_hi + x_hi w_lo with fp32 accumulation -- a relative error
+// of about 2^-17 per product, inside the fp32 tolerance of the path.
 // LDS rows are 64 elements + 8 of padding (144 bytes), which makes the 16-byte
 // fragment reads of 16 consecutive rows hit 64 distinct banks.  The finished
 // tile is staged through LDS once more so that y is written in full 16-byte,
 // row-contiguous stores.
+#include <type_traits>
 #include <utility>
 
 #include "qmm_args.h"
@@ -89,8 +96,11 @@ template <typename T, int BITS>
 struct PairDequant {
   uint32_t lo, hi; // 4-bit: codes 0,2,4,6 / 1,3,5,7 of the current dword as bytes
 
+  // low_part: return v - T(v) instead of v (the second term of the split of an
+  // fp32 weight into two T values); wave-uniform.
   template <int Q>
-  __device__ __forceinline__ uint32_t pair(const uint32_t (&w)[BITS], float s, float b) {
+  __device__ __forceinline__ uint32_t
+  pair(const uint32_t (&w)[BITS], float s, float b, bool low_part = false) {
     float c0, c1;
     if constexpr (BITS == 4) {
       constexpr int d = Q / 4;
@@ -114,7 +124,13 @@ struct PairDequant {
       c0 = static_cast<float>(code32<BITS>(w, 2 * Q));
       c1 = static_cast<float>(code32<BITS>(w, 2 * Q + 1));
     }
-    return pack2<T>(fmaf(s, c0, b), fmaf(s, c1, b));
+    float v0 = fmaf(s, c0, b);
+    float v1 = fmaf(s, c1, b);
+    if (low_part) {
+      v0 -= static_cast<float>(static_cast<T>(v0));
+      v1 -= static_cast<float>(static_cast<T>(v1));
+    }
+    return pack2<T>(v0, v1);
   }
 };
 
@@ -168,8 +184,14 @@ constexpr int wstore_at(int m, int ns) {
 // GROUPED: blockIdx.y walks the tile list of a gather grouped by expert (M == 1
 // per index pair): the tile's rows are the x rows of up to 256 index pairs that
 // share one expert, fetched and written back through the permutation.
-template <typename T, int BITS, int NT, bool GROUPED>
+//
+// T is the MFMA operand type (what x and the LDS tiles hold), TS the type of
+// scales, biases and y: the same as T, or float in the split fp32 mode (where
+// a.x points at the [hi | lo | hi] bf16 image of x and spans 3 K).
+template <typename T, typename TS, int BITS, int NT, bool GROUPED>
 __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, const int gs_shift) {
+  constexpr bool kSplit = !std::is_same<T, TS>::value;
+  static_assert(!(kSplit && GROUPED), "the grouped gather runs on 16-bit types only");
   constexpr int kBN = 32 * NT;
   constexpr int kNS = 8 * NT; // MFMAs per wavefront per K-step
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -190,7 +212,15 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   int M = a.M;
   int m0 = blockIdx.y * kBM;
   int row0 = 0; // grouped: first sorted position of the tile
-  QmmProblem<T> p;
+  // operands of this workgroup's problem
+  struct {
+    const T* x;
+    const uint8_t* w;
+    const TS* scales;
+    const TS* biases;
+    TS* out;
+    bool valid;
+  } p;
   if constexpr (GROUPED) {
     const int tile = blockIdx.y;
     if (tile >= *a.group_ntiles) {
@@ -202,13 +232,31 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
     m0 = 0;
     p.x = static_cast<const T*>(a.x);
     p.w = reinterpret_cast<const uint8_t*>(a.w + static_cast<int64_t>(e) * a.w_batch_stride);
-    p.scales = static_cast<const T*>(a.scales) + static_cast<int64_t>(e) * a.sb_batch_stride;
-    p.biases = static_cast<const T*>(a.biases) + static_cast<int64_t>(e) * a.sb_batch_stride;
-    p.out = static_cast<T*>(a.out);
+    p.scales = static_cast<const TS*>(a.scales) + static_cast<int64_t>(e) * a.sb_batch_stride;
+    p.biases = static_cast<const TS*>(a.biases) + static_cast<int64_t>(e) * a.sb_batch_stride;
+    p.out = static_cast<TS*>(a.out);
     p.valid = true;
   } else {
-    p = resolve_problem<T>(a, blockIdx.z);
+    // same resolution as resolve_problem(), with the two element types
+    const int l = blockIdx.z;
+    int64_t xb = l;
+    int64_t wb = l;
+    p.valid = true;
+    if (a.lhs_indices != nullptr) {
+      const uint32_t xi = a.lhs_indices[l];
+      const uint32_t wi = a.rhs_indices[l];
+      p.valid = xi < static_cast<uint32_t>(a.x_batches) && wi < static_cast<uint32_t>(a.n_experts);
+      xb = p.valid ? xi : 0;
+      wb = p.valid ? wi : 0;
+    }
+    p.x = static_cast<const T*>(a.x) + xb * a.x_batch_stride;
+    p.w = reinterpret_cast<const uint8_t*>(a.w + wb * a.w_batch_stride);
+    p.scales = static_cast<const TS*>(a.scales) + wb * a.sb_batch_stride;
+    p.biases = static_cast<const TS*>(a.biases) + wb * a.sb_batch_stride;
+    p.out = static_cast<TS*>(a.out) + static_cast<int64_t>(l) * a.M * static_cast<int64_t>(a.N);
   }
+  // x as the kernel sees it: three 64-wide blocks per block of K when split
+  const int Kx = kSplit ? 3 * K : K;
 
   const int groups = K >> gs_shift;
   const int row_words = K / 32 * BITS;
@@ -224,8 +272,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
   const uint32_t* wsrc = reinterpret_cast<const uint32_t*>(p.w) +
       static_cast<size_t>(w_row) * row_words + wh * BITS;
-  const T* ssrc = p.scales + static_cast<size_t>(w_row) * groups;
-  const T* bsrc = p.biases + static_cast<size_t>(w_row) * groups;
+  const TS* ssrc = p.scales + static_cast<size_t>(w_row) * groups;
+  const TS* bsrc = p.biases + static_cast<size_t>(w_row) * groups;
   // Rows of x past M are never stored, so they may read any valid row: the
   // loads then need no predicate.  32-bit element offsets from p.x.
   uint32_t xoff0, xoff1, xoff2, xoff3;
@@ -237,7 +285,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
         const uint32_t pair = static_cast<uint32_t>(a.group_perm[row0 + mc]);
         return a.lhs_indices[pair] * static_cast<uint32_t>(a.x_batch_stride) + xc * 8;
       } else {
-        return static_cast<uint32_t>(mc) * static_cast<uint32_t>(K) + xc * 8;
+        return static_cast<uint32_t>(mc) * static_cast<uint32_t>(Kx) + xc * 8;
       }
     };
     xoff0 = row_off(0);
@@ -256,7 +304,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 // scratch memory
 #define QMM_XQ(set, i) (*((kXSets == 2 && (set) == 1) ? &xb##i : &xa##i))
   uint32_t wreg[BITS], wnext[BITS];
-  T sreg, breg, snext, bnext; // converted when used, so the loads are not waited for early
+  TS sreg, breg, snext, bnext; // converted when used, so the loads are not waited for early
 
 #define QMM_LOAD_X(set, k0)                                                      \
   do {                                                                           \
@@ -268,11 +316,13 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 
 #define QMM_LOAD_W(k0)                                                           \
   do {                                                                           \
-    const uint32_t* wp__ = wsrc + ((k0) / 32) * BITS;                            \
+    /* split mode: blocks 3t, 3t+1, 3t+2 of x all meet block t of W */           \
+    const int kw__ = kSplit ? ((k0) / (3 * kBK)) * kBK : (k0);                   \
+    const uint32_t* wp__ = wsrc + (kw__ / 32) * BITS;                            \
     _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
       wnext[j__] = wp__[j__];                                                    \
     }                                                                            \
-    const int g__ = ((k0) + 32 * wh) >> gs_shift;                                \
+    const int g__ = (kw__ + 32 * wh) >> gs_shift;                                \
     snext = ssrc[g__];                                                           \
     bnext = bsrc[g__];                                                           \
   } while (0)
@@ -355,7 +405,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   //     without waiting for LDS.
   // Every step is the same code, the last one included: its fetches are clamped
   // to the last tile and what it stores is never read.
-  const int nk = K / kBK;
+  const int nk = Kx / kBK;
   const int klast = (nk - 1) * kBK;
   auto kclamp = [&](int t) { return t * kBK < klast ? t * kBK : klast; };
   QMM_LOAD_X(0, 0);
@@ -408,7 +458,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
       QMM_LOAD_W(k2);                                                            \
     }                                                                            \
     if constexpr (pair_at((m), kNS) >= 0) {                                      \
-      dqv[pair_at((m), kNS)] = dq.template pair<pair_at((m), kNS)>(wreg, sf, bf); \
+      dqv[pair_at((m), kNS)] =                                                   \
+          dq.template pair<pair_at((m), kNS)>(wreg, sf, bf, low_part);           \
     }                                                                            \
     if constexpr (wstore_at((m), kNS) >= 0) {                                    \
       constexpr int r__ = wstore_at((m), kNS);                                   \
@@ -452,6 +503,9 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
     uint4* wdst = reinterpret_cast<uint4*>(&xs[kXTile + wr * kLdsStride + wh * 32]); \
     const float sf = to_f32(sreg);                                               \
     const float bf = to_f32(breg);                                               \
+    /* the tile prepared in step tt is tile tt + 1: block (tt + 1) % 3 of its   \
+       group of three takes the weights' low parts */                           \
+    const bool low_part = kSplit && ((tt) + 1) % 3 == 2;                         \
     PairDequant<T, BITS> dq;                                                     \
     uint32_t dqv[16];                                                            \
     __builtin_amdgcn_sched_barrier(0);                                           \
@@ -473,53 +527,69 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 #undef QMM_SLOT
 
   // ---- epilogue.  D[n][m] tiles: register r of lane (col, quad) holds
-  // n = 4 quad + r, m = col.  The tile is rounded to T and staged in LDS as
+  // n = 4 quad + r, m = col.  The tile is rounded to TS and staged in LDS as
   // ys[m][n] (the K loop is done with it), then written out row by row in
-  // 16-byte pieces, 32 NT * 2 contiguous bytes per row.
-  __syncthreads();
+  // 16-byte pieces, whole rows of the tile contiguous.  fp32 tiles go in two
+  // halves of 128 rows, which is what fits.
+  constexpr int kPasses = sizeof(TS) == 4 ? 2 : 1;
+  constexpr int kPassRows = kBM / kPasses;
+  constexpr int kPiece = 16 / static_cast<int>(sizeof(TS)); // elements per 16 bytes
   constexpr int kOutStride = kBN + kOutPad;
-  T* ys = lds;
-  {
-    const int col = lane & 15;
-    const int quad = lane >> 4;
+  TS* ys = reinterpret_cast<TS*>(smem);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      T* yrow = ys + (wm * 64 + j * 16 + col) * kOutStride + wn * 16 * NT + 4 * quad;
+  for (int pass = 0; pass < kPasses; ++pass) {
+    __syncthreads(); // LDS is free: K loop (pass 0) or the previous half is done
+    if (wm * 64 / kPassRows == pass) {
+      const int col = lane & 15;
+      const int quad = lane >> 4;
 #pragma unroll
-      for (int i = 0; i < NT; ++i) {
-        uint2 packed;
-        packed.x = pack2<T>(acc[i][j][0], acc[i][j][1]);
-        packed.y = pack2<T>(acc[i][j][2], acc[i][j][3]);
-        if (!p.valid) {
-          packed = make_uint2(0u, 0u);
+      for (int j = 0; j < 4; ++j) {
+        TS* yrow = ys + ((wm * 64) % kPassRows + j * 16 + col) * kOutStride +
+            wn * 16 * NT + 4 * quad;
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+          if constexpr (sizeof(TS) == 4) {
+            float4 v = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+            if (!p.valid) {
+              v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
+            *reinterpret_cast<float4*>(yrow + 16 * i) = v;
+          } else {
+            uint2 packed;
+            packed.x = pack2<TS>(acc[i][j][0], acc[i][j][1]);
+            packed.y = pack2<TS>(acc[i][j][2], acc[i][j][3]);
+            if (!p.valid) {
+              packed = make_uint2(0u, 0u);
+            }
+            *reinterpret_cast<uint2*>(yrow + 16 * i) = packed;
+          }
         }
-        *reinterpret_cast<uint2*>(yrow + 16 * i) = packed;
       }
     }
-  }
-  __syncthreads();
-  {
-    constexpr int kChunks = kBN / 8;             // 16-byte pieces per tile row
-    constexpr int kRowsPerPass = kThreads / 32;  // 32 lanes cover up to 256 columns
-    const int c = tid & 31;
-    const int r0 = tid >> 5;
-    const bool vec_ok = (N % 8) == 0; // rows of y stay 16-byte aligned
+    __syncthreads();
+    constexpr int kChunks = kBN / kPiece;        // 16-byte pieces per tile row
+    constexpr int kLanesPerRow = 256 / kPiece;   // a power of two >= kChunks
+    constexpr int kRowsPerIter = kThreads / kLanesPerRow;
+    const int c = tid % kLanesPerRow;
+    const int r0 = tid / kLanesPerRow;
+    const bool vec_ok = (N % kPiece) == 0; // rows of y stay 16-byte aligned
     if (c < kChunks) {
 #pragma unroll 4
-      for (int r = r0; r < kBM; r += kRowsPerPass) {
-        const int m = m0 + r;
-        const int n = n0 + c * 8;
-        if (m >= M || n >= N) {
+      for (int r = r0; r < kPassRows; r += kRowsPerIter) {
+        const int mr = pass * kPassRows + r; // row inside the tile
+        const int m = m0 + mr;
+        const int n = n0 + c * kPiece;
+        if (mr >= M - m0 || m >= M || n >= N) {
           continue;
         }
-        const T* src = ys + r * kOutStride + c * 8;
+        const TS* src = ys + r * kOutStride + c * kPiece;
         const size_t orow =
-            GROUPED ? static_cast<size_t>(a.group_perm[row0 + r]) : static_cast<size_t>(m);
-        T* dst = p.out + orow * N + n;
-        if (vec_ok && n + 8 <= N) {
+            GROUPED ? static_cast<size_t>(a.group_perm[row0 + mr]) : static_cast<size_t>(m);
+        TS* dst = p.out + orow * N + n;
+        if (vec_ok && n + kPiece <= N) {
           *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
         } else {
-          for (int e = 0; e < 8 && n + e < N; ++e) {
+          for (int e = 0; e < kPiece && n + e < N; ++e) {
             dst[e] = src[e];
           }
         }
@@ -538,6 +608,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 template <int NT>
 constexpr size_t qmm_smem_bytes() {
   constexpr size_t stages = static_cast<size_t>(2) * (kBM + 32 * NT) * kLdsStride * 2;
+  // staged y tile: all 256 rows of a 16-bit tile or 128 rows of an fp32 tile
   constexpr size_t out = static_cast<size_t>(kBM) * (32 * NT + kOutPad) * 2;
   return stages > out ? stages : out;
 }
@@ -573,13 +644,13 @@ int choose_nt(int M, int N, int L) {
   return best;
 }
 
-template <typename T, int BITS, int NT, bool GROUPED>
+template <typename T, typename TS, int BITS, int NT, bool GROUPED>
 int launch_variant(const QmmArgs& a, int gs_shift, dim3 grid, hipStream_t s) {
   constexpr size_t smem = qmm_smem_bytes<NT>();
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
-  auto kern = qmm_t_mfma_kernel<T, BITS, NT, GROUPED>;
+  auto kern = qmm_t_mfma_kernel<T, TS, BITS, NT, GROUPED>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -618,15 +689,79 @@ int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
       constexpr int B = decltype(bval)::value;
       switch (nt) {
         case 5:
-          return launch_variant<T, B, 5, false>(a, gs_shift, grid, s);
+          return launch_variant<T, T, B, 5, false>(a, gs_shift, grid, s);
         case 6:
-          return launch_variant<T, B, 6, false>(a, gs_shift, grid, s);
+          return launch_variant<T, T, B, 6, false>(a, gs_shift, grid, s);
         default:
-          return launch_variant<T, B, 7, false>(a, gs_shift, grid, s);
+          return launch_variant<T, T, B, 7, false>(a, gs_shift, grid, s);
       }
     });
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
+}
+
+// fp32 operands: `a.x` already points at the [hi | lo | hi] bf16 image of x
+// (split_x_for_mfma) and a.x_batch_stride counts its elements (M * 3 K).
+int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s) {
+  constexpr int kNT = 7;
+  const int gs_shift = shift_of(gs);
+  const dim3 grid((a.N + 32 * kNT - 1) / (32 * kNT), (a.M + kBM - 1) / kBM, a.L);
+  return dispatch_bits(bits, [&](auto bval) {
+    constexpr int B = decltype(bval)::value;
+    return launch_variant<bf16_t, float, B, kNT, false>(a, gs_shift, grid, s);
+  });
+}
+
+namespace {
+
+// 8 consecutive fp32 of x -> 8 bf16 high parts and 8 bf16 low parts, written to
+// blocks 0/2 and 1 of the element's group of three 64-wide blocks.
+__global__ __launch_bounds__(256) void split_x_kernel(
+    const float* x,
+    bf16_t* xs,
+    size_t rows,
+    int K) {
+  const size_t unit = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t units_per_row = static_cast<size_t>(K) / 8;
+  if (unit >= rows * units_per_row) {
+    return;
+  }
+  const size_t row = unit / units_per_row;
+  const int k = static_cast<int>(unit - row * units_per_row) * 8;
+  const float4 v0 = *reinterpret_cast<const float4*>(x + row * K + k);
+  const float4 v1 = *reinterpret_cast<const float4*>(x + row * K + k + 4);
+  const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+  uint32_t hi[4], lo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float h0 = static_cast<float>(static_cast<bf16_t>(v[2 * i]));
+    const float h1 = static_cast<float>(static_cast<bf16_t>(v[2 * i + 1]));
+    hi[i] = pack2<bf16_t>(v[2 * i], v[2 * i + 1]);
+    lo[i] = pack2<bf16_t>(v[2 * i] - h0, v[2 * i + 1] - h1);
+  }
+  bf16_t* dst = xs + row * (3 * static_cast<size_t>(K)) + static_cast<size_t>(k / 64) * 192 + k % 64;
+  const uint4 h = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+  *reinterpret_cast<uint4*>(dst) = h;
+  *reinterpret_cast<uint4*>(dst + 64) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+  *reinterpret_cast<uint4*>(dst + 128) = h;
+}
+
+} // namespace
+
+size_t split_x_bytes(size_t rows, int K) {
+  return rows * 3 * static_cast<size_t>(K) * sizeof(bf16_t);
+}
+
+int split_x_for_mfma(const void* x, void* xs, size_t rows, int K, hipStream_t s) {
+  const size_t units = rows * (static_cast<size_t>(K) / 8);
+  const size_t blocks = (units + 255) / 256;
+  if (blocks > 0x7fffffffull) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmm] x is too large to split");
+  }
+  split_x_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(
+      static_cast<const float*>(x), static_cast<bf16_t*>(xs), rows, K);
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return MLXROCM_OK;
 }
 
 // Gather grouped by expert: `a` carries the tile list; one grid row per
@@ -640,7 +775,7 @@ int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipSt
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
       constexpr int B = decltype(bval)::value;
-      return launch_variant<T, B, kNT, true>(a, gs_shift, grid, s);
+      return launch_variant<T, T, B, kNT, true>(a, gs_shift, grid, s);
     });
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});

@@ -141,3 +141,30 @@ def test_qmm_type_promotion(gpu):
     assert out.dtype == torch.float32
     out16 = mlx_amd.quantized_matmul(x.to(torch.float16), wq, s, b)
     assert out16.dtype == torch.float32  # float16 x bfloat16 -> float32
+
+
+def test_qmm_t_fp32_runs_on_the_matrix_path(oracle, gpu):
+    """fp32 prefill (M > 8, K a multiple of 64) is computed on the bf16 matrix
+    cores from operands split into high and low parts: the fp32 bound still
+    holds, also for batched x, batched weights, ragged M / N and heavy-tailed
+    weights (Student-t, 3 degrees of freedom)."""
+    from mlx_amd import _lib
+    lib = _lib.load()
+    assert lib.mlxrocm_qmm_kernel_name(1024, 11008, 4096, 1, 32, 3, 0, 1) == b"qmm_t"
+    g = torch.Generator().manual_seed(3)
+    for (M, N, K, bits, gs) in ((9, 50, 64, 4, 32), (300, 232, 1024, 8, 128), (513, 67, 448, 5, 64)):
+        t = torch.distributions.StudentT(3.0).sample((N, K)) * 0.02
+        w = t.clamp(-1.0, 1.0).float()
+        x = activations((M, K), torch.float32, seed=M)
+        _check_qmm(oracle, gpu, x, w, gs, bits)
+    # batched x against one weight and against batched weights
+    gs, bits = 64, 4
+    x = activations((3, 40, 256), torch.float32)
+    w3 = normal_weights((3, 96, 256), torch.float32, seed=7)
+    wq3, s3, b3 = oracle.quantize(w3, gs, bits)
+    for q in ((wq3[0], s3[0], b3[0]), (wq3, s3, b3)):
+        got = mlx_amd.quantized_matmul(x.to(gpu), *(t.to(gpu) for t in q), True, gs, bits)
+        ref = oracle.qmm_batched(x, *q, True, gs, bits)
+        assert got.shape == (3, 40, 96)
+        assert float((got.cpu() - ref).abs().max()) <= matmul_tolerance(
+            torch.float32, 256, x, exact_affine_weights(wq3, s3, b3, gs, bits))
