@@ -199,6 +199,21 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
 }
 
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
+  // A few rows of x, beyond what the row-streaming GEMV keeps in registers.
+  // Measured on gate/up and down projection shapes (4- and 8-bit):
+  //   3..8 rows   the 32-row MFMA GEMV up to K = 8192, the wide kernel (K split
+  //               over the wavefronts of a workgroup) beyond;
+  //   9..16 rows  the wide kernel;
+  //   17..32 rows the 64-row LDS-staged kernel.
+  if (a.M >= 3 && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
+    const bool gemv_better = a.M <= 8 && a.K <= 8192 && qmv_mfma_supported(a, gs, bits, dtype);
+    if (!gemv_better) {
+      return launch_qmv_wide(a, gs, bits, dtype, s);
+    }
+  }
+  if (a.M > 16 && qmm_skinny_supported(a, gs, bits, dtype, transpose)) {
+    return launch_qmm_skinny(a, gs, bits, dtype, s);
+  }
   switch (choose_family(a.M, a.N, a.K, a.L, dtype, transpose)) {
     case Family::QmmT:
       if (qmm_mfma_supported(a, gs, bits, dtype, transpose)) {

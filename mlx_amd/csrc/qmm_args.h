@@ -88,6 +88,10 @@ bool qmv_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype);
 int launch_qmv_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+bool qmv_wide_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
+int launch_qmv_wide(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+bool qmm_skinny_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
+int launch_qmm_skinny(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 int launch_zero_fill(void* p, size_t bytes, hipStream_t s);
 
 // Grouping of gathered index pairs by expert (gather_group.hip) and the grouped

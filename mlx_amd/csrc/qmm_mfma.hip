@@ -30,130 +30,18 @@
 // fragment reads of 16 consecutive rows hit 64 distinct banks.  The finished
 // tile is staged through LDS once more so that y is written in full 16-byte,
 // row-contiguous stores.
-#include <type_traits>
-#include <utility>
-
+#include "mfma_dequant.h"
 #include "qmm_args.h"
 
 namespace mlxrocm {
 
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-
 constexpr int kBM = 256;
 constexpr int kBK = 64;
 constexpr int kLdsStride = kBK + 8; // elements per LDS row
 constexpr int kThreads = 512;
 constexpr int kOutPad = 8; // elements of padding per row of the staged y tile
-
-template <typename T>
-__device__ __forceinline__ floatx4 mfma16(const uint4& a, const uint4& b, const floatx4& c);
-
-template <>
-__device__ __forceinline__ floatx4
-mfma16<bf16_t>(const uint4& a, const uint4& b, const floatx4& c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-      __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
-template <>
-__device__ __forceinline__ floatx4
-mfma16<f16_t>(const uint4& a, const uint4& b, const floatx4& c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(
-      __builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-
-// Two floats -> two T in one dword (lo in the low half), round to nearest even;
-// the vector convert selects the packed hardware convert.
-template <typename T>
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  typedef T Tx2 __attribute__((ext_vector_type(2)));
-  const floatx2 v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, Tx2));
-}
-
-// Code i (0..31) of the 32 codes held in BITS consecutive dwords.
-template <int BITS>
-__device__ __forceinline__ uint32_t code32(const uint32_t (&w)[BITS], int i) {
-  const int bit = i * BITS;
-  const int word = bit >> 5;
-  const int sh = bit & 31;
-  uint32_t v = w[word] >> sh;
-  if (sh + BITS > 32) {
-    v |= w[word + 1] << (32 - sh);
-  }
-  return v & ((1u << BITS) - 1u);
-}
-
-// Dequantization of the 32 codes held in BITS consecutive dwords, two codes at
-// a time so that the work can be spread between MFMAs: pair<Q>() returns
-// elements 2Q and 2Q+1 as fma(s, code, b) in fp32, rounded once to T and packed.
-template <typename T, int BITS>
-struct PairDequant {
-  uint32_t lo, hi; // 4-bit: codes 0,2,4,6 / 1,3,5,7 of the current dword as bytes
-
-  // low_part: return v - T(v) instead of v (the second term of the split of an
-  // fp32 weight into two T values); wave-uniform.
-  template <int Q>
-  __device__ __forceinline__ uint32_t
-  pair(const uint32_t (&w)[BITS], float s, float b, bool low_part = false) {
-    float c0, c1;
-    if constexpr (BITS == 4) {
-      constexpr int d = Q / 4;
-      constexpr int j = Q % 4;
-      if constexpr (j == 0) {
-        lo = w[d] & 0x0f0f0f0fu;
-        hi = (w[d] >> 4) & 0x0f0f0f0fu;
-        // keep the byte form: otherwise the shifts are folded back into one
-        // bit-field extract per code
-        asm("" : "+v"(lo));
-        asm("" : "+v"(hi));
-      }
-      c0 = static_cast<float>((lo >> (8 * j)) & 0xffu);
-      c1 = static_cast<float>((hi >> (8 * j)) & 0xffu);
-    } else if constexpr (BITS == 8) {
-      constexpr int d = Q / 2;
-      constexpr int j = Q % 2;
-      c0 = static_cast<float>((w[d] >> (16 * j)) & 0xffu);
-      c1 = static_cast<float>((w[d] >> (16 * j + 8)) & 0xffu);
-    } else {
-      c0 = static_cast<float>(code32<BITS>(w, 2 * Q));
-      c1 = static_cast<float>(code32<BITS>(w, 2 * Q + 1));
-    }
-    float v0 = fmaf(s, c0, b);
-    float v1 = fmaf(s, c1, b);
-    if (low_part) {
-      v0 -= static_cast<float>(static_cast<T>(v0));
-      v1 -= static_cast<float>(static_cast<T>(v1));
-    }
-    return pack2<T>(v0, v1);
-  }
-};
-
-template <typename T, int BITS, int... Q>
-__device__ __forceinline__ void dequant32_impl(
-    const uint32_t (&w)[BITS],
-    float s,
-    float b,
-    uint32_t (&out)[16],
-    std::integer_sequence<int, Q...>) {
-  PairDequant<T, BITS> dq;
-  ((out[Q] = dq.template pair<Q>(w, s, b)), ...);
-}
-
-// 32 codes -> 32 elements of T in one go (prologue).
-template <typename T, int BITS>
-__device__ __forceinline__ void dequant32(
-    const uint32_t (&w)[BITS],
-    float s,
-    float b,
-    uint32_t (&out)[16]) {
-  dequant32_impl<T, BITS>(w, s, b, out, std::make_integer_sequence<int, 16>{});
-}
 
 // ---- placement of the side work in the MFMA slots of one K-step -------------
 // NS = 8 NT slots.  Everything that writes LDS has to be issued before the
