@@ -28,8 +28,8 @@ BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes, scaled by
 # a copy of known size (profiles/qmv_stream_4bit_g64_bf16_14336x4096.md and
 # profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md).
-QMV_TRAFFIC_BYTES = 33224900
-QMM_T_TRAFFIC_BYTES = 276972000
+QMV_TRAFFIC_BYTES = 33221941
+QMM_T_TRAFFIC_BYTES = 258712822
 
 N, K = 14336, 4096
 BITS, GS = 4, 64
@@ -175,15 +175,33 @@ def sweep(torch, mlx_amd, dev) -> list:
         return _lib.load().mlxrocm_qmm_kernel_name(M, n, k, 1, gs, bits, code, 1).decode()
 
     def matmul_case(cfg, M, n, k, bits, gs, dtype):
+        """One quantized_matmul shape through the C ABI.  Launches that last a few
+        microseconds (M <= 64) replay a HIP graph over the weight ring, like the
+        headline figure; the others are launched one by one."""
+        from mlx_amd import _lib
+        lib = _lib.load()
         esz = 4 if dtype == torch.float32 else 2
+        code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
         q = mlx_amd.quantize(weights(n, k, dtype), gs, bits)
         wbytes = n * k * bits // 8 + 2 * n * (k // gs) * esz
-        ring = ring_of(q, wbytes) if M <= 64 else [q]
+        small = M <= 64
+        ring = ring_of(q, wbytes) if small else [q]
         x = torch.randn((M, k), generator=g, dtype=torch.float32).to(dtype).to(dev)
-        fn = lambda i: mlx_amd.quantized_matmul(x, *ring[i % len(ring)], True, gs, bits)
-        ms = timed(fn)
+        out = torch.empty((M, n), dtype=dtype, device=dev)
+
+        def step(i, stream):
+            wq_, s_, b_ = ring[i % len(ring)]
+            rc = lib.mlxrocm_qmm(x.data_ptr(), wq_.data_ptr(), s_.data_ptr(), b_.data_ptr(),
+                                 out.data_ptr(), M, n, k, 1, M * k, 0, 0, gs, bits, code, 1, stream)
+            if rc != 0:
+                raise RuntimeError(_lib.last_error())
+
+        launcher = Launcher(torch, step, len(ring), small)
+        launcher.run(len(ring))
+        torch.cuda.synchronize()
+        ms = hip_event_ms(lib, launcher, max(len(ring) * (20 if small else 1), 10))
         name = f"x {str(dtype)[6:]} [{M},{k}] W [{n},{k}] b{bits} g{gs}"
-        if M <= 64:
+        if small:
             add(cfg, name, ms, nbytes=qmv_bytes(M, n, k, bits, gs, esz),
                 kernel=kname(M, n, k, gs, bits, dtype))
         else:

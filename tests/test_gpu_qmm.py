@@ -168,3 +168,16 @@ def test_qmm_t_fp32_runs_on_the_matrix_path(oracle, gpu):
         assert got.shape == (3, 40, 96)
         assert float((got.cpu() - ref).abs().max()) <= matmul_tolerance(
             torch.float32, 256, x, exact_affine_weights(wq3, s3, b3, gs, bits))
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("bits", ALL_BITS)
+def test_qmm_few_rows_kernels(oracle, gpu, dtype, bits):
+    """3 <= M <= 32 goes to the few-row kernels (K split over wavefronts up to 16
+    rows, 64-row LDS-staged tiles up to 32): ragged N, K of one and of several
+    steps, every group size."""
+    for gs in ALL_GROUPS:
+        for M, N, K in ((5, 67, 128), (12, 130, 1280), (16, 48, 8704), (17, 200, 256), (32, 67, 1792)):
+            w = normal_weights((N, K), dtype, seed=bits + gs + M)
+            x = activations((M, K), dtype, seed=M)
+            _check_qmm(oracle, gpu, x, w, gs, bits)
