@@ -164,12 +164,21 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
   if (static_cast<uint64_t>(rows_per_block) * 3u * static_cast<uint64_t>(a.K) >= (uint64_t(1) << 32)) {
     return launch_qmm_naive(a, gs, bits, MLXROCM_FLOAT32, true, s);
   }
+  // few tiles: also cut K (one row block, one batch entry only)
+  int k_splits = 1;
+  if (rows_per_block == a.M && a.L == 1 && (static_cast<int64_t>(a.M) * a.N) % 4 == 0) {
+    k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, 1);
+  }
+  const size_t x_bytes = (split_x_bytes(rows_per_block, a.K) + 255) / 256 * 256;
+  const size_t plane = static_cast<size_t>(a.M) * a.N;
+  const size_t partial_bytes = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
   std::lock_guard<std::mutex> lock(g_scratch_mu);
   void* scratch = nullptr;
-  int rc = stream_scratch(s, split_x_bytes(rows_per_block, a.K), &scratch);
+  int rc = stream_scratch(s, x_bytes + partial_bytes, &scratch);
   if (rc != MLXROCM_OK) {
     return rc;
   }
+  void* partial = static_cast<char*>(scratch) + x_bytes;
   for (int l = 0; l < a.L; ++l) {
     for (int m_begin = 0; m_begin < a.M; m_begin += rows_per_block) {
       const int rows = (a.M - m_begin < rows_per_block) ? a.M - m_begin : rows_per_block;
@@ -187,15 +196,41 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
       part.w = a.w + l * a.w_batch_stride;
       part.scales = static_cast<const float*>(a.scales) + l * a.sb_batch_stride;
       part.biases = static_cast<const float*>(a.biases) + l * a.sb_batch_stride;
-      part.out = static_cast<float*>(a.out) +
+      float* out = static_cast<float*>(a.out) +
           (static_cast<int64_t>(l) * a.M + m_begin) * static_cast<int64_t>(a.N);
-      rc = launch_qmm_mfma_split(part, gs, bits, s);
+      part.out = k_splits > 1 ? partial : out;
+      rc = launch_qmm_mfma_split(part, gs, bits, s, k_splits);
       if (rc != MLXROCM_OK) {
         return rc;
+      }
+      if (k_splits > 1) {
+        rc = reduce_k_splits(partial, out, plane, k_splits, MLXROCM_FLOAT32, s);
+        if (rc != MLXROCM_OK) {
+          return rc;
+        }
       }
     }
   }
   return MLXROCM_OK;
+}
+
+// 16-bit prefill whose tiles would leave most compute units idle: K is cut into
+// ranges, the fp32 partial tiles go to scratch and are added up.
+int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
+  const size_t plane = static_cast<size_t>(a.M) * a.N;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  void* scratch = nullptr;
+  int rc = stream_scratch(s, plane * k_splits * sizeof(float), &scratch);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  QmmArgs part = a;
+  part.out = scratch;
+  rc = launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  return reduce_k_splits(scratch, a.out, plane, k_splits, dtype, s);
 }
 
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
@@ -217,6 +252,12 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   switch (choose_family(a.M, a.N, a.K, a.L, dtype, transpose)) {
     case Family::QmmT:
       if (qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
+        if (a.lhs_indices == nullptr && (static_cast<int64_t>(a.M) * a.N) % 4 == 0) {
+          const int k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, a.L);
+          if (k_splits > 1) {
+            return run_k_split(a, gs, bits, dtype, k_splits, s);
+          }
+        }
         return launch_qmm_mfma(a, gs, bits, dtype, s);
       }
       if (dtype == MLXROCM_FLOAT32 && a.lhs_indices == nullptr) {

@@ -104,7 +104,12 @@ int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s);
 // launch_qmm_mfma_split runs with a.x pointing at that buffer.
 size_t split_x_bytes(size_t rows, int K);
 int split_x_for_mfma(const void* x, void* xs, size_t rows, int K, hipStream_t s);
-int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s);
+int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s, int k_splits);
+// Few tiles: K is cut into qmm_mfma_k_splits() ranges whose fp32 partial tiles
+// (k_splits planes of M x N behind a.out) reduce_k_splits() adds up.
+int qmm_mfma_k_splits(int M, int N, int K, int L);
+int launch_qmm_mfma_ksplit(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
+int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int dtype, hipStream_t s);
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 
 } // namespace mlxrocm

@@ -74,10 +74,15 @@ constexpr int wstore_at(int m, int ns) {
 // share one expert, fetched and written back through the permutation.
 //
 // T is the MFMA operand type (what x and the LDS tiles hold), TS the type of
-// scales, biases and y: the same as T, or float in the split fp32 mode (where
-// a.x points at the [hi | lo | hi] bf16 image of x and spans 3 K).
-template <typename T, typename TS, int BITS, int NT, bool GROUPED>
-__global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, const int gs_shift) {
+// scales and biases: the same as T, or float in the split fp32 mode (where a.x
+// points at the [hi | lo | hi] bf16 image of x and spans 3 K).  TO is the type
+// of y: TS, or float when K is cut into k_splits ranges (blockIdx.z), each of
+// which writes its partial tile to plane blockIdx.z of a.out.
+template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED>
+__global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
+    const QmmArgs a,
+    const int gs_shift,
+    const int k_splits) {
   constexpr bool kSplit = !std::is_same<T, TS>::value;
   static_assert(!(kSplit && GROUPED), "the grouped gather runs on 16-bit types only");
   constexpr int kBN = 32 * NT;
@@ -106,7 +111,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
     const uint8_t* w;
     const TS* scales;
     const TS* biases;
-    TS* out;
+    TO* out;
     bool valid;
   } p;
   if constexpr (GROUPED) {
@@ -122,11 +127,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
     p.w = reinterpret_cast<const uint8_t*>(a.w + static_cast<int64_t>(e) * a.w_batch_stride);
     p.scales = static_cast<const TS*>(a.scales) + static_cast<int64_t>(e) * a.sb_batch_stride;
     p.biases = static_cast<const TS*>(a.biases) + static_cast<int64_t>(e) * a.sb_batch_stride;
-    p.out = static_cast<TS*>(a.out);
+    p.out = static_cast<TO*>(a.out);
     p.valid = true;
   } else {
-    // same resolution as resolve_problem(), with the two element types
-    const int l = blockIdx.z;
+    // same resolution as resolve_problem(), with the two element types; with a
+    // split K there is one problem and blockIdx.z is the split
+    const int l = k_splits > 1 ? 0 : blockIdx.z;
     int64_t xb = l;
     int64_t wb = l;
     p.valid = true;
@@ -141,7 +147,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
     p.w = reinterpret_cast<const uint8_t*>(a.w + wb * a.w_batch_stride);
     p.scales = static_cast<const TS*>(a.scales) + wb * a.sb_batch_stride;
     p.biases = static_cast<const TS*>(a.biases) + wb * a.sb_batch_stride;
-    p.out = static_cast<TS*>(a.out) + static_cast<int64_t>(l) * a.M * static_cast<int64_t>(a.N);
+    const int64_t plane = k_splits > 1 ? blockIdx.z : l;
+    p.out = static_cast<TO*>(a.out) + plane * a.M * static_cast<int64_t>(a.N);
   }
   // x as the kernel sees it: three 64-wide blocks per block of K when split
   const int Kx = kSplit ? 3 * K : K;
@@ -293,11 +300,23 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
   //     without waiting for LDS.
   // Every step is the same code, the last one included: its fetches are clamped
   // to the last tile and what it stores is never read.
-  const int nk = Kx / kBK;
+  // This workgroup's K range, in steps of the x image: everything, or split
+  // blockIdx.z of k_splits (whole groups of three steps in the split fp32 mode).
+  int step_begin = 0;
+  int nk = Kx / kBK;
+  if (k_splits > 1) {
+    constexpr int kUnit = kSplit ? 3 : 1;
+    const int units = nk / kUnit;
+    const int z = blockIdx.z;
+    step_begin = units * z / k_splits * kUnit;
+    nk = units * (z + 1) / k_splits * kUnit - step_begin;
+  }
+  const int kbeg = step_begin * kBK;
   const int klast = (nk - 1) * kBK;
-  auto kclamp = [&](int t) { return t * kBK < klast ? t * kBK : klast; };
-  QMM_LOAD_X(0, 0);
-  QMM_LOAD_W(0);
+  // x-image offset of local step t, clamped to the range's last step
+  auto kclamp = [&](int t) { return kbeg + (t * kBK < klast ? t * kBK : klast); };
+  QMM_LOAD_X(0, kbeg);
+  QMM_LOAD_W(kbeg);
   QMM_ROTATE_W();
   QMM_STORE_X(0, 0);
   QMM_STORE_W(0);
@@ -415,15 +434,15 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
 #undef QMM_SLOT
 
   // ---- epilogue.  D[n][m] tiles: register r of lane (col, quad) holds
-  // n = 4 quad + r, m = col.  The tile is rounded to TS and staged in LDS as
+  // n = 4 quad + r, m = col.  The tile is rounded to TO and staged in LDS as
   // ys[m][n] (the K loop is done with it), then written out row by row in
   // 16-byte pieces, whole rows of the tile contiguous.  fp32 tiles go in two
   // halves of 128 rows, which is what fits.
-  constexpr int kPasses = sizeof(TS) == 4 ? 2 : 1;
+  constexpr int kPasses = sizeof(TO) == 4 ? 2 : 1;
   constexpr int kPassRows = kBM / kPasses;
-  constexpr int kPiece = 16 / static_cast<int>(sizeof(TS)); // elements per 16 bytes
+  constexpr int kPiece = 16 / static_cast<int>(sizeof(TO)); // elements per 16 bytes
   constexpr int kOutStride = kBN + kOutPad;
-  TS* ys = reinterpret_cast<TS*>(smem);
+  TO* ys = reinterpret_cast<TO*>(smem);
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
     __syncthreads(); // LDS is free: K loop (pass 0) or the previous half is done
@@ -432,11 +451,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
       const int quad = lane >> 4;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        TS* yrow = ys + ((wm * 64) % kPassRows + j * 16 + col) * kOutStride +
+        TO* yrow = ys + ((wm * 64) % kPassRows + j * 16 + col) * kOutStride +
             wn * 16 * NT + 4 * quad;
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
-          if constexpr (sizeof(TS) == 4) {
+          if constexpr (sizeof(TO) == 4) {
             float4 v = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
             if (!p.valid) {
               v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -444,8 +463,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
             *reinterpret_cast<float4*>(yrow + 16 * i) = v;
           } else {
             uint2 packed;
-            packed.x = pack2<TS>(acc[i][j][0], acc[i][j][1]);
-            packed.y = pack2<TS>(acc[i][j][2], acc[i][j][3]);
+            packed.x = pack2<TO>(acc[i][j][0], acc[i][j][1]);
+            packed.y = pack2<TO>(acc[i][j][2], acc[i][j][3]);
             if (!p.valid) {
               packed = make_uint2(0u, 0u);
             }
@@ -470,10 +489,10 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(const QmmArgs a, c
         if (mr >= M - m0 || m >= M || n >= N) {
           continue;
         }
-        const TS* src = ys + r * kOutStride + c * kPiece;
+        const TO* src = ys + r * kOutStride + c * kPiece;
         const size_t orow =
             GROUPED ? static_cast<size_t>(a.group_perm[row0 + mr]) : static_cast<size_t>(m);
-        TS* dst = p.out + orow * N + n;
+        TO* dst = p.out + orow * N + n;
         if (vec_ok && n + kPiece <= N) {
           *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
         } else {
@@ -532,13 +551,13 @@ int choose_nt(int M, int N, int L) {
   return best;
 }
 
-template <typename T, typename TS, int BITS, int NT, bool GROUPED>
-int launch_variant(const QmmArgs& a, int gs_shift, dim3 grid, hipStream_t s) {
+template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED>
+int launch_variant(const QmmArgs& a, int gs_shift, dim3 grid, hipStream_t s, int k_splits = 1) {
   constexpr size_t smem = qmm_smem_bytes<NT>();
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
-  auto kern = qmm_t_mfma_kernel<T, TS, BITS, NT, GROUPED>;
+  auto kern = qmm_t_mfma_kernel<T, TS, TO, BITS, NT, GROUPED>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -547,7 +566,7 @@ int launch_variant(const QmmArgs& a, int gs_shift, dim3 grid, hipStream_t s) {
         static_cast<int>(smem)));
     configured = true;
   }
-  kern<<<grid, kThreads, smem, s>>>(a, gs_shift);
+  kern<<<grid, kThreads, smem, s>>>(a, gs_shift, k_splits);
   MLXROCM_HIP_TRY(hipGetLastError());
   return static_cast<int>(MLXROCM_OK);
 }
@@ -577,26 +596,131 @@ int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
       constexpr int B = decltype(bval)::value;
       switch (nt) {
         case 5:
-          return launch_variant<T, T, B, 5, false>(a, gs_shift, grid, s);
+          return launch_variant<T, T, T, B, 5, false>(a, gs_shift, grid, s);
         case 6:
-          return launch_variant<T, T, B, 6, false>(a, gs_shift, grid, s);
+          return launch_variant<T, T, T, B, 6, false>(a, gs_shift, grid, s);
         default:
-          return launch_variant<T, T, B, 7, false>(a, gs_shift, grid, s);
+          return launch_variant<T, T, T, B, 7, false>(a, gs_shift, grid, s);
       }
     });
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
 }
 
-// fp32 operands: `a.x` already points at the [hi | lo | hi] bf16 image of x
-// (split_x_for_mfma) and a.x_batch_stride counts its elements (M * 3 K).
-int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s) {
+// How many ranges to cut K into so that a launch with few tiles still fills the
+// compute units (1 = no split): only for a single problem, and every range
+// keeps at least eight steps.
+int qmm_mfma_k_splits(int M, int N, int K, int L) {
+  if (L != 1) {
+    return 1;
+  }
+  const long cus = compute_units();
+  const long tiles = static_cast<long>((M + kBM - 1) / kBM) * ((N + 32 * 7 - 1) / (32 * 7));
+  const long steps = K / kBK;
+  long s = cus / tiles;
+  if (s > steps / 8) {
+    s = steps / 8;
+  }
+  if (s > 8) {
+    s = 8;
+  }
+  return s < 2 ? 1 : static_cast<int>(s);
+}
+
+// 16-bit operands with K cut into k_splits ranges: `a.out` points at k_splits
+// fp32 planes of M x N (reduce_k_splits adds them up into y).
+int launch_qmm_mfma_ksplit(
+    const QmmArgs& a,
+    int gs,
+    int bits,
+    int dtype,
+    int k_splits,
+    hipStream_t s) {
   constexpr int kNT = 7;
   const int gs_shift = shift_of(gs);
-  const dim3 grid((a.N + 32 * kNT - 1) / (32 * kNT), (a.M + kBM - 1) / kBM, a.L);
+  const dim3 grid((a.N + 32 * kNT - 1) / (32 * kNT), (a.M + kBM - 1) / kBM, k_splits);
+  auto run = [&](auto tval) -> int {
+    using T = decltype(tval);
+    return dispatch_bits(bits, [&](auto bval) {
+      constexpr int B = decltype(bval)::value;
+      return launch_variant<T, T, float, B, kNT, false>(a, gs_shift, grid, s, k_splits);
+    });
+  };
+  return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
+}
+
+namespace {
+
+template <typename TO>
+__global__ __launch_bounds__(256) void reduce_k_splits_kernel(
+    const float* partial,
+    TO* out,
+    size_t n,
+    int k_splits) {
+  const size_t i = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i >= n) {
+    return;
+  }
+  if (i + 4 <= n) {
+    float4 acc = *reinterpret_cast<const float4*>(partial + i);
+    for (int z = 1; z < k_splits; ++z) {
+      const float4 v = *reinterpret_cast<const float4*>(partial + z * n + i);
+      acc.x += v.x;
+      acc.y += v.y;
+      acc.z += v.z;
+      acc.w += v.w;
+    }
+    if constexpr (sizeof(TO) == 4) {
+      *reinterpret_cast<float4*>(out + i) = acc;
+    } else {
+      uint2 packed;
+      packed.x = pack2<TO>(acc.x, acc.y);
+      packed.y = pack2<TO>(acc.z, acc.w);
+      *reinterpret_cast<uint2*>(out + i) = packed;
+    }
+  } else {
+    for (size_t e = i; e < n; ++e) {
+      float acc = 0.0f;
+      for (int z = 0; z < k_splits; ++z) {
+        acc += partial[z * n + e];
+      }
+      out[e] = static_cast<TO>(acc);
+    }
+  }
+}
+
+} // namespace
+
+// y = sum of the k_splits fp32 planes (n = M * N elements each, a multiple of 4
+// apart); y must be 16-byte aligned.
+int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int dtype, hipStream_t s) {
+  const size_t blocks = (n / 4 + 1 + 255) / 256;
+  if (blocks > 0x7fffffffull) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmm] output too large for the split-K reduction");
+  }
+  const float* p = static_cast<const float*>(partial);
+  const unsigned g = static_cast<unsigned>(blocks);
+  if (dtype == MLXROCM_FLOAT32) {
+    reduce_k_splits_kernel<float><<<g, 256, 0, s>>>(p, static_cast<float*>(out), n, k_splits);
+  } else if (dtype == MLXROCM_BFLOAT16) {
+    reduce_k_splits_kernel<bf16_t><<<g, 256, 0, s>>>(p, static_cast<bf16_t*>(out), n, k_splits);
+  } else {
+    reduce_k_splits_kernel<f16_t><<<g, 256, 0, s>>>(p, static_cast<f16_t*>(out), n, k_splits);
+  }
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return MLXROCM_OK;
+}
+
+// fp32 operands: `a.x` already points at the [hi | lo | hi] bf16 image of x
+// (split_x_for_mfma) and a.x_batch_stride counts its elements (M * 3 K).
+int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s, int k_splits) {
+  constexpr int kNT = 7;
+  const int gs_shift = shift_of(gs);
+  const dim3 grid(
+      (a.N + 32 * kNT - 1) / (32 * kNT), (a.M + kBM - 1) / kBM, k_splits > 1 ? k_splits : a.L);
   return dispatch_bits(bits, [&](auto bval) {
     constexpr int B = decltype(bval)::value;
-    return launch_variant<bf16_t, float, B, kNT, false>(a, gs_shift, grid, s);
+    return launch_variant<bf16_t, float, float, B, kNT, false>(a, gs_shift, grid, s, k_splits);
   });
 }
 
@@ -663,7 +787,7 @@ int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipSt
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
       constexpr int B = decltype(bval)::value;
-      return launch_variant<T, T, B, kNT, true>(a, gs_shift, grid, s);
+      return launch_variant<T, T, T, B, kNT, true>(a, gs_shift, grid, s);
     });
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
