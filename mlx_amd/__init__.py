@@ -2,6 +2,7 @@
 (gfx950): ``quantize`` / ``dequantize`` / ``quantized_matmul`` / ``gather_qmm``
 with the reference's operator names and semantics, backed by hand-written HIP
 kernels through the C ABI declared in ``include/mlx_rocm_qmm.h``."""
+from . import nn
 from .ops import dequantize, gather_qmm, quantize, quantized_matmul
 
-__all__ = ["quantize", "dequantize", "quantized_matmul", "gather_qmm"]
+__all__ = ["quantize", "dequantize", "quantized_matmul", "gather_qmm", "nn"]

@@ -1,0 +1,162 @@
+"""Callers of the quantized-matmul path: the layers of
+``python/mlx/nn/layers/quantized.py`` (``QuantizedLinear`` :205-307,
+``QuantizedEmbedding`` :103-202, ``quantize`` :27-100) over this package's
+operators.
+
+The host module system is ``torch.nn`` (torch is the device-memory plumbing of
+this package): a quantized layer keeps ``weight`` (uint32 codes), ``scales`` and
+``biases`` as buffers -- frozen, as in MLX -- and an optional trainable-free
+``bias``.  Only ``mode="affine"`` exists here.
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable, Optional, Union
+
+import torch
+
+from . import ops
+
+__all__ = ["QuantizedLinear", "QuantizedEmbedding", "quantize"]
+
+
+def _defaults_for_mode(mode: str, group_size: Optional[int], bits: Optional[int]):
+    # python/mlx/nn/layers/quantized.py:12-24
+    if mode != "affine":
+        raise ValueError(
+            f"[quantize] quantization mode '{mode}' is not available; only 'affine' is"
+        )
+    return (64 if group_size is None else group_size, 4 if bits is None else bits)
+
+
+class QuantizedLinear(torch.nn.Module):
+    """``y = quantized_matmul(x, weight, scales, biases, transpose=True) + bias``."""
+
+    def __init__(self, input_dims: int, output_dims: int, bias: bool = True,
+                 group_size: Optional[int] = None, bits: Optional[int] = None,
+                 mode: str = "affine", device=None, dtype=torch.float32):
+        super().__init__()
+        self.group_size, self.bits = _defaults_for_mode(mode, group_size, bits)
+        self.mode = mode
+        device = torch.device("cuda:0") if device is None else torch.device(device)
+        scale = math.sqrt(1.0 / input_dims)
+        weight = (torch.rand((output_dims, input_dims), device=device) * 2 - 1) * scale
+        self._set_quantized(weight.to(dtype))
+        self.register_buffer(
+            "bias", torch.zeros((output_dims,), device=device, dtype=dtype) if bias else None)
+
+    def _set_quantized(self, weight: torch.Tensor) -> None:
+        wq, scales, biases = ops.quantize(weight, self.group_size, self.bits, self.mode)
+        for name, t in (("weight", wq), ("scales", scales), ("biases", biases)):
+            if name in self._buffers:
+                self._buffers[name] = t
+            else:
+                self.register_buffer(name, t)
+
+    def extra_repr(self) -> str:
+        out_dims, in_dims = self.weight.shape
+        in_dims = (in_dims * 32) // self.bits
+        return (f"input_dims={in_dims}, output_dims={out_dims}, bias={self.bias is not None}, "
+                f"group_size={self.group_size}, bits={self.bits}, mode={self.mode}")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        y = ops.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                                 group_size=self.group_size, bits=self.bits, mode=self.mode)
+        if self.bias is not None:
+            y = y + self.bias
+        return y
+
+    @classmethod
+    def from_linear(cls, linear_layer, group_size: Optional[int] = None,
+                    bits: Optional[int] = None, mode: str = "affine") -> "QuantizedLinear":
+        output_dims, input_dims = linear_layer.weight.shape
+        w = linear_layer.weight.detach()
+        ql = cls(input_dims, output_dims, False, group_size, bits, mode,
+                 device=w.device, dtype=w.dtype)
+        ql._set_quantized(w)
+        if getattr(linear_layer, "bias", None) is not None:
+            ql._buffers["bias"] = linear_layer.bias.detach()
+        return ql
+
+
+class QuantizedEmbedding(torch.nn.Module):
+    """Embedding with a quantized table: a lookup dequantizes the selected rows;
+    ``as_linear`` uses the table as an output projection (tied weights)."""
+
+    def __init__(self, num_embeddings: int, dims: int, group_size: Optional[int] = None,
+                 bits: Optional[int] = None, mode: str = "affine", device=None,
+                 dtype=torch.float32):
+        super().__init__()
+        self.group_size, self.bits = _defaults_for_mode(mode, group_size, bits)
+        self.mode = mode
+        self.num_embeddings, self.dims = num_embeddings, dims
+        device = torch.device("cuda:0") if device is None else torch.device(device)
+        weight = torch.randn((num_embeddings, dims), device=device) * math.sqrt(1.0 / dims)
+        self._set_quantized(weight.to(dtype))
+
+    _set_quantized = QuantizedLinear._set_quantized
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        # torch cannot index uint32 tensors: gather the rows through an int32 view
+        rows = self.weight.view(torch.int32)[x].view(torch.uint32)
+        return ops.dequantize(rows, self.scales[x], self.biases[x],
+                              group_size=self.group_size, bits=self.bits, mode=self.mode)
+
+    def as_linear(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                                    group_size=self.group_size, bits=self.bits, mode=self.mode)
+
+    def extra_repr(self) -> str:
+        return (f"{self.num_embeddings}, {self.dims}, group_size={self.group_size}, "
+                f"bits={self.bits}, mode={self.mode}")
+
+    @classmethod
+    def from_embedding(cls, embedding_layer, group_size: Optional[int] = None,
+                       bits: Optional[int] = None, mode: str = "affine") -> "QuantizedEmbedding":
+        num, dims = embedding_layer.weight.shape
+        w = embedding_layer.weight.detach()
+        ql = cls(num, dims, group_size, bits, mode, device=w.device, dtype=w.dtype)
+        ql._set_quantized(w)
+        return ql
+
+
+def _to_quantized(m, **kwargs):
+    if isinstance(m, torch.nn.Linear):
+        return QuantizedLinear.from_linear(m, **kwargs)
+    if isinstance(m, torch.nn.Embedding):
+        return QuantizedEmbedding.from_embedding(m, **kwargs)
+    return None
+
+
+def quantize(model: torch.nn.Module, group_size: Optional[int] = None,
+             bits: Optional[int] = None, *, mode: str = "affine",
+             quantize_input: bool = False,
+             class_predicate: Optional[Callable[[str, torch.nn.Module], Union[bool, dict]]] = None):
+    """Replace, in place, the ``Linear`` and ``Embedding`` leaves of ``model`` that
+    the predicate accepts by their quantized counterparts (``nn.quantize``).
+    ``class_predicate(path, module)`` returns a bool or a dict of parameters for
+    the conversion."""
+    if quantize_input:
+        raise ValueError("[quantize] quantize_input needs an fp quantization mode")
+    _defaults_for_mode(mode, group_size, bits)
+    quantizable = lambda m: isinstance(m, (torch.nn.Linear, torch.nn.Embedding))  # noqa: E731
+    class_predicate = class_predicate or (lambda _, m: quantizable(m))
+    for path, parent in list(model.named_modules()):
+        for name, child in list(parent.named_children()):
+            if len(list(child.children())) != 0:
+                continue  # not a leaf
+            full = f"{path}.{name}" if path else name
+            decision = class_predicate(full, child)
+            if not decision:
+                continue
+            if not quantizable(child):
+                raise ValueError(f"Unable to quantize model of type {type(child)}")
+            if isinstance(decision, bool):
+                kwargs = {"group_size": group_size, "bits": bits, "mode": mode}
+            elif isinstance(decision, dict):
+                kwargs = dict(decision)
+            else:
+                raise ValueError("``class_predicate`` must return a bool or a dict of "
+                                 "parameters to pass to ``to_quantized``")
+            setattr(parent, name, _to_quantized(child, **kwargs))
+    return model
