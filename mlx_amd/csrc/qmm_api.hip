@@ -240,7 +240,10 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   //               over the wavefronts of a workgroup) beyond;
   //   9..16 rows  the wide kernel;
   //   17..32 rows the 64-row LDS-staged kernel.
-  if (a.M >= 3 && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
+  //   1..2 rows   of a width the row-streaming GEMV does not cover: the wide
+  //               kernel as well.
+  const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype);
+  if (few_rows && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
     const bool gemv_better = a.M <= 8 && a.K <= 8192 && qmv_mfma_supported(a, gs, bits, dtype);
     if (!gemv_better) {
       return launch_qmv_wide(a, gs, bits, dtype, s);
