@@ -73,13 +73,37 @@ __global__ __launch_bounds__(kQuantBlock) void affine_quantize_kernel(
     bias = edge;
   }
 
+  // The eight quotients (v - bias) / scale share their divisor.  The correctly
+  // rounded fp32 division is a reciprocal refined once, then per numerator
+  // q = a r, two residual corrections q += (a - scale q) r -- the compiler's own
+  // expansion without its range scaling, which only acts on operands far outside
+  // what occurs here (|scale| in [1e-7, 1e38), quotients far from overflow; a
+  // numerator small enough to be scaled gives a quotient that rounds to 0 either
+  // way).  Groups with a non-finite edge take the plain division.
   uint64_t packed = 0;
+  const bool regular = fabsf(edge) < 3.0e38f && fabsf(scale) >= 1e-7f; // false for NaN
+  if (regular) {
+    float r = __builtin_amdgcn_rcpf(scale);
+    r = __builtin_fmaf(__builtin_fmaf(-scale, r, 1.0f), r, r);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    float q = rintf((v[i] - bias) / scale);
-    q = (q < 0.0f) ? 0.0f : q;
-    q = (n_bins < q) ? n_bins : q;
-    packed |= static_cast<uint64_t>(static_cast<uint32_t>(q)) << (i * BITS);
+    for (int i = 0; i < 8; ++i) {
+      const float a = v[i] - bias;
+      float q = a * r;
+      q = __builtin_fmaf(__builtin_fmaf(-scale, q, a), r, q);
+      q = __builtin_fmaf(__builtin_fmaf(-scale, q, a), r, q);
+      q = rintf(q);
+      q = (q < 0.0f) ? 0.0f : q;
+      q = (n_bins < q) ? n_bins : q;
+      packed |= static_cast<uint64_t>(static_cast<uint32_t>(q)) << (i * BITS);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float q = rintf((v[i] - bias) / scale);
+      q = (q < 0.0f) ? 0.0f : q;
+      q = (n_bins < q) ? n_bins : q;
+      packed |= static_cast<uint64_t>(static_cast<uint32_t>(q)) << (i * BITS);
+    }
   }
 
   if (active && (threadIdx.x % LPG) == 0) {

@@ -120,3 +120,34 @@ def test_quantize_batched_and_empty(oracle, gpu):
     e = torch.zeros((0, 64), dtype=torch.float32, device=gpu)
     wq, s, b = mlx_amd.quantize(e)
     assert wq.shape == (0, 8) and s.shape == (0, 1)
+
+
+@pytest.mark.parametrize("bits", (2, 4, 5, 8))
+def test_quantize_division_corner_magnitudes(oracle, gpu, bits):
+    """Every code is a correctly rounded fp32 quotient rounded to an integer: run
+    many groups whose quotients sit on or next to the rounding ties (values on a
+    half-integer grid of the scale), at magnitudes from 1e-30 to 1e30, with
+    heavy tails, and with infinities / NaNs in some groups."""
+    g = torch.Generator().manual_seed(bits)
+    n_bins = (1 << bits) - 1
+    rows = []
+    for exp in (-30, -20, -7, -3, 0, 4, 20, 30):
+        base = torch.rand((64, 64), generator=g) * 2 - 1
+        # half-integer grid: quotients k + 0.5 exactly where representable
+        grid = (torch.randint(0, 2 * n_bins + 1, (64, 64), generator=g).float() / 2) / n_bins - 0.5
+        tails = torch.distributions.StudentT(2.0).sample((64, 64)).clamp(-1e4, 1e4) * 0.01
+        rows += [base * 10.0 ** exp, grid * 10.0 ** exp, tails * 10.0 ** exp]
+    w = torch.cat(rows).float()
+    _check_quantize(oracle, gpu, w, 64, bits)
+    _check_quantize(oracle, gpu, w.reshape(-1, 128), 32, bits)
+    # non-finite members: the group is garbage in the reference too, but it must
+    # be the same garbage wherever the reference's result is well defined
+    w2 = w[:64].clone()
+    w2[3, 5] = float("inf")
+    w2[7, 9] = float("-inf")
+    ref = oracle.quantize(w2, 64, bits)
+    got = mlx_amd.quantize(w2.to(gpu), 64, bits)
+    clean = torch.ones(64, dtype=torch.bool)
+    clean[3] = clean[7] = False
+    for r, t in zip(ref, got):
+        assert bits_equal(r[clean], t.cpu()[clean])
