@@ -29,7 +29,7 @@ BF16_PEAK_TFLOPS = 2500.0
 # a copy of known size (profiles/qmv_stream_4bit_g64_bf16_14336x4096.md and
 # profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md).
 QMV_TRAFFIC_BYTES = 33221941
-QMM_T_TRAFFIC_BYTES = 258712822
+QMM_T_TRAFFIC_BYTES = 258695787
 
 N, K = 14336, 4096
 BITS, GS = 4, 64
