@@ -105,6 +105,14 @@ int mlxrocm_affine_dequantize(
  * [L, M, N].  w_batch_stride (uint32 words) and sb_batch_stride (elements) are
  * 0 when one weight matrix is shared by every batch (w.ndim() == 2 in MLX).
  * The kernel is picked from M, N, K, bits, group_size and dtype.
+ *
+ * Two kinds of call keep device scratch inside the library -- one buffer per
+ * stream, allocated (hipMalloc) or grown on the first call that needs it and
+ * kept until the process ends: float32 operands with M > 8 (x is split into two
+ * bfloat16 parts for the matrix cores) and 16-bit calls whose tile grid would
+ * leave compute units idle (K is split; fp32 partial results).  Every other
+ * call allocates nothing.  A call that needs a larger buffer than the stream
+ * holds synchronizes that stream before replacing it.
  */
 int mlxrocm_qmm(
     const void* x,
@@ -136,9 +144,13 @@ int mlxrocm_qmm(
  * n_experts matrices w_expert_stride words (sb_expert_stride elements) apart, so
  * a sliced expert stack needs no copy.  out is a dense [n_indices, M, N].
  * rhs_sorted != 0 promises rhs_indices is non-decreasing (right_sorted_).
- * workspace must hold mlxrocm_gather_qmm_workspace_size(...) bytes (may be NULL
- * when that is 0).  Index values are range-checked on the device; an
- * out-of-range pair produces zeros instead of a wild access.
+ * workspace (4-byte aligned device memory) must hold
+ * mlxrocm_gather_qmm_workspace_size(...) bytes and may be NULL when that is 0:
+ * with many index pairs per expert (M == 1, 16-bit types) the pairs are sorted
+ * by expert into it and every expert's weights are read once for all its rows;
+ * without a workspace the call falls back to one product per pair.  Index
+ * values are range-checked on the device; an out-of-range pair produces zeros
+ * instead of a wild access.
  */
 int mlxrocm_gather_qmm(
     const void* x,

@@ -118,7 +118,7 @@ struct StreamShape {
   static constexpr int kGroupChunks = 64 * GS / kChunkCodes;
   static constexpr int kChunksPerWave = kGroupChunks < kMaxChunks ? kGroupChunks : kMaxChunks;
   // rows per wave: 8 KiB of packed weights in flight per wave either way
-  static constexpr int kRowsPerWave = 8 / kChunksPerWave;
+  static constexpr int kRowsPerWave = 4 / kChunksPerWave;
   static_assert(kChunksPerWave >= 1, "shape");
 };
 
