@@ -191,3 +191,42 @@ def test_gather_qmm_grouped_matches_ungrouped(gpu):
     diff = (grouped.float() - single.float()).abs().max()
     scale = single.float().abs().max()
     assert float(diff) <= 2 ** -7 * float(scale)
+
+
+def test_gather_qmm_full_size_moe_permutation_invariant(oracle, gpu):
+    """8 experts of [14336, 4096], 4-bit group 64, T = 2048 tokens routed top-2
+    (seeded): the grouped GEMM gives, for every index pair, a row that depends on
+    that pair only -- so the run on expert-sorted pairs must reproduce the
+    unsorted run bit for bit after un-permuting -- and sampled rows agree with
+    the CPU oracle."""
+    E, N, K, T = 8, 14336, 4096, 2048
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn((E, N, K), generator=g) * 0.02).to(torch.bfloat16)
+    wq, s, b = mlx_amd.quantize(w.to(gpu), 64, 4)
+    del w
+    x = torch.randn((T, 1, 1, K), generator=g).to(torch.bfloat16)
+    idx = torch.randint(0, E, (T, 2), generator=torch.Generator().manual_seed(0))
+    gx, gidx = x.to(gpu), idx.to(gpu)
+    unsorted = mlx_amd.gather_qmm(gx, wq, s, b, rhs_indices=gidx, transpose=True,
+                                  group_size=64, bits=4)
+    assert unsorted.shape == (T, 2, 1, N)
+    flat = gidx.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    xs = gx.reshape(T, 1, K)[order // 2].contiguous()
+    ys = mlx_amd.gather_qmm(xs, wq, s, b, rhs_indices=flat[order].contiguous(),
+                            transpose=True, group_size=64, bits=4, sorted_indices=True)
+    resorted = ys[torch.argsort(order)].reshape(T, 2, 1, N)
+    assert torch.equal(unsorted.view(torch.int16), resorted.view(torch.int16))
+    # oracle on a few pairs
+    cq = [t.cpu() for t in (wq, s, b)]
+    for t, j in ((0, 0), (777, 1), (2047, 1)):
+        e = int(idx[t, j])
+        ref = oracle.qmm(x[t].reshape(1, K), cq[0][e], cq[1][e], cq[2][e], True, 64, 4)
+        w_hat = exact_affine_weights(cq[0][e], cq[1][e], cq[2][e], 64, 4)
+        exact = x[t].reshape(1, K).double() @ w_hat.T
+        got = unsorted[t, j].cpu().double()
+        tol = matmul_tolerance(torch.bfloat16, K, x[t], w_hat) + float(
+            (ref.double() - exact).abs().max())
+        assert float((got - ref.double()).abs().max()) <= tol
+        assert float((got - exact).abs().max()) <= exact_tolerance(
+            torch.bfloat16, K, x[t], w_hat, exact)
