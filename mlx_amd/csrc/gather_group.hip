@@ -8,8 +8,10 @@
 //   count    one atomic per pair into counts[expert]; pairs with an index out of
 //            range are left out and their output rows are zero-filled here;
 //   plan     one workgroup: exclusive scan of the counts -> first sorted
-//            position of every expert, and the list of 256-row tiles
-//            {expert, first position, rows}; the tile count stays on the device;
+//            position of every expert, and the list of tiles {expert, first
+//            position, rows} of up to tile_rows rows (256 for the tile GEMM, 32
+//            for the few-row kernel when the groups are small); the tile count
+//            stays on the device;
 //   scatter  perm[position] = pair, position handed out by a per-expert cursor.
 // The order inside an expert's run is arbitrary; every output row depends on
 // its own x row only, so the result does not depend on it.
@@ -19,7 +21,6 @@ namespace mlxrocm {
 
 namespace {
 
-constexpr int kTileRows = 256;
 constexpr int kMaxExperts = 4096; // plan kernel keeps the counts in LDS
 
 template <typename T>
@@ -50,6 +51,7 @@ __global__ __launch_bounds__(256) void group_count_kernel(
 
 __global__ __launch_bounds__(256) void group_plan_kernel(
     int n_experts,
+    int tile_rows,
     const int32_t* counts,
     int32_t* offsets,
     int32_t* tiles,
@@ -68,7 +70,7 @@ __global__ __launch_bounds__(256) void group_plan_kernel(
       first_pos[e] = pos;
       first_tile[e] = tile;
       pos += cnt[e];
-      tile += (cnt[e] + kTileRows - 1) / kTileRows;
+      tile += (cnt[e] + tile_rows - 1) / tile_rows;
     }
     *n_tiles = tile;
   }
@@ -77,10 +79,10 @@ __global__ __launch_bounds__(256) void group_plan_kernel(
     offsets[e] = first_pos[e];
     const int c = cnt[e];
     int t = first_tile[e];
-    for (int r = 0; r < c; r += kTileRows, ++t) {
+    for (int r = 0; r < c; r += tile_rows, ++t) {
       tiles[3 * t + 0] = e;
       tiles[3 * t + 1] = first_pos[e] + r;
-      tiles[3 * t + 2] = (c - r < kTileRows) ? c - r : kTileRows;
+      tiles[3 * t + 2] = (c - r < tile_rows) ? c - r : tile_rows;
     }
   }
 }
@@ -119,9 +121,9 @@ size_t align_up(size_t v, size_t a) {
 
 } // namespace
 
-int gather_group_max_tiles(int n_indices, int n_experts) {
+int gather_group_max_tiles(int n_indices, int n_experts, int tile_rows) {
   // every expert may end on a partial tile
-  return (n_indices + kTileRows - 1) / kTileRows + n_experts;
+  return (n_indices + tile_rows - 1) / tile_rows + n_experts;
 }
 
 size_t gather_group_workspace_bytes(int n_indices, int n_experts) {
@@ -129,12 +131,13 @@ size_t gather_group_workspace_bytes(int n_indices, int n_experts) {
     return 0;
   }
   const size_t ints = static_cast<size_t>(3) * n_experts + 4 +
-      static_cast<size_t>(3) * gather_group_max_tiles(n_indices, n_experts) + n_indices;
+      static_cast<size_t>(3) * gather_group_max_tiles(n_indices, n_experts, kGroupSmallTile) +
+      n_indices; // sized for the smaller tile
   return align_up(ints * sizeof(int32_t), 256);
 }
 
 // Fills the workspace and points the grouped-mode fields of `a` into it.
-int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s) {
+int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, hipStream_t s) {
   const int E = a.n_experts;
   const int n = a.L;
   int32_t* ws = static_cast<int32_t*>(workspace);
@@ -143,7 +146,7 @@ int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s) {
   int32_t* offsets = cursor + E;
   int32_t* n_tiles = offsets + E;
   int32_t* tiles = n_tiles + 4;
-  int32_t* perm = tiles + 3 * gather_group_max_tiles(n, E);
+  int32_t* perm = tiles + 3 * gather_group_max_tiles(n, E, tile_rows);
 
   // counts and cursors start at zero (a fill kernel, so that the sequence can be
   // captured into a graph)
@@ -160,7 +163,7 @@ int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s) {
         static_cast<f16_t*>(a.out), a.N);
   }
   MLXROCM_HIP_TRY(hipGetLastError());
-  group_plan_kernel<<<1, 256, 0, s>>>(E, counts, offsets, tiles, n_tiles);
+  group_plan_kernel<<<1, 256, 0, s>>>(E, tile_rows, counts, offsets, tiles, n_tiles);
   MLXROCM_HIP_TRY(hipGetLastError());
   group_scatter_kernel<<<blocks, 256, 0, s>>>(
       a.lhs_indices, a.rhs_indices, n, a.x_batches, E, offsets, cursor, perm);
@@ -169,6 +172,7 @@ int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s) {
   a.group_tiles = tiles;
   a.group_perm = perm;
   a.group_ntiles = n_tiles;
+  a.group_tile_rows = tile_rows;
   return MLXROCM_OK;
 }
 

@@ -386,7 +386,7 @@ bool group_gather(
   if (static_cast<int64_t>(x_batches) * x_batch_stride + K >= (int64_t(1) << 32)) {
     return false;
   }
-  if (gather_group_max_tiles(n_indices, n_experts) > 65535) {
+  if (gather_group_max_tiles(n_indices, n_experts, kGroupSmallTile) > 65535) {
     return false;
   }
   return gather_group_workspace_bytes(n_indices, n_experts) > 0;
@@ -486,11 +486,16 @@ extern "C" int mlxrocm_gather_qmm(
     if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) {
       return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qmm] workspace must be 4-byte aligned");
     }
-    rc = launch_gather_group(a, dtype, workspace, s);
+    // small groups (at most 64 pairs per expert on average) go to the few-row
+    // kernel in 32-row tiles, larger ones to the 256-row tile GEMM
+    const bool small = K % 128 == 0 &&
+        static_cast<int64_t>(n_indices) <= 64 * static_cast<int64_t>(n_experts);
+    rc = launch_gather_group(a, dtype, small ? kGroupSmallTile : kGroupLargeTile, workspace, s);
     if (rc != MLXROCM_OK) {
       return rc;
     }
-    return launch_qmm_mfma_grouped(a, group_size, bits, dtype, s);
+    return small ? launch_qmm_skinny_grouped(a, group_size, bits, dtype, s)
+                 : launch_qmm_mfma_grouped(a, group_size, bits, dtype, s);
   }
   // One grid z-slot per index pair; large index lists go in slices.
   constexpr int kMaxZ = 65535;

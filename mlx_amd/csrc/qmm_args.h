@@ -26,13 +26,14 @@ struct QmmArgs {
   int x_batches; // bounds for gathered indices
   int n_experts;
   // Grouped gather (M == 1): the index pairs sorted by expert and cut into tiles
-  // of up to 256 rows.  group_tiles holds {expert, first sorted position, rows}
+  // of up to group_tile_rows rows.  group_tiles holds {expert, first sorted position, rows}
   // per tile, group_perm maps a sorted position to its index pair, group_ntiles
   // points at the number of tiles (known on the device only).  All null
   // otherwise.
   const int32_t* group_tiles;
   const int32_t* group_perm;
   const int32_t* group_ntiles;
+  int group_tile_rows;
 };
 
 // Resolved operand pointers of problem l.  `valid` is false when a gathered
@@ -96,9 +97,12 @@ int launch_zero_fill(void* p, size_t bytes, hipStream_t s);
 
 // Grouping of gathered index pairs by expert (gather_group.hip) and the grouped
 // launch of the matrix-core GEMM over its tiles (qmm_mfma.hip).
+constexpr int kGroupLargeTile = 256; // rows per tile of the tile GEMM
+constexpr int kGroupSmallTile = 32;  // rows per tile of the few-row kernel
 size_t gather_group_workspace_bytes(int n_indices, int n_experts);
-int gather_group_max_tiles(int n_indices, int n_experts);
-int launch_gather_group(QmmArgs& a, int dtype, void* workspace, hipStream_t s);
+int gather_group_max_tiles(int n_indices, int n_experts, int tile_rows);
+int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, hipStream_t s);
+int launch_qmm_skinny_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 // fp32 operands on the bf16 matrix path: x is first split into bf16 high and
 // low parts (split_x_for_mfma into a buffer of split_x_bytes), then
 // launch_qmm_mfma_split runs with a.x pointing at that buffer.

@@ -782,7 +782,7 @@ int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipSt
   constexpr int kNT = 7;
   const int gs_shift = shift_of(gs);
   const dim3 grid(
-      (a.N + 32 * kNT - 1) / (32 * kNT), gather_group_max_tiles(a.L, a.n_experts), 1);
+      (a.N + 32 * kNT - 1) / (32 * kNT), gather_group_max_tiles(a.L, a.n_experts, kGroupLargeTile), 1);
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {

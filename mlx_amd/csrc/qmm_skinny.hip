@@ -1,20 +1,21 @@
-// qmm_skinny.hip -- transpose=true products with a few rows of x (3 <= M <= 32)
-// for 16-bit element types: batched decode and small expert groups.
+// qmm_skinny.hip -- transpose=true products with 17..32 rows of x for 16-bit
+// element types, and small expert groups of a gather (tiles of up to 32 rows).
 //
 //   y[M, N] = x[M, K] * dequant(W)[N, K]^T
 //
 // The weights are read once and the work is bound by that stream, so the
 // kernel is built around full-line coalesced fetches of the packed rows:
 // a workgroup of 256 threads (4 wavefronts) owns 64 rows of W and walks K in
-// steps of 256 codes.  Per step
-//   * every thread fetches two 32-code pieces (row r and row r + 32; eight
-//     consecutive lanes cover the 256 codes of a row, i.e. whole cache lines for
-//     4-bit codes and wider), three steps ahead of their use;
+// steps of 128 codes (52 KiB of LDS, so three workgroups share a compute unit
+// and hide each other's barrier and LDS latencies).  Per step
+//   * every thread fetches one 32-code piece (four consecutive lanes cover the
+//     128 codes of a row; consecutive steps use up the rest of the cache line),
+//     three steps ahead of its use;
 //   * the pieces are dequantized (fp32 fma(s, code, b), one rounding to T) into
 //     the idle LDS stage, next to the x tile of the step (M rows x 256);
 //   * wavefront w multiplies rows [16 w, 16 w + 16) of the tile with
 //     v_mfma_f32_16x16x32 (A = W rows, B = x rows), fp32 accumulators.
-// LDS rows are 256 elements + 8 of padding (528 bytes): the 16-byte fragment
+// LDS rows are 128 elements + 8 of padding (272 bytes): the 16-byte fragment
 // reads of 16 consecutive rows fall on distinct banks.
 #include "mfma_dequant.h"
 #include "qmm_args.h"
@@ -24,7 +25,7 @@ namespace mlxrocm {
 namespace {
 
 constexpr int kSkBN = 64;
-constexpr int kSkBK = 256;
+constexpr int kSkBK = 128;
 constexpr int kSkStride = kSkBK + 8; // elements per LDS row
 constexpr int kSkThreads = 256;
 constexpr int kSkAhead = 3; // packed-W fetch distance in steps
@@ -34,10 +35,10 @@ constexpr size_t skinny_smem_bytes() {
   return static_cast<size_t>(2) * (kSkBN + MROWS) * kSkStride * 2;
 }
 
-// MROWS: rows of x staged per step (8, 16 or 32; M <= MROWS).  With 8 rows the
-// MFMA's 16-row x operand reads every staged row twice (the upper half of the
-// result is discarded), which keeps two workgroups resident per compute unit.
-template <typename T, int BITS, int MROWS>
+// MROWS: rows of x staged per step (16 or 32; M <= MROWS).
+// GROUPED: blockIdx.y walks the 32-row tile list of a gather grouped by expert
+// (one x row per index pair, fetched and written back through the permutation).
+template <typename T, int BITS, int MROWS, bool GROUPED>
 __global__ __launch_bounds__(kSkThreads) void qmm_skinny_kernel(const QmmArgs a, const int gs_shift) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int kMRows = MROWS;
@@ -50,42 +51,72 @@ __global__ __launch_bounds__(kSkThreads) void qmm_skinny_kernel(const QmmArgs a,
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int M = a.M;
   const int N = a.N;
   const int K = a.K;
   const int n0 = blockIdx.x * kSkBN;
-  const QmmProblem<T> p = resolve_problem<T>(a, blockIdx.y);
+  int M = a.M;
+  int row0 = 0; // grouped: first sorted position of the tile
+  QmmProblem<T> p;
+  if constexpr (GROUPED) {
+    const int tile = blockIdx.y;
+    if (tile >= *a.group_ntiles) {
+      return; // the grid covers the worst-case tile count
+    }
+    const int e = a.group_tiles[3 * tile];
+    row0 = a.group_tiles[3 * tile + 1];
+    M = a.group_tiles[3 * tile + 2];
+    p.x = static_cast<const T*>(a.x);
+    p.w = reinterpret_cast<const uint8_t*>(a.w + static_cast<int64_t>(e) * a.w_batch_stride);
+    p.scales = static_cast<const T*>(a.scales) + static_cast<int64_t>(e) * a.sb_batch_stride;
+    p.biases = static_cast<const T*>(a.biases) + static_cast<int64_t>(e) * a.sb_batch_stride;
+    p.out = static_cast<T*>(a.out);
+    p.valid = true;
+  } else {
+    p = resolve_problem<T>(a, blockIdx.y);
+  }
 
   const int groups = K >> gs_shift;
   const int row_words = K / 32 * BITS;
   const int nk = K / kSkBK;
 
   // ---- loader roles ----
-  // W: thread covers piece (tid % 8) -- codes [32 piece, 32 piece + 32) of the
-  // step -- of tile rows tid / 8 and tid / 8 + 32.
-  const int piece = tid & 7;
-  const int wr0 = tid >> 3;
-  const uint32_t* wsrc[2];
-  const T* ssrc[2];
-  const T* bsrc[2];
+  // W: thread covers piece (tid % 4) -- codes [32 piece, 32 piece + 32) of the
+  // step -- of tile row tid / 4.
+  constexpr int kPieces = kSkBK / 32;              // pieces per row and step
+  constexpr int kWRows = kSkThreads / kPieces;     // rows covered by one pass
+  constexpr int kWPasses = kSkBN / kWRows;         // 1
+  const int piece = tid % kPieces;
+  const int wr0 = tid / kPieces;
+  const uint32_t* wsrc[kWPasses];
+  const T* ssrc[kWPasses];
+  const T* bsrc[kWPasses];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int n = n0 + wr0 + 32 * h;
+  for (int h = 0; h < kWPasses; ++h) {
+    const int n = n0 + wr0 + kWRows * h;
     const int row = n < N ? n : N - 1; // clamp: loads stay in bounds
     wsrc[h] = reinterpret_cast<const uint32_t*>(p.w) + static_cast<size_t>(row) * row_words +
         piece * BITS;
     ssrc[h] = p.scales + static_cast<size_t>(row) * groups;
     bsrc[h] = p.biases + static_cast<size_t>(row) * groups;
   }
-  // x: 32 sixteen-byte pieces per row and step; thread covers piece (tid % 32)
-  // of rows tid / 32 + 8 i.  Rows past M reread row M - 1 (never stored).
+  // x: 16 sixteen-byte pieces per row and step; thread covers piece (tid % 16)
+  // of rows tid / 16 + 16 i.  Rows past M reread row M - 1 (never stored).
   // (named registers: small arrays indexed inside lambdas end up in scratch)
-  constexpr int kXLoads = kMRows / 8; // 1, 2 or 4
-  const int xpiece = tid & 31;
-  const int xr0 = tid >> 5;
+  constexpr int kXPieces = kSkBK / 8;
+  constexpr int kXRows = kSkThreads / kXPieces;    // rows covered by one pass
+  constexpr int kXLoads = kMRows / kXRows;         // 1 or 2
+  static_assert(kXLoads >= 1 && kXLoads <= 4, "x staging shape");
+  const int xpiece = tid % kXPieces;
+  const int xr0 = tid / kXPieces;
   auto x_row_off = [&](int i) {
-    const int m = xr0 + 8 * i;
-    return static_cast<uint32_t>(m < M ? m : M - 1) * static_cast<uint32_t>(K) + xpiece * 8;
+    const int m = xr0 + kXRows * i;
+    const int mc = m < M ? m : M - 1;
+    if constexpr (GROUPED) {
+      const uint32_t pair = static_cast<uint32_t>(a.group_perm[row0 + mc]);
+      return a.lhs_indices[pair] * static_cast<uint32_t>(a.x_batch_stride) + xpiece * 8;
+    } else {
+      return static_cast<uint32_t>(mc) * static_cast<uint32_t>(K) + xpiece * 8;
+    }
   };
   const uint32_t xoff0 = x_row_off(0);
   const uint32_t xoff1 = x_row_off(1);
@@ -95,12 +126,12 @@ __global__ __launch_bounds__(kSkThreads) void qmm_skinny_kernel(const QmmArgs a,
   uint4 xq00, xq01, xq02, xq03, xq10, xq11, xq12, xq13, xq20, xq21, xq22, xq23;
 
   // packed W, scales and biases of the next kSkAhead steps
-  uint32_t wq[kSkAhead][2][BITS];
-  T sq[kSkAhead][2], bq[kSkAhead][2];
+  uint32_t wq[kSkAhead][kWPasses][BITS];
+  T sq[kSkAhead][kWPasses], bq[kSkAhead][kWPasses];
   auto fetch_w = [&](int slot, int step) {
     const int st = step < nk ? step : nk - 1; // past the end: refetch, never used
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < kWPasses; ++h) {
       const uint32_t* wp = wsrc[h] + st * (kSkBK / 32) * BITS;
 #pragma unroll
       for (int j = 0; j < BITS; ++j) {
@@ -127,23 +158,23 @@ __global__ __launch_bounds__(kSkThreads) void qmm_skinny_kernel(const QmmArgs a,
 #define SKINNY_STORE_X(stage, slot)                                              \
   do {                                                                           \
     T* xs__ = lds + (stage) * kStage + kWTile;                                   \
-    *reinterpret_cast<uint4*>(&xs__[(xr0 + 0) * kSkStride + xpiece * 8]) = xq##slot##0; \
+    *reinterpret_cast<uint4*>(&xs__[(xr0 + 0 * kXRows) * kSkStride + xpiece * 8]) = xq##slot##0; \
     if constexpr (kXLoads > 1) {                                                 \
-      *reinterpret_cast<uint4*>(&xs__[(xr0 + 8) * kSkStride + xpiece * 8]) = xq##slot##1; \
+      *reinterpret_cast<uint4*>(&xs__[(xr0 + 1 * kXRows) * kSkStride + xpiece * 8]) = xq##slot##1; \
     }                                                                            \
     if constexpr (kXLoads > 2) {                                                 \
-      *reinterpret_cast<uint4*>(&xs__[(xr0 + 16) * kSkStride + xpiece * 8]) = xq##slot##2; \
-      *reinterpret_cast<uint4*>(&xs__[(xr0 + 24) * kSkStride + xpiece * 8]) = xq##slot##3; \
+      *reinterpret_cast<uint4*>(&xs__[(xr0 + 2 * kXRows) * kSkStride + xpiece * 8]) = xq##slot##2; \
+      *reinterpret_cast<uint4*>(&xs__[(xr0 + 3 * kXRows) * kSkStride + xpiece * 8]) = xq##slot##3; \
     }                                                                            \
   } while (0)
 
   auto store_w = [&](int stage, int slot) {
     T* ws = lds + stage * kStage;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < kWPasses; ++h) {
       uint32_t dq[16];
       dequant32<T, BITS>(wq[slot][h], to_f32(sq[slot][h]), to_f32(bq[slot][h]), dq);
-      uint4* dst = reinterpret_cast<uint4*>(&ws[(wr0 + 32 * h) * kSkStride + piece * 32]);
+      uint4* dst = reinterpret_cast<uint4*>(&ws[(wr0 + kWRows * h) * kSkStride + piece * 32]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         dst[j] = make_uint4(dq[4 * j], dq[4 * j + 1], dq[4 * j + 2], dq[4 * j + 3]);
@@ -231,7 +262,9 @@ __global__ __launch_bounds__(kSkThreads) void qmm_skinny_kernel(const QmmArgs a,
     if (m >= M) {
       continue;
     }
-    T* yrow = p.out + static_cast<size_t>(m) * N;
+    const size_t orow =
+        GROUPED ? static_cast<size_t>(a.group_perm[row0 + m]) : static_cast<size_t>(m);
+    T* yrow = p.out + orow * N;
     float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -264,7 +297,7 @@ bool qmm_skinny_supported(const QmmArgs& a, int gs, int bits, int dtype, bool tr
   if (a.M < 1 || a.M > 32) {
     return false;
   }
-  // whole steps of 256 codes; 32-bit element offsets into x
+  // whole steps of 128 codes; 32-bit element offsets into x
   if (a.K % kSkBK != 0 || a.K < kSkBK) {
     return false;
   }
@@ -284,7 +317,7 @@ int launch_qmm_skinny(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t
       auto go = [&](auto mrv) -> int {
         constexpr int MR = decltype(mrv)::value;
         constexpr size_t smem = skinny_smem_bytes<MR>();
-        auto kern = qmm_skinny_kernel<T, B, MR>;
+        auto kern = qmm_skinny_kernel<T, B, MR, false>;
         static bool configured = false; // per instantiation
         if (!configured) {
           MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -297,7 +330,38 @@ int launch_qmm_skinny(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t
         MLXROCM_HIP_TRY(hipGetLastError());
         return static_cast<int>(MLXROCM_OK);
       };
-      return a.M <= 8 ? go(IntC<8>{}) : (a.M <= 16 ? go(IntC<16>{}) : go(IntC<32>{}));
+      return a.M <= 16 ? go(IntC<16>{}) : go(IntC<32>{});
+    });
+  };
+  return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
+}
+
+// Gather grouped by expert in 32-row tiles: `a` carries the tile list; one grid
+// row per possible tile, rows past the device-side tile count exit at once.
+int launch_qmm_skinny_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
+  const dim3 grid(
+      (a.N + kSkBN - 1) / kSkBN, gather_group_max_tiles(a.L, a.n_experts, kGroupSmallTile));
+  if (grid.y > 65535u) {
+    return fail(MLXROCM_UNSUPPORTED, "[gather_qmm] %d index pairs exceed the grid", a.L);
+  }
+  auto run = [&](auto tval) -> int {
+    using T = decltype(tval);
+    return dispatch_bits(bits, [&](auto bval) {
+      constexpr int B = decltype(bval)::value;
+      constexpr size_t smem = skinny_smem_bytes<kGroupSmallTile>();
+      auto kern = qmm_skinny_kernel<T, B, kGroupSmallTile, true>;
+      static bool configured = false; // per instantiation
+      if (!configured) {
+        MLXROCM_HIP_TRY(hipFuncSetAttribute(
+            reinterpret_cast<const void*>(kern),
+            hipFuncAttributeMaxDynamicSharedMemorySize,
+            static_cast<int>(smem)));
+        configured = true;
+      }
+      kern<<<grid, kSkThreads, smem, s>>>(a, gs_shift);
+      MLXROCM_HIP_TRY(hipGetLastError());
+      return static_cast<int>(MLXROCM_OK);
     });
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});

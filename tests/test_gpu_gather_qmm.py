@@ -230,3 +230,32 @@ def test_gather_qmm_full_size_moe_permutation_invariant(oracle, gpu):
         assert float((got - ref.double()).abs().max()) <= tol
         assert float((got - exact).abs().max()) <= exact_tolerance(
             torch.bfloat16, K, x[t], w_hat, exact)
+
+
+@pytest.mark.parametrize("bits,gs", ((4, 64), (5, 32), (8, 128)))
+def test_gather_qmm_small_groups(oracle, gpu, bits, gs):
+    """A few index pairs per expert (at most 64 on average): the pairs are
+    grouped into 32-row tiles for the few-row kernel.  One expert gets more than
+    one tile, one gets none; ragged N; x rows shared between pairs."""
+    E, N, K, T = 8, 200, 384, 100
+    dtype = torch.bfloat16
+    assert _grouped_ws_bytes(1, N, K, T, E, gs, bits) > 0
+    w = normal_weights((E, N, K), dtype, std=0.5)
+    wq, s, b = oracle.quantize(w, gs, bits)
+    X = 16
+    x = activations((X, 1, K), dtype)
+    g = torch.Generator().manual_seed(3)
+    rhs = torch.multinomial(torch.tensor([0.45, 0.0, 0.1, 0.1, 0.1, 0.1, 0.1, 0.05]), T,
+                            replacement=True, generator=g)
+    lhs = torch.randint(0, X, (T,), generator=g)
+    assert int((rhs == 0).sum()) > 32 and int((rhs == 1).sum()) == 0
+    gx, gwq, gsc, gb, glhs, grhs = _to(gpu, x, wq, s, b, lhs, rhs)
+    got = mlx_amd.gather_qmm(gx, gwq, gsc, gb, glhs, grhs, True, gs, bits).cpu()
+    ref = oracle.gather_qmm(x, wq, s, b, lhs, rhs, True, gs, bits)
+    w_hat = exact_affine_weights(wq, s, b, gs, bits)
+    exact = torch.einsum("tk,tnk->tn", x.reshape(X, K).double()[lhs], w_hat[rhs])
+    assert float((got.reshape(T, N).double() - exact).abs().max()) <= exact_tolerance(
+        dtype, K, x, w_hat, exact)
+    tol = matmul_tolerance(dtype, K, x, w_hat) + float(
+        (ref.reshape(T, N).double() - exact).abs().max())
+    assert float((got.double() - ref.double()).abs().max()) <= tol
