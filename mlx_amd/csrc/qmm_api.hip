@@ -238,19 +238,24 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   // Measured on gate/up and down projection shapes (4- and 8-bit):
   //   3..8 rows   the 32-row MFMA GEMV up to K = 8192, the wide kernel (K split
   //               over the wavefronts of a workgroup) beyond;
-  //   9..16 rows  the wide kernel;
-  //   17..32 rows the 64-row LDS-staged kernel.
+  //   9..16 rows  the 64-row LDS-staged kernel when N gives it enough
+  //               workgroups, the wide kernel otherwise;
+  //   17..32 rows the 64-row LDS-staged kernel;
   //   1..2 rows   of a width the row-streaming GEMV does not cover: the wide
   //               kernel as well.
   const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype);
-  if (few_rows && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
+  const bool staged = a.M > 16 || (a.M > 8 && a.N >= 8192);
+  if (few_rows && !staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
     const bool gemv_better = a.M <= 8 && a.K <= 8192 && qmv_mfma_supported(a, gs, bits, dtype);
     if (!gemv_better) {
       return launch_qmv_wide(a, gs, bits, dtype, s);
     }
   }
-  if (a.M > 16 && qmm_skinny_supported(a, gs, bits, dtype, transpose)) {
+  if (staged && qmm_skinny_supported(a, gs, bits, dtype, transpose)) {
     return launch_qmm_skinny(a, gs, bits, dtype, s);
+  }
+  if (staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
+    return launch_qmv_wide(a, gs, bits, dtype, s);
   }
   switch (choose_family(a.M, a.N, a.K, a.L, dtype, transpose)) {
     case Family::QmmT:
