@@ -320,11 +320,15 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   QMM_ROTATE_W();
   QMM_STORE_X(0, 0);
   QMM_STORE_W(0);
+  // same order as in the loop (x of one step, packed W, x of the next step): the
+  // compiler's wait counts at the loop head are the stricter of this path's and
+  // the back edge's, and a different order here makes every step wait for loads
+  // it has only just issued
   QMM_LOAD_X(0, kclamp(1));
+  QMM_LOAD_W(kclamp(1));
   if constexpr (kXSets == 2) {
     QMM_LOAD_X(1, kclamp(2));
   }
-  QMM_LOAD_W(kclamp(1));
   QMM_ROTATE_W();
   __syncthreads();
   read_b(0, 0, 0);
