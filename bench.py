@@ -256,6 +256,14 @@ def sweep(torch, mlx_amd, dev) -> list:
             matmul_case("cfg5", 1, 11008, 4096, bits, 32, dtype)
             matmul_case("cfg5", 1024, 11008, 4096, bits, 32, dtype)
             matmul_case("cfg5", 1, 4096, 11008, bits, 32, dtype)
+
+    # GGUF blocks -> affine triplet (load-time conversion of a [14336, 4096] tensor)
+    from mlx_amd import gguf
+    for name, type_id, block_bytes, out_bytes in (("Q4_0", 2, 18, 20), ("Q4_1", 3, 20, 20), ("Q8_0", 8, 34, 36)):
+        n_blocks = 14336 * 4096 // 32
+        blocks = torch.randint(0, 256, (n_blocks * block_bytes,), generator=g, dtype=torch.uint8).to(dev)
+        ms = timed(lambda i: gguf.repack(blocks, type_id, (14336, 4096)))
+        add("gguf", f"repack {name} [14336,4096] -> affine g32", ms, nbytes=n_blocks * (block_bytes + out_bytes))
     return rows
 
 

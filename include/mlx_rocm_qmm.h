@@ -90,6 +90,37 @@ int mlxrocm_affine_dequantize(
     int dtype,
     mlxrocm_stream_t stream);
 
+/*
+ * GGML tensor types the GGUF loader keeps quantized (ids as in the GGUF file
+ * format; every other quantized type is dequantized to fp16 by MLX's loader,
+ * mlx/io/gguf.cpp, and is not handled here).
+ */
+typedef enum {
+  MLXROCM_GGML_Q4_0 = 2,
+  MLXROCM_GGML_Q4_1 = 3,
+  MLXROCM_GGML_Q8_0 = 8
+} mlxrocm_ggml_type_t;
+
+/*
+ * Replaces the load-time conversion gguf_load_quantized (mlx/io/gguf_quants.cpp:
+ * 102-166; block decoders extract_q4_0_data :33-52, extract_q4_1_data :54-74,
+ * extract_q8_0_data :76-100, nibble order unpack_32_4 :13-31) for tensor data
+ * already resident in device memory.  blocks holds n_blocks GGML blocks of 32
+ * weights (18, 20 or 34 bytes each, back to back); outputs are the affine
+ * triplet with group size 32: wq n_blocks*4 words (Q4_*, bits = 4) or
+ * n_blocks*8 words (Q8_0, bits = 8), scales and biases n_blocks fp16 values
+ * (Q4_0: bias = -8 d, Q8_0: bias = -128 d and codes = int8 + 128).  blocks and
+ * wq must be 16-byte aligned.
+ */
+int mlxrocm_gguf_repack(
+    const void* blocks,
+    uint32_t* wq,
+    void* scales,
+    void* biases,
+    size_t n_blocks,
+    int ggml_type,
+    mlxrocm_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* Quantized matmul                                                          */
 /* ------------------------------------------------------------------------ */

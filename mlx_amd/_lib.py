@@ -28,6 +28,7 @@ SIGNATURES = {
     "mlxrocm_last_error": (ctypes.c_char_p, []),
     "mlxrocm_affine_quantize": (_i, [_p, _p, _p, _p, _sz, _i, _i, _i, _p]),
     "mlxrocm_affine_dequantize": (_i, [_p, _p, _p, _p, _sz, _i, _i, _i, _p]),
+    "mlxrocm_gguf_repack": (_i, [_p, _p, _p, _p, _sz, _i, _p]),
     "mlxrocm_qmm": (
         _i,
         [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p],

@@ -11,13 +11,13 @@ this package): a quantized layer keeps ``weight`` (uint32 codes), ``scales`` and
 from __future__ import annotations
 
 import math
-from typing import Callable, Optional, Union
+from typing import Callable, List, Optional, Tuple, Union
 
 import torch
 
 from . import ops
 
-__all__ = ["QuantizedLinear", "QuantizedEmbedding", "quantize"]
+__all__ = ["QuantizedLinear", "QuantizedEmbedding", "quantize", "save_weights", "load_weights"]
 
 
 def _defaults_for_mode(mode: str, group_size: Optional[int], bits: Optional[int]):
@@ -159,4 +159,67 @@ def quantize(model: torch.nn.Module, group_size: Optional[int] = None,
                 raise ValueError("``class_predicate`` must return a bool or a dict of "
                                  "parameters to pass to ``to_quantized``")
             setattr(parent, name, _to_quantized(child, **kwargs))
+    return model
+
+
+def save_weights(model: torch.nn.Module, file: str) -> None:
+    """``Module.save_weights`` (python/mlx/nn/layers/base.py:209-224) for the
+    ``.safetensors`` format: every parameter and buffer under its dotted path, so
+    a quantized layer is stored as the triplet ``weight`` (U32 codes), ``scales``,
+    ``biases`` (+ ``bias``) exactly as MLX stores a quantized model, with the
+    ``{"format": "mlx"}`` metadata ``mx.save_safetensors`` writes."""
+    from safetensors.torch import save_file
+
+    if not str(file).endswith(".safetensors"):
+        raise ValueError(f"Unsupported file extension for {file}. Use '.safetensors'.")
+    tensors = {k: v.detach().contiguous().cpu() for k, v in model.state_dict().items()}
+    save_file(tensors, str(file), metadata={"format": "mlx"})
+
+
+def load_weights(model: torch.nn.Module,
+                 file_or_weights: Union[str, List[Tuple[str, torch.Tensor]]],
+                 strict: bool = True) -> torch.nn.Module:
+    """``Module.load_weights`` (python/mlx/nn/layers/base.py:123-207): update the
+    model from a ``.safetensors`` file or a list of (name, tensor) pairs.  With
+    ``strict`` the names must match the model's exactly and the shapes agree;
+    otherwise only the names the model has are taken.  Tensors keep their stored
+    dtype (a layer's ``scales`` may be float16 in the file and the model built in
+    float32) and move to the device of the tensor they replace."""
+    weights = file_or_weights
+    if isinstance(weights, (str, bytes)) or hasattr(weights, "__fspath__"):
+        from safetensors.torch import load_file
+
+        if not str(weights).endswith(".safetensors"):
+            raise ValueError(f"Unsupported file extension for {weights}. Use '.safetensors'.")
+        weights = list(load_file(str(weights)).items())
+    weights = list(weights)
+    current = model.state_dict()
+    if strict:
+        new = dict(weights)
+        if extras := (new.keys() - current.keys()):
+            listing = ",\n".join(sorted(extras))
+            raise ValueError(f"Received {len(extras)} parameters not in model: \n{listing}.")
+        if missing := (current.keys() - new.keys()):
+            listing = ",\n".join(sorted(missing))
+            raise ValueError(f"Missing {len(missing)} parameters: \n{listing}.")
+        for k, v in current.items():
+            v_new = new[k]
+            if not isinstance(v_new, torch.Tensor):
+                raise ValueError(f"Expected a tensor but received {type(v_new)} for parameter {k}")
+            if tuple(v_new.shape) != tuple(v.shape):
+                raise ValueError(
+                    f"Expected shape {tuple(v.shape)} but received shape {tuple(v_new.shape)} "
+                    f"for parameter {k}"
+                )
+    for name, value in weights:
+        if name not in current:
+            continue
+        path, _, leaf = name.rpartition(".")
+        owner = model.get_submodule(path) if path else model
+        value = value.to(current[name].device)
+        if leaf in owner._parameters:
+            owner._parameters[leaf] = torch.nn.Parameter(value, requires_grad=owner._parameters[leaf].requires_grad
+                                                         and value.is_floating_point())
+        else:
+            owner._buffers[leaf] = value
     return model

@@ -4,6 +4,7 @@ import torch
 
 import mlx_amd
 from mlx_amd import nn as qnn
+from util import bits_equal
 
 pytestmark = pytest.mark.gpu
 
@@ -66,3 +67,47 @@ def test_quantized_linear_shapes(gpu, bits):
                                 dtype=torch.bfloat16)
     y = fresh(torch.randn(2, 7, 512, device=gpu, dtype=torch.bfloat16))
     assert y.shape == (2, 7, 64) and y.dtype == torch.bfloat16
+
+
+def test_safetensors_triplet_round_trip(tmp_path):
+    # a quantized model is stored as (weight U32, scales, biases [, bias]) per layer
+    # and loads back bit for bit; strict loading reports extra / missing / misshapen names
+    import json
+    import struct
+
+    from mlx_amd import nn as qnn
+
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Linear(128, 64), torch.nn.ReLU(), torch.nn.Linear(64, 32, bias=False))
+    model = model.cuda().to(torch.bfloat16)
+    qnn.quantize(model, group_size=32, bits=4)
+    path = tmp_path / "model.safetensors"
+    qnn.save_weights(model, str(path))
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+    assert header["__metadata__"] == {"format": "mlx"}
+    assert header["0.weight"]["dtype"] == "U32" and header["0.weight"]["shape"] == [64, 16]
+    assert header["0.scales"]["dtype"] == "BF16" and header["0.scales"]["shape"] == [64, 4]
+    assert sorted(k for k in header if k != "__metadata__") == [
+        "0.bias", "0.biases", "0.scales", "0.weight", "2.biases", "2.scales", "2.weight"]
+
+    fresh = torch.nn.Sequential(torch.nn.Linear(128, 64), torch.nn.ReLU(), torch.nn.Linear(64, 32, bias=False))
+    fresh = fresh.cuda().to(torch.bfloat16)
+    qnn.quantize(fresh, group_size=32, bits=4)
+    qnn.load_weights(fresh, str(path))
+    for (k, a), (_, b) in zip(model.state_dict().items(), fresh.state_dict().items()):
+        assert bits_equal(a, b), k
+    x = torch.randn(3, 128, device="cuda", dtype=torch.bfloat16)
+    assert torch.equal(model(x), fresh(x))
+
+    with pytest.raises(ValueError, match="Missing 1 parameters"):
+        qnn.load_weights(fresh, [(k, v) for k, v in model.state_dict().items() if k != "2.scales"])
+    with pytest.raises(ValueError, match="not in model"):
+        qnn.load_weights(fresh, list(model.state_dict().items()) + [("3.weight", torch.zeros(1))])
+    with pytest.raises(ValueError, match="Expected shape"):
+        qnn.load_weights(fresh, [(k, v[:1] if k == "0.bias" else v) for k, v in model.state_dict().items()])
+    qnn.load_weights(fresh, [("0.bias", torch.ones(64, dtype=torch.bfloat16))], strict=False)
+    assert torch.equal(fresh[0].bias, torch.ones(64, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError, match="Unsupported file extension"):
+        qnn.save_weights(model, str(tmp_path / "model.npz"))
