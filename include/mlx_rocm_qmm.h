@@ -222,7 +222,7 @@ size_t mlxrocm_gather_qmm_workspace_size(
     int rhs_sorted);
 
 /* Name of the kernel family the dispatcher would pick (for logs and tests):
- * "qmv", "qmm_t", "qmm_generic", ...  Returns NULL for invalid arguments. */
+ * "qmv", "qmm_t", "qmm_n", "qmm_generic".  Returns NULL for invalid arguments. */
 const char* mlxrocm_qmm_kernel_name(
     int M,
     int N,

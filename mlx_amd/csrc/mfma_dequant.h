@@ -99,6 +99,75 @@ struct PairDequant {
   }
 };
 
+// Dequantization of a 4 (k) x 8 (n) block of a [K, N] weight matrix whose codes
+// run along n: w holds, row by row, the BITS / 4 words with the 8 codes of each
+// of the 4 rows, s / b the rows' scale and bias.  pair<Q>() returns column
+// Q / 2, rows 2 (Q % 2) and 2 (Q % 2) + 1, rounded to T and packed: two
+// neighbours along k, which is how the LDS tile wants them.
+template <typename T, int BITS>
+struct ColDequant {
+  static_assert(BITS == 4 || BITS == 8, "columns of 4- and 8-bit codes");
+  uint32_t lo[4], hi[4]; // 4-bit: even / odd columns of a row as bytes
+
+  template <int Q>
+  __device__ __forceinline__ uint32_t
+  pair(const uint32_t (&w)[BITS], const float (&s)[4], const float (&b)[4]) {
+    constexpr int i = Q / 2;      // column 0..7
+    constexpr int j0 = 2 * (Q % 2); // first of the two rows
+    float c0, c1;
+    if constexpr (BITS == 4) {
+      if constexpr (i == 0) {
+        lo[j0] = w[j0] & 0x0f0f0f0fu;
+        lo[j0 + 1] = w[j0 + 1] & 0x0f0f0f0fu;
+        asm("" : "+v"(lo[j0]));
+        asm("" : "+v"(lo[j0 + 1]));
+      }
+      if constexpr (i == 1) {
+        hi[j0] = (w[j0] >> 4) & 0x0f0f0f0fu;
+        hi[j0 + 1] = (w[j0 + 1] >> 4) & 0x0f0f0f0fu;
+        asm("" : "+v"(hi[j0]));
+        asm("" : "+v"(hi[j0 + 1]));
+      }
+      constexpr int sh = 8 * (i / 2);
+      if constexpr (i % 2 == 0) {
+        c0 = static_cast<float>((lo[j0] >> sh) & 0xffu);
+        c1 = static_cast<float>((lo[j0 + 1] >> sh) & 0xffu);
+      } else {
+        c0 = static_cast<float>((hi[j0] >> sh) & 0xffu);
+        c1 = static_cast<float>((hi[j0 + 1] >> sh) & 0xffu);
+      }
+    } else {
+      constexpr int word = i / 4;
+      constexpr int sh = 8 * (i % 4);
+      c0 = static_cast<float>((w[2 * j0 + word] >> sh) & 0xffu);
+      c1 = static_cast<float>((w[2 * (j0 + 1) + word] >> sh) & 0xffu);
+    }
+    return pack2<T>(fmaf(s[j0], c0, b[j0]), fmaf(s[j0 + 1], c1, b[j0 + 1]));
+  }
+};
+
+template <typename T, int BITS, int... Q>
+__device__ __forceinline__ void dequant_cols_impl(
+    const uint32_t (&w)[BITS],
+    const float (&s)[4],
+    const float (&b)[4],
+    uint32_t (&out)[16],
+    std::integer_sequence<int, Q...>) {
+  ColDequant<T, BITS> dq;
+  ((out[Q] = dq.template pair<Q>(w, s, b)), ...);
+}
+
+// The whole 4 x 8 block in one go (prologue): out[2 i], out[2 i + 1] hold rows
+// 0..3 of column i.
+template <typename T, int BITS>
+__device__ __forceinline__ void dequant_cols(
+    const uint32_t (&w)[BITS],
+    const float (&s)[4],
+    const float (&b)[4],
+    uint32_t (&out)[16]) {
+  dequant_cols_impl<T, BITS>(w, s, b, out, std::make_integer_sequence<int, 16>{});
+}
+
 template <typename T, int BITS, int... Q>
 __device__ __forceinline__ void dequant32_impl(
     const uint32_t (&w)[BITS],

@@ -9,18 +9,21 @@ namespace mlxrocm {
 
 namespace {
 
-enum class Family { Qmv, QmmT, QmmNaive };
+enum class Family { Qmv, QmmT, QmmN, QmmNaive };
 
 // M up to which the transpose=true path is a row-streaming GEMV: every packed
 // weight row is read once and reused across the few rows of x.
 constexpr int kQmvMaxM = 8;
 
-Family choose_family(int M, int /*N*/, int K, int /*L*/, int dtype, bool transpose) {
+Family choose_family(int M, int /*N*/, int K, int /*L*/, int bits, int dtype, bool transpose) {
   if (transpose && M <= kQmvMaxM) {
     return Family::Qmv;
   }
   if (transpose && K % 64 == 0 && K >= 64) {
     return Family::QmmT; // fp32 runs on the same matrix path, operands split in two
+  }
+  if (!transpose && K % 64 == 0 && K >= 64 && dtype != MLXROCM_FLOAT32 && (bits == 4 || bits == 8)) {
+    return Family::QmmN; // w [K, N]: the matrix path with a column loader, any M
   }
   return Family::QmmNaive;
 }
@@ -31,6 +34,8 @@ const char* family_name(Family f) {
       return "qmv";
     case Family::QmmT:
       return "qmm_t";
+    case Family::QmmN:
+      return "qmm_n";
     case Family::QmmNaive:
       return "qmm_generic";
   }
@@ -216,7 +221,8 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
 
 // 16-bit prefill whose tiles would leave most compute units idle: K is cut into
 // ranges, the fp32 partial tiles go to scratch and are added up.
-int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
+int run_k_split(
+    const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s, bool transpose = true) {
   const size_t plane = static_cast<size_t>(a.M) * a.N;
   std::lock_guard<std::mutex> lock(g_scratch_mu);
   void* scratch = nullptr;
@@ -226,7 +232,8 @@ int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hip
   }
   QmmArgs part = a;
   part.out = scratch;
-  rc = launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s);
+  rc = transpose ? launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s)
+                 : launch_qmm_mfma_n(part, gs, bits, dtype, k_splits, s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
@@ -257,7 +264,7 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   if (staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
     return launch_qmv_wide(a, gs, bits, dtype, s);
   }
-  switch (choose_family(a.M, a.N, a.K, a.L, dtype, transpose)) {
+  switch (choose_family(a.M, a.N, a.K, a.L, bits, dtype, transpose)) {
     case Family::QmmT:
       if (qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
         if (a.lhs_indices == nullptr && (static_cast<int64_t>(a.M) * a.N) % 4 == 0) {
@@ -280,6 +287,17 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
         return launch_qmv_mfma(a, gs, bits, dtype, s);
       }
       return launch_qmv_generic(a, gs, bits, dtype, s);
+    case Family::QmmN:
+      if (a.lhs_indices == nullptr && qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
+        if ((static_cast<int64_t>(a.M) * a.N) % 4 == 0) {
+          const int k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, a.L);
+          if (k_splits > 1) {
+            return run_k_split(a, gs, bits, dtype, k_splits, s, false);
+          }
+        }
+        return launch_qmm_mfma_n(a, gs, bits, dtype, 1, s);
+      }
+      return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
     case Family::QmmNaive:
       return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
   }
@@ -305,7 +323,7 @@ extern "C" const char* mlxrocm_qmm_kernel_name(
       MLXROCM_OK) {
     return nullptr;
   }
-  return family_name(choose_family(M, N, K, L, dtype, transpose != 0));
+  return family_name(choose_family(M, N, K, L, bits, dtype, transpose != 0));
 }
 
 extern "C" int mlxrocm_qmm(

@@ -112,6 +112,9 @@ int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s, int
 // Few tiles: K is cut into qmm_mfma_k_splits() ranges whose fp32 partial tiles
 // (k_splits planes of M x N behind a.out) reduce_k_splits() adds up.
 int qmm_mfma_k_splits(int M, int N, int K, int L);
+// transpose=false (w [K, N*bits/32]), 4/8-bit, 16-bit types, K % 64 == 0; with
+// k_splits > 1 `a.out` points at k_splits fp32 planes as for the k-split launch.
+int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
 int launch_qmm_mfma_ksplit(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
 int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int dtype, hipStream_t s);
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);

@@ -78,13 +78,21 @@ constexpr int wstore_at(int m, int ns) {
 // points at the [hi | lo | hi] bf16 image of x and spans 3 K).  TO is the type
 // of y: TS, or float when K is cut into k_splits ranges (blockIdx.z), each of
 // which writes its partial tile to plane blockIdx.z of a.out.
-template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED>
+//
+// WN: the weights are [K, N] with the codes (and the groups) running along n
+// (transpose=false).  Only the W loader differs: a thread then owns a 4 (k) x
+// 8 (n) block of the step's tile -- one word (4-bit) or two (8-bit) from each of
+// four consecutive rows of W, each row with its own scale and bias -- and
+// stores it to the same [n][k] LDS tile as eight 8-byte column pieces.
+template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED, bool WN = false>
 __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const QmmArgs a,
     const int gs_shift,
     const int k_splits) {
   constexpr bool kSplit = !std::is_same<T, TS>::value;
   static_assert(!(kSplit && GROUPED), "the grouped gather runs on 16-bit types only");
+  static_assert(!(WN && (kSplit || GROUPED)), "[K, N] weights: plain 16-bit problems only");
+  static_assert(!WN || BITS == 4 || BITS == 8, "[K, N] weights: 4- and 8-bit codes");
   constexpr int kBN = 32 * NT;
   constexpr int kNS = 8 * NT; // MFMAs per wavefront per K-step
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -153,8 +161,9 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   // x as the kernel sees it: three 64-wide blocks per block of K when split
   const int Kx = kSplit ? 3 * K : K;
 
-  const int groups = K >> gs_shift;
-  const int row_words = K / 32 * BITS;
+  // groups and packed words per row of W (rows run along k, or along n when WN)
+  const int groups = (WN ? N : K) >> gs_shift;
+  const int row_words = (WN ? N : K) / 32 * BITS;
 
   // ---- loader roles ----
   // x: thread covers 16-byte chunk (tid % 8) of rows tid/8 + 64 i, i < 4.
@@ -164,11 +173,32 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   // threads past the tile's rows repeat its last row (same values, same place).
   const int wr = (tid >> 1) < kBN ? (tid >> 1) : kBN - 1;
   const int wh = tid & 1;
-  const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
-  const uint32_t* wsrc = reinterpret_cast<const uint32_t*>(p.w) +
-      static_cast<size_t>(w_row) * row_words + wh * BITS;
-  const TS* ssrc = p.scales + static_cast<size_t>(w_row) * groups;
-  const TS* bsrc = p.biases + static_cast<size_t>(w_row) * groups;
+  // WN: thread (kg, ng) covers rows 4 kg .. 4 kg + 3 of the step and columns
+  // 8 ng .. 8 ng + 7 of the tile; kg runs fastest, so that the 8-byte LDS
+  // stores of 16 neighbouring lanes fill one 128-byte tile row.  Threads past
+  // the tile repeat its last block.
+  constexpr int kColBlocks = kBN / 8;
+  constexpr int kWPR = BITS / 4 > 0 ? BITS / 4 : 1; // words per 8 codes (WN: 1 or 2)
+  constexpr int kSB = WN ? 4 : 1;                   // scale / bias pairs per thread
+  const int wt = tid < 16 * kColBlocks ? tid : 16 * kColBlocks - 1;
+  const int kg = wt & 15;
+  const int ng = wt >> 4;
+  const uint32_t* wsrc;
+  const TS* ssrc;
+  const TS* bsrc;
+  if constexpr (WN) {
+    const int ncol = (n0 + 8 * ng < N) ? n0 + 8 * ng : N - 8; // clamp: stay in bounds
+    wsrc = reinterpret_cast<const uint32_t*>(p.w) +
+        static_cast<size_t>(4 * kg) * row_words + ncol / 8 * kWPR;
+    ssrc = p.scales + static_cast<size_t>(4 * kg) * groups + (ncol >> gs_shift);
+    bsrc = p.biases + static_cast<size_t>(4 * kg) * groups + (ncol >> gs_shift);
+  } else {
+    const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
+    wsrc = reinterpret_cast<const uint32_t*>(p.w) +
+        static_cast<size_t>(w_row) * row_words + wh * BITS;
+    ssrc = p.scales + static_cast<size_t>(w_row) * groups;
+    bsrc = p.biases + static_cast<size_t>(w_row) * groups;
+  }
   // Rows of x past M are never stored, so they may read any valid row: the
   // loads then need no predicate.  32-bit element offsets from p.x.
   uint32_t xoff0, xoff1, xoff2, xoff3;
@@ -199,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 // scratch memory
 #define QMM_XQ(set, i) (*((kXSets == 2 && (set) == 1) ? &xb##i : &xa##i))
   uint32_t wreg[BITS], wnext[BITS];
-  TS sreg, breg, snext, bnext; // converted when used, so the loads are not waited for early
+  TS sreg[kSB], breg[kSB], snext[kSB], bnext[kSB]; // converted when used, so the loads are not waited for early
 
 #define QMM_LOAD_X(set, k0)                                                      \
   do {                                                                           \
@@ -211,15 +241,27 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 
 #define QMM_LOAD_W(k0)                                                           \
   do {                                                                           \
-    /* split mode: blocks 3t, 3t+1, 3t+2 of x all meet block t of W */           \
-    const int kw__ = kSplit ? ((k0) / (3 * kBK)) * kBK : (k0);                   \
-    const uint32_t* wp__ = wsrc + (kw__ / 32) * BITS;                            \
-    _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
-      wnext[j__] = wp__[j__];                                                    \
+    if constexpr (WN) {                                                          \
+      const uint32_t* wp__ = wsrc + static_cast<size_t>(k0) * row_words;         \
+      const size_t g__ = static_cast<size_t>(k0) * groups;                       \
+      _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
+        _Pragma("unroll") for (int u__ = 0; u__ < kWPR; ++u__) {                 \
+          wnext[j__ * kWPR + u__] = wp__[static_cast<size_t>(j__) * row_words + u__]; \
+        }                                                                        \
+        snext[j__] = ssrc[g__ + static_cast<size_t>(j__) * groups];              \
+        bnext[j__] = bsrc[g__ + static_cast<size_t>(j__) * groups];              \
+      }                                                                          \
+    } else {                                                                     \
+      /* split mode: blocks 3t, 3t+1, 3t+2 of x all meet block t of W */         \
+      const int kw__ = kSplit ? ((k0) / (3 * kBK)) * kBK : (k0);                 \
+      const uint32_t* wp__ = wsrc + (kw__ / 32) * BITS;                          \
+      _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                   \
+        wnext[j__] = wp__[j__];                                                  \
+      }                                                                          \
+      const int g__ = (kw__ + 32 * wh) >> gs_shift;                              \
+      snext[0] = ssrc[g__];                                                      \
+      bnext[0] = bsrc[g__];                                                      \
     }                                                                            \
-    const int g__ = (kw__ + 32 * wh) >> gs_shift;                                \
-    snext = ssrc[g__];                                                           \
-    bnext = bsrc[g__];                                                           \
   } while (0)
 
 #define QMM_ROTATE_W()                                                           \
@@ -227,8 +269,10 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
       wreg[j__] = wnext[j__];                                                    \
     }                                                                            \
-    sreg = snext;                                                                \
-    breg = bnext;                                                                \
+    _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
+      sreg[j__] = snext[j__];                                                    \
+      breg[j__] = bnext[j__];                                                    \
+    }                                                                            \
   } while (0)
 
 #define QMM_STORE_X(set, stage)                                                  \
@@ -244,11 +288,25 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   do {                                                                           \
     T* ws__ = lds + (stage) * kStage + kXTile;                                   \
     uint32_t dq__[16];                                                           \
-    dequant32<T, BITS>(wreg, to_f32(sreg), to_f32(breg), dq__);                  \
-    uint4* dst__ = reinterpret_cast<uint4*>(&ws__[wr * kLdsStride + wh * 32]);   \
-    _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                        \
-      dst__[j__] = make_uint4(                                                   \
-          dq__[4 * j__], dq__[4 * j__ + 1], dq__[4 * j__ + 2], dq__[4 * j__ + 3]); \
+    if constexpr (WN) {                                                          \
+      float sf__[4], bf__[4];                                                    \
+      _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
+        sf__[j__] = to_f32(sreg[j__]);                                           \
+        bf__[j__] = to_f32(breg[j__]);                                           \
+      }                                                                          \
+      dequant_cols<T, BITS>(wreg, sf__, bf__, dq__);                             \
+      T* col__ = &ws__[(8 * ng) * kLdsStride + 4 * kg];                          \
+      _Pragma("unroll") for (int i__ = 0; i__ < 8; ++i__) {                      \
+        *reinterpret_cast<uint2*>(col__ + i__ * kLdsStride) =                    \
+            make_uint2(dq__[2 * i__], dq__[2 * i__ + 1]);                        \
+      }                                                                          \
+    } else {                                                                     \
+      dequant32<T, BITS>(wreg, to_f32(sreg[0]), to_f32(breg[0]), dq__);          \
+      uint4* dst__ = reinterpret_cast<uint4*>(&ws__[wr * kLdsStride + wh * 32]); \
+      _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
+        dst__[j__] = make_uint4(                                                 \
+            dq__[4 * j__], dq__[4 * j__ + 1], dq__[4 * j__ + 2], dq__[4 * j__ + 3]); \
+      }                                                                          \
     }                                                                            \
   } while (0)
 
@@ -369,13 +427,25 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
       QMM_LOAD_W(k2);                                                            \
     }                                                                            \
     if constexpr (pair_at((m), kNS) >= 0) {                                      \
-      dqv[pair_at((m), kNS)] =                                                   \
-          dq.template pair<pair_at((m), kNS)>(wreg, sf, bf, low_part);           \
+      if constexpr (WN) {                                                        \
+        dqv[pair_at((m), kNS)] = cdq.template pair<pair_at((m), kNS)>(wreg, sf, bf); \
+      } else {                                                                   \
+        dqv[pair_at((m), kNS)] =                                                 \
+            dq.template pair<pair_at((m), kNS)>(wreg, sf[0], bf[0], low_part);   \
+      }                                                                          \
     }                                                                            \
     if constexpr (wstore_at((m), kNS) >= 0) {                                    \
       constexpr int r__ = wstore_at((m), kNS);                                   \
-      wdst[r__] = make_uint4(                                                    \
-          dqv[4 * r__], dqv[4 * r__ + 1], dqv[4 * r__ + 2], dqv[4 * r__ + 3]);   \
+      if constexpr (WN) {                                                        \
+        /* pairs 4r .. 4r+3: columns 2r and 2r+1, four rows (k) each */          \
+        *reinterpret_cast<uint2*>(wcol + (2 * r__) * kLdsStride) =               \
+            make_uint2(dqv[4 * r__], dqv[4 * r__ + 1]);                          \
+        *reinterpret_cast<uint2*>(wcol + (2 * r__ + 1) * kLdsStride) =           \
+            make_uint2(dqv[4 * r__ + 2], dqv[4 * r__ + 3]);                      \
+      } else {                                                                   \
+        wdst[r__] = make_uint4(                                                  \
+            dqv[4 * r__], dqv[4 * r__ + 1], dqv[4 * r__ + 2], dqv[4 * r__ + 3]); \
+      }                                                                          \
     }                                                                            \
     if constexpr ((m) == 1) {                                                    \
       *reinterpret_cast<uint4*>(&xs[(xr + 0) * kLdsStride + xc * 8]) = QMM_XQ(P, 0);   \
@@ -412,12 +482,17 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const int kx = kclamp((tt) + 1 + kXSets);                                    \
     T* xs = lds + nxt * kStage;                                                  \
     uint4* wdst = reinterpret_cast<uint4*>(&xs[kXTile + wr * kLdsStride + wh * 32]); \
-    const float sf = to_f32(sreg);                                               \
-    const float bf = to_f32(breg);                                               \
+    T* wcol = &xs[kXTile + (8 * ng) * kLdsStride + 4 * kg];                      \
+    float sf[kSB], bf[kSB];                                                      \
+    _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
+      sf[j__] = to_f32(sreg[j__]);                                               \
+      bf[j__] = to_f32(breg[j__]);                                               \
+    }                                                                            \
     /* the tile prepared in step tt is tile tt + 1: block (tt + 1) % 3 of its   \
        group of three takes the weights' low parts */                           \
     const bool low_part = kSplit && ((tt) + 1) % 3 == 2;                         \
     PairDequant<T, BITS> dq;                                                     \
+    ColDequant<T, (WN ? BITS : 4)> cdq;                                          \
     uint32_t dqv[16];                                                            \
     __builtin_amdgcn_sched_barrier(0);                                           \
     QMM_SLOTS8(0, P) QMM_SLOTS8(8, P) QMM_SLOTS8(16, P) QMM_SLOTS8(24, P)        \
@@ -555,13 +630,13 @@ int choose_nt(int M, int N, int L) {
   return best;
 }
 
-template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED>
+template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED, bool WN = false>
 int launch_variant(const QmmArgs& a, int gs_shift, dim3 grid, hipStream_t s, int k_splits = 1) {
   constexpr size_t smem = qmm_smem_bytes<NT>();
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
-  auto kern = qmm_t_mfma_kernel<T, TS, TO, BITS, NT, GROUPED>;
+  auto kern = qmm_t_mfma_kernel<T, TS, TO, BITS, NT, GROUPED, WN>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -583,11 +658,46 @@ int shift_of(int gs) {
 
 bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose) {
   (void)gs;
-  (void)bits;
-  if (!transpose || dtype == MLXROCM_FLOAT32) {
+  if (dtype == MLXROCM_FLOAT32) {
     return false;
   }
+  if (!transpose && !(bits == 4 || bits == 8)) {
+    return false; // [K, N] weights: the column loader reads whole words per 8 codes
+  }
   return a.K % kBK == 0 && a.K >= kBK;
+}
+
+namespace {
+
+// [K, N] weights (transpose=false), 4- or 8-bit; TO = float when K is split.
+template <typename T, typename TO, int NT>
+int launch_wn(const QmmArgs& a, int gs_shift, int bits, dim3 grid, hipStream_t s, int k_splits) {
+  if (bits == 4) {
+    return launch_variant<T, T, TO, 4, NT, false, true>(a, gs_shift, grid, s, k_splits);
+  }
+  return launch_variant<T, T, TO, 8, NT, false, true>(a, gs_shift, grid, s, k_splits);
+}
+
+} // namespace
+
+// transpose=false on the matrix cores: same tiles, column loader for W.
+int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
+  const int gs_shift = shift_of(gs);
+  if (k_splits > 1) {
+    const dim3 grid((a.N + 32 * 6 - 1) / (32 * 6), (a.M + kBM - 1) / kBM, k_splits);
+    return dtype == MLXROCM_BFLOAT16
+        ? launch_wn<bf16_t, float, 6>(a, gs_shift, bits, grid, s, k_splits)
+        : launch_wn<f16_t, float, 6>(a, gs_shift, bits, grid, s, k_splits);
+  }
+  int nt = choose_nt(a.M, a.N, a.L);
+  nt = nt > 6 ? 6 : nt; // the column loader's registers leave room for 6 x 32 columns
+  const dim3 grid((a.N + 32 * nt - 1) / (32 * nt), (a.M + kBM - 1) / kBM, a.L);
+  auto run = [&](auto tval) -> int {
+    using T = decltype(tval);
+    return nt == 5 ? launch_wn<T, T, 5>(a, gs_shift, bits, grid, s, 1)
+                   : launch_wn<T, T, 6>(a, gs_shift, bits, grid, s, 1);
+  };
+  return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
 }
 
 int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {

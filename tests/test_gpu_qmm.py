@@ -181,3 +181,38 @@ def test_qmm_few_rows_kernels(oracle, gpu, dtype, bits):
             w = normal_weights((N, K), dtype, seed=bits + gs + M)
             x = activations((M, K), dtype, seed=M)
             _check_qmm(oracle, gpu, x, w, gs, bits)
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("bits,gs", ((4, 32), (4, 64), (8, 64), (8, 128)))
+def test_qmm_n_on_the_matrix_path(oracle, gpu, dtype, bits, gs):
+    # transpose=False (w [K, N], groups along n; cpu/quantized.cpp:96-152) with
+    # K % 64 == 0 runs on the matrix cores: one row (qvm), a ragged M, a width
+    # that is not a tile multiple, and a K long enough to be cut into ranges
+    from mlx_amd import _lib
+
+    code = {torch.float16: 1, torch.bfloat16: 2}[dtype]
+    for M, K, N in ((1, 256, 384), (300, 192, 640), (70, 2048, 128), (5, 64, 256)):
+        assert _lib.load().mlxrocm_qmm_kernel_name(M, N, K, 1, gs, bits, code, 0) == b"qmm_n"
+        w = normal_weights((K, N), dtype, seed=bits + gs + M)
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, w, gs, bits, transpose=False)
+
+
+def test_qmm_n_batched_and_full_size(oracle, gpu):
+    # a batch of problems with one shared weight matrix, and the benchmark's
+    # gate/up shape read the other way round, checked on sampled rows
+    dtype = torch.bfloat16
+    K, N = 128, 256
+    w = normal_weights((K, N), dtype, seed=3)
+    wq, s, b = oracle.quantize(w, 64, 4)
+    x = activations((3, 40, K), dtype, seed=5)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq.to(gpu), s.to(gpu), b.to(gpu), False, 64, 4).cpu()
+    for l in range(3):
+        ref = oracle.qmm(x[l], wq, s, b, False, 64, 4)
+        tol = matmul_tolerance(dtype, K, x[l], exact_affine_weights(wq, s, b, 64, 4))
+        assert float((got[l].double() - ref.double()).abs().max()) <= 2 * tol
+    K, N, M = 4096, 14336, 512
+    w = normal_weights((K, N), dtype, seed=0)
+    x = activations((M, K), dtype, seed=0)
+    _check_qmm(oracle, gpu, x, w, 64, 4, transpose=False, rows=torch.tensor([0, 255, 256, 511]))
