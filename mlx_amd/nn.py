@@ -17,7 +17,8 @@ import torch
 
 from . import ops
 
-__all__ = ["QuantizedLinear", "QuantizedEmbedding", "quantize", "save_weights", "load_weights"]
+__all__ = ["QuantizedLinear", "QuantizedEmbedding", "QuantizedSwitchLinear", "SwitchGLU",
+           "quantize", "save_weights", "load_weights"]
 
 
 def _defaults_for_mode(mode: str, group_size: Optional[int], bits: Optional[int]):
@@ -118,6 +119,87 @@ class QuantizedEmbedding(torch.nn.Module):
         ql = cls(num, dims, group_size, bits, mode, device=w.device, dtype=w.dtype)
         ql._set_quantized(w)
         return ql
+
+
+class QuantizedSwitchLinear(torch.nn.Module):
+    """A stack of ``num_experts`` quantized linear layers evaluated through
+    ``gather_qmm``: ``y[..., i, :, :] = x[..., :, :] @ dequant(weight[indices[..., i]]).T``
+    (the expert-routed caller of the path, built on mlx/ops.cpp:5553-5629; x is
+    ``[..., 1 | k, M, input_dims]`` and ``indices`` ``[..., k]``).  With
+    ``sorted_indices`` the caller promises ascending indices, which lets the
+    kernel group the rows of each expert."""
+
+    def __init__(self, input_dims: int, output_dims: int, num_experts: int, bias: bool = True,
+                 group_size: Optional[int] = None, bits: Optional[int] = None,
+                 mode: str = "affine", device=None, dtype=torch.float32):
+        super().__init__()
+        self.group_size, self.bits = _defaults_for_mode(mode, group_size, bits)
+        self.mode = mode
+        device = torch.device("cuda:0") if device is None else torch.device(device)
+        scale = math.sqrt(1.0 / input_dims)
+        weight = (torch.rand((num_experts, output_dims, input_dims), device=device) * 2 - 1) * scale
+        self._set_quantized(weight.to(dtype))
+        self.register_buffer(
+            "bias", torch.zeros((num_experts, output_dims), device=device, dtype=dtype) if bias else None)
+
+    _set_quantized = QuantizedLinear._set_quantized
+
+    @property
+    def num_experts(self) -> int:
+        return self.weight.shape[0]
+
+    def forward(self, x: torch.Tensor, indices: torch.Tensor, sorted_indices: bool = False) -> torch.Tensor:
+        y = ops.gather_qmm(x, self.weight, self.scales, self.biases, rhs_indices=indices,
+                           transpose=True, group_size=self.group_size, bits=self.bits,
+                           mode=self.mode, sorted_indices=sorted_indices)
+        if self.bias is not None:
+            y = y + self.bias[indices.long()].unsqueeze(-2)
+        return y
+
+    def extra_repr(self) -> str:
+        e, out_dims, in_dims = self.weight.shape
+        return (f"input_dims={in_dims * 32 // self.bits}, output_dims={out_dims}, num_experts={e}, "
+                f"bias={self.bias is not None}, group_size={self.group_size}, bits={self.bits}")
+
+
+class SwitchGLU(torch.nn.Module):
+    """Expert-routed gated MLP: ``down(act(gate(x)) * up(x))`` with every
+    projection a :class:`QuantizedSwitchLinear` and token ``t`` sent to the
+    experts ``indices[t, :]``.  From 64 routed rows on, the rows are ordered by
+    expert first (one argsort), so that all three projections run with
+    ``sorted_indices=True``, and put back afterwards."""
+
+    def __init__(self, input_dims: int, hidden_dims: int, num_experts: int,
+                 activation: Callable[[torch.Tensor], torch.Tensor] = torch.nn.functional.silu,
+                 bias: bool = False, group_size: Optional[int] = None, bits: Optional[int] = None,
+                 device=None, dtype=torch.float32, sort_threshold: int = 64):
+        super().__init__()
+        kw = dict(bias=bias, group_size=group_size, bits=bits, device=device, dtype=dtype)
+        self.gate_proj = QuantizedSwitchLinear(input_dims, hidden_dims, num_experts, **kw)
+        self.up_proj = QuantizedSwitchLinear(input_dims, hidden_dims, num_experts, **kw)
+        self.down_proj = QuantizedSwitchLinear(hidden_dims, input_dims, num_experts, **kw)
+        self.activation = activation
+        self.sort_threshold = sort_threshold
+
+    def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+        """x ``[..., D]``, indices ``[..., k]`` -> ``[..., k, D]``."""
+        k = indices.shape[-1]
+        x = x.unsqueeze(-2).unsqueeze(-3)  # [..., 1, 1, D]
+        do_sort = indices.numel() >= self.sort_threshold
+        idx = indices
+        if do_sort:
+            flat = indices.reshape(-1)
+            order = torch.argsort(flat.long(), stable=True)
+            inverse = torch.argsort(order)
+            x = x.reshape(-1, 1, x.shape[-1])[order // k]  # [n, 1, D]: one row per routed pair
+            # torch cannot index uint32 tensors: reorder through an integer copy
+            idx = flat.long()[order].to(indices.dtype)
+        up = self.up_proj(x, idx, sorted_indices=do_sort)
+        gate = self.gate_proj(x, idx, sorted_indices=do_sort)
+        y = self.down_proj(self.activation(gate) * up, idx, sorted_indices=do_sort)
+        if do_sort:
+            y = y[inverse].reshape(*indices.shape, 1, y.shape[-1])
+        return y.squeeze(-2)
 
 
 def _to_quantized(m, **kwargs):

@@ -111,3 +111,48 @@ def test_safetensors_triplet_round_trip(tmp_path):
     assert torch.equal(fresh[0].bias, torch.ones(64, dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(ValueError, match="Unsupported file extension"):
         qnn.save_weights(model, str(tmp_path / "model.npz"))
+
+
+@pytest.mark.parametrize("tokens", (3, 80))
+def test_switch_glu_matches_per_expert_dense(tokens):
+    # every routed (token, expert) pair equals the dense gated MLP of that expert's
+    # dequantized weights; 80 tokens x 2 take the sort-by-expert route, 3 x 2 do not
+    torch.manual_seed(tokens)
+    D, H, E, k = 128, 256, 4, 2
+    dt = torch.bfloat16
+    glu = qnn.SwitchGLU(D, H, E, group_size=64, bits=4, dtype=dt)
+    x = torch.randn(tokens, D, device="cuda", dtype=dt)
+    indices = torch.stack([torch.randperm(E, device="cuda")[:k] for _ in range(tokens)]).to(torch.uint32)
+    y = glu(x, indices)
+    assert tuple(y.shape) == (tokens, k, D)
+
+    def dense(layer, e):
+        return mlx_amd.dequantize(layer.weight[e], layer.scales[e], layer.biases[e],
+                                  group_size=64, bits=4).double()
+
+    worst = 0.0
+    for t in range(tokens):
+        for j in range(k):
+            e = int(indices[t, j])
+            xt = x[t].double()
+            up = (dense(glu.up_proj, e) @ xt).to(dt).double()
+            gate = (dense(glu.gate_proj, e) @ xt).to(dt).double()
+            h = (torch.nn.functional.silu(gate.to(dt)) * up.to(dt)).double()
+            want = dense(glu.down_proj, e) @ h
+            worst = max(worst, float((y[t, j].double() - want).abs().max()))
+    # three bf16 roundings of intermediate activations of magnitude ~1
+    assert worst <= 0.05, worst
+
+
+def test_switch_linear_bias_and_sorted_flag():
+    torch.manual_seed(1)
+    layer = qnn.QuantizedSwitchLinear(64, 96, 3, bias=True, group_size=32, bits=8, dtype=torch.float16)
+    layer.bias.copy_(torch.randn(3, 96, device="cuda", dtype=torch.float16))
+    x = torch.randn(6, 1, 64, device="cuda", dtype=torch.float16)
+    idx = torch.tensor([0, 0, 1, 2, 2, 2], device="cuda", dtype=torch.uint32)
+    a = layer(x, idx, sorted_indices=True)
+    b = layer(x, idx, sorted_indices=False)
+    assert torch.equal(a, b) and tuple(a.shape) == (6, 1, 96)
+    w1 = mlx_amd.dequantize(layer.weight[1], layer.scales[1], layer.biases[1], group_size=32, bits=8)
+    want = x[2, 0].double() @ w1.double().T + layer.bias[1].double()
+    assert float((a[2, 0].double() - want).abs().max()) <= 2e-2
