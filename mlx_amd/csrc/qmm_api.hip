@@ -250,6 +250,21 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   //   17..32 rows the 64-row LDS-staged kernel;
   //   1..2 rows   of a width the row-streaming GEMV does not cover: the wide
   //               kernel as well.
+  // 4-bit decode with a few rows of x: the 4x4x4 matrix-instruction GEMV.
+  // Measured against the kernels below on gate/up, down-projection and group-32
+  // shapes: it wins for 2..4 rows everywhere; for one row only where the
+  // row-streaming GEMV splits a long K over all eight wavefronts (K > 8192);
+  // for 5..8 rows (two operand sets, half the occupancy) only there and with
+  // 32-wide groups.
+  if (transpose && a.M <= 8 && qmv_quad_supported(a, gs, bits, dtype)) {
+    const bool long_k = a.K > 8192;
+    const bool use = (a.M >= 2 && a.M <= 4) ||
+        (a.M == 1 && (long_k || !qmv_stream_supported(a, gs, bits, dtype))) ||
+        (a.M >= 5 && (long_k || gs == 32));
+    if (use) {
+      return launch_qmv_quad(a, gs, bits, dtype, s);
+    }
+  }
   const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype);
   const bool staged = a.M > 16 || (a.M > 8 && a.N >= 8192);
   if (few_rows && !staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {

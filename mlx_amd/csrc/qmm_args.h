@@ -115,6 +115,10 @@ int qmm_mfma_k_splits(int M, int N, int K, int L);
 // transpose=false (w [K, N*bits/32]), 4/8-bit, 16-bit types, K % 64 == 0; with
 // k_splits > 1 `a.out` points at k_splits fp32 planes as for the k-split launch.
 int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
+// 1..8 rows of x on the 4x4x4 matrix instruction: transpose=true, 16-bit types,
+// 4-bit, K a multiple of 512 codes and at most 16384, an even number of groups.
+bool qmv_quad_supported(const QmmArgs& a, int gs, int bits, int dtype);
+int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 int launch_qmm_mfma_ksplit(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
 int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int dtype, hipStream_t s);
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);

@@ -216,3 +216,40 @@ def test_qmm_n_batched_and_full_size(oracle, gpu):
     w = normal_weights((K, N), dtype, seed=0)
     x = activations((M, K), dtype, seed=0)
     _check_qmm(oracle, gpu, x, w, 64, 4, transpose=False, rows=torch.tensor([0, 255, 256, 511]))
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("gs", ALL_GROUPS)
+def test_qmv_matrix_instruction_gemv(oracle, gpu, dtype, gs):
+    """4-bit decode with 2..4 rows of x (and 1 or 5..8 rows where K is long or the
+    groups are 32 wide) runs on the 4x4x4 matrix-instruction GEMV: K of one slot,
+    of a slot count that leaves the last wavefront's slots empty (1536, 14336),
+    of every k-wave split, ragged N, both operand sets of x."""
+    shapes = (
+        (2, 67, 512), (3, 100, 1024), (4, 36, 1536), (2, 64, 2048), (4, 130, 4096),
+        (3, 40, 8192), (1, 24, 14336), (4, 24, 14336), (8, 20, 14336), (7, 33, 16384),
+    )
+    if gs == 32:
+        shapes += ((5, 67, 1024), (8, 40, 4096))
+    for M, N, K in shapes:
+        w = normal_weights((N, K), dtype, seed=gs + M + K)
+        x = activations((M, K), dtype, seed=M + K)
+        _check_qmm(oracle, gpu, x, w, gs, 4)
+
+
+def test_qmv_matrix_instruction_gemv_batched(oracle, gpu):
+    # a batch of problems, each with its own weights: blockIdx.y walks the batch
+    dtype, gs, L, M, N, K = torch.bfloat16, 64, 3, 3, 48, 1024
+    ws = [normal_weights((N, K), dtype, seed=10 + l) for l in range(L)]
+    qs = [oracle.quantize(w, gs, 4) for w in ws]
+    wq = torch.stack([q[0] for q in qs]).to(gpu)
+    s = torch.stack([q[1] for q in qs]).to(gpu)
+    b = torch.stack([q[2] for q in qs]).to(gpu)
+    x = activations((L, M, K), dtype, seed=4)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq, s, b, True, gs, 4).cpu()
+    for l in range(L):
+        ref = oracle.qmm(x[l], *qs[l], True, gs, 4)
+        w_hat = exact_affine_weights(*qs[l], gs, 4)
+        exact = x[l].double() @ w_hat.T
+        tol = matmul_tolerance(dtype, K, x[l], w_hat) + float((ref.double() - exact).abs().max())
+        assert float((got[l].double() - ref.double()).abs().max()) <= tol
