@@ -111,7 +111,8 @@ constexpr int kQuadsPerWave = 4; // row quads whose loads are in flight together
 // each) of K per wavefront.  KW: wavefronts that split K.
 // XLDS: x reaches the lanes through one coalesced read per workgroup and LDS
 // (4 MB K elements of LDS); otherwise every lane fetches its slices itself.
-template <typename T, int BITS, int MB, int S, int KW, int kSbLoads, bool XLDS>
+// MC: columns of an operand set that are live (rows of x: M = 1, 2, or more).
+template <typename T, int BITS, int MB, int S, int KW, int kSbLoads, bool XLDS, int MC>
 __global__ __launch_bounds__(512) void qmv_quad_kernel(const QmmArgs a, const int gs_shift) {
   constexpr int RW = 8 / KW;
   constexpr int kLaneCodes = 128 / BITS;      // codes in a lane's 16 bytes
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(512) void qmv_quad_kernel(const QmmArgs a, const in
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < MC; ++j) {
         y[q][mb][j] = 0.0f;
       }
     }
@@ -350,7 +351,7 @@ __global__ __launch_bounds__(512) void qmv_quad_kernel(const QmmArgs a, const in
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < MC; ++j) {
           y[q][mb][j] = fmaf(s, d[mb][j], y[q][mb][j]);
           y[q][mb][j] = fmaf(beff, sx[mb][c][j], y[q][mb][j]);
         }
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(512) void qmv_quad_kernel(const QmmArgs a, const in
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < MC; ++j) {
         y[q][mb][j] = sum_blocks(y[q][mb][j], lane);
       }
     }
@@ -378,7 +379,7 @@ __global__ __launch_bounds__(512) void qmv_quad_kernel(const QmmArgs a, const in
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < MC; ++j) {
           red[(((rw * KW + kw) * kQuadsPerWave + q) * (MB * 4) + mb * 4 + j) * 4 + lane] =
               y[q][mb][j];
         }
@@ -471,12 +472,13 @@ int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
   // dwords of scales per row and wave, eight per load
   const int sb_words = pl.s * 16 * (128 / bits) / gs / 2;
   const int sb_loads = sb_words <= 8 ? 1 : (sb_words <= 16 ? 2 : 4);
-  auto go = [&](auto tval, auto bval, auto mbv, auto sval, auto kwv) -> int {
+  auto go = [&](auto tval, auto bval, auto mbv, auto sval, auto kwv, auto mcv) -> int {
     using T = decltype(tval);
     constexpr int B = decltype(bval)::value;
     constexpr int MB = decltype(mbv)::value;
     constexpr int S = decltype(sval)::value;
     constexpr int KW = decltype(kwv)::value;
+    constexpr int MC = decltype(mcv)::value;
     auto launch = [&](auto kern) -> int {
       if (smem > 48 * 1024) {
         MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -491,29 +493,40 @@ int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
     if (xlds) {
       // the x image needs whole slots: S * KW covers K exactly or x is zero there
       if (sb_loads == 1) {
-        return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, true>);
+        return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, true, MC>);
       } else if (sb_loads == 2) {
-        return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, true>);
+        return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, true, MC>);
       }
-      return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, true>);
+      return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, true, MC>);
     }
     if (sb_loads == 1) {
-      return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, false>);
+      return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, false, MC>);
     } else if (sb_loads == 2) {
-      return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, false>);
+      return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, false, MC>);
     }
-    return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, false>);
+    return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, false, MC>);
+  };
+  auto by_mc = [&](auto tval, auto bval, auto mbv, auto sval, auto kwv) -> int {
+    if constexpr (decltype(mbv)::value == 1) {
+      if (a.M == 1) {
+        return go(tval, bval, mbv, sval, kwv, IntC<1>{});
+      }
+      if (a.M == 2) {
+        return go(tval, bval, mbv, sval, kwv, IntC<2>{});
+      }
+    }
+    return go(tval, bval, mbv, sval, kwv, IntC<4>{});
   };
   auto by_kw = [&](auto tval, auto bval, auto mbv, auto sval) -> int {
     switch (pl.kw) {
       case 1:
-        return go(tval, bval, mbv, sval, IntC<1>{});
+        return by_mc(tval, bval, mbv, sval, IntC<1>{});
       case 2:
-        return go(tval, bval, mbv, sval, IntC<2>{});
+        return by_mc(tval, bval, mbv, sval, IntC<2>{});
       case 4:
-        return go(tval, bval, mbv, sval, IntC<4>{});
+        return by_mc(tval, bval, mbv, sval, IntC<4>{});
       default:
-        return go(tval, bval, mbv, sval, IntC<8>{});
+        return by_mc(tval, bval, mbv, sval, IntC<8>{});
     }
   };
   auto by_s = [&](auto tval, auto bval, auto mbv) -> int {
