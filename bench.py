@@ -169,20 +169,21 @@ def sweep(torch, mlx_amd, dev) -> list:
         rows.append(row)
         print(json.dumps(row), file=sys.stderr, flush=True)
 
-    def kname(M, n, k, gs, bits, dtype):
+    def kname(M, n, k, gs, bits, dtype, transpose=True):
         from mlx_amd import _lib
         code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
-        return _lib.load().mlxrocm_qmm_kernel_name(M, n, k, 1, gs, bits, code, 1).decode()
+        return _lib.load().mlxrocm_qmm_kernel_name(M, n, k, 1, gs, bits, code, int(transpose)).decode()
 
-    def matmul_case(cfg, M, n, k, bits, gs, dtype):
+    def matmul_case(cfg, M, n, k, bits, gs, dtype, transpose=True):
         """One quantized_matmul shape through the C ABI.  Launches that last a few
         microseconds (M <= 64) replay a HIP graph over the weight ring, like the
-        headline figure; the others are launched one by one."""
+        headline figure; the others are launched one by one.  transpose=False: the
+        weight is [k, n] and quantized along n."""
         from mlx_amd import _lib
         lib = _lib.load()
         esz = 4 if dtype == torch.float32 else 2
         code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
-        q = mlx_amd.quantize(weights(n, k, dtype), gs, bits)
+        q = mlx_amd.quantize(weights(n, k, dtype) if transpose else weights(k, n, dtype), gs, bits)
         wbytes = n * k * bits // 8 + 2 * n * (k // gs) * esz
         small = M <= 64
         ring = ring_of(q, wbytes) if small else [q]
@@ -192,7 +193,8 @@ def sweep(torch, mlx_amd, dev) -> list:
         def step(i, stream):
             wq_, s_, b_ = ring[i % len(ring)]
             rc = lib.mlxrocm_qmm(x.data_ptr(), wq_.data_ptr(), s_.data_ptr(), b_.data_ptr(),
-                                 out.data_ptr(), M, n, k, 1, M * k, 0, 0, gs, bits, code, 1, stream)
+                                 out.data_ptr(), M, n, k, 1, M * k, 0, 0, gs, bits, code,
+                                 int(transpose), stream)
             if rc != 0:
                 raise RuntimeError(_lib.last_error())
 
@@ -200,12 +202,14 @@ def sweep(torch, mlx_amd, dev) -> list:
         launcher.run(len(ring))
         torch.cuda.synchronize()
         ms = hip_event_ms(lib, launcher, max(len(ring) * (20 if small else 1), 10))
-        name = f"x {str(dtype)[6:]} [{M},{k}] W [{n},{k}] b{bits} g{gs}"
+        wshape = f"[{n},{k}]" if transpose else f"[{k},{n}] transpose=False"
+        name = f"x {str(dtype)[6:]} [{M},{k}] W {wshape} b{bits} g{gs}"
         if small:
             add(cfg, name, ms, nbytes=qmv_bytes(M, n, k, bits, gs, esz),
-                kernel=kname(M, n, k, gs, bits, dtype))
+                kernel=kname(M, n, k, gs, bits, dtype, transpose))
         else:
-            add(cfg, name, ms, flops=2.0 * M * n * k, kernel=kname(M, n, k, gs, bits, dtype))
+            add(cfg, name, ms, flops=2.0 * M * n * k,
+                kernel=kname(M, n, k, gs, bits, dtype, transpose))
 
     bf16, f32 = torch.bfloat16, torch.float32
     # Cfg1: fp32 4096 x 4096, 4-bit group 64
@@ -220,13 +224,17 @@ def sweep(torch, mlx_amd, dev) -> list:
     # Cfg2: decode, Llama-3-8B MLP shapes
     for (n, k) in ((14336, 4096), (4096, 14336)):
         for (bits, gs) in ((4, 64), (8, 128)):
-            for B in (1, 4, 8):
+            for B in (1, 2, 4, 8):
                 matmul_case("cfg2", B, n, k, bits, gs, bf16)
     # Cfg3: prefill
     for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336)):
         for (bits, gs) in ((4, 64), (8, 128)):
             for M in (512, 2048, 8192):
                 matmul_case("cfg3", M, n, k, bits, gs, bf16)
+    # transpose=False (the vjp of a quantized linear layer): w [k, n] quantized along n
+    for M in (1, 512, 2048):
+        matmul_case("f3", M, 14336, 4096, 4, 64, bf16, transpose=False)
+        matmul_case("f3", M, 4096, 14336, 8, 128, bf16, transpose=False)
     # Cfg4: 8 experts, top-2 routing
     E, n, k = 8, 14336, 4096
     wq, sc, bi = mlx_amd.quantize(

@@ -221,8 +221,7 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
 
 // 16-bit prefill whose tiles would leave most compute units idle: K is cut into
 // ranges, the fp32 partial tiles go to scratch and are added up.
-int run_k_split(
-    const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s, bool transpose = true) {
+int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
   const size_t plane = static_cast<size_t>(a.M) * a.N;
   std::lock_guard<std::mutex> lock(g_scratch_mu);
   void* scratch = nullptr;
@@ -232,12 +231,54 @@ int run_k_split(
   }
   QmmArgs part = a;
   part.out = scratch;
-  rc = transpose ? launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s)
-                 : launch_qmm_mfma_n(part, gs, bits, dtype, k_splits, s);
+  rc = launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
   return reduce_k_splits(scratch, a.out, plane, k_splits, dtype, s);
+}
+
+// transpose=false on the matrix cores.  The column loader wants the four
+// scales of four consecutive rows of W side by side, so scales and biases are
+// first transposed to [group][k] in the stream's scratch buffer (a few MB, a
+// few microseconds); few-row shapes also cut K and keep their fp32 partial
+// planes there.
+int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  const int G = a.N / gs;
+  const int batches = a.sb_batch_stride == 0 ? 1 : a.L;
+  int k_splits = 1;
+  if ((static_cast<int64_t>(a.M) * a.N) % 4 == 0) {
+    k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, a.L);
+  }
+  const size_t sb_bytes = (qmm_n_sb_bytes(a.K, G, batches, dtype) + 255) / 256 * 256;
+  const size_t plane = static_cast<size_t>(a.M) * a.N;
+  const size_t partial_bytes = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  void* scratch = nullptr;
+  int rc = stream_scratch(s, sb_bytes + partial_bytes, &scratch);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  rc = transpose_sb_for_qmm_n(
+      a.scales, a.biases, scratch, a.K, G, batches, a.sb_batch_stride, dtype, s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  const size_t image = static_cast<size_t>(a.K) * G; // elements of one [G][K] image
+  QmmArgs part = a;
+  part.scales = scratch;
+  part.biases = static_cast<char*>(scratch) + image * dtype_size(dtype);
+  part.sb_batch_stride = batches == 1 ? 0 : static_cast<int64_t>(2 * image);
+  if (k_splits <= 1) {
+    return launch_qmm_mfma_n(part, gs, bits, dtype, 1, s);
+  }
+  void* partial = static_cast<char*>(scratch) + sb_bytes;
+  part.out = partial;
+  rc = launch_qmm_mfma_n(part, gs, bits, dtype, k_splits, s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  return reduce_k_splits(partial, a.out, plane, k_splits, dtype, s);
 }
 
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
@@ -304,13 +345,7 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
       return launch_qmv_generic(a, gs, bits, dtype, s);
     case Family::QmmN:
       if (a.lhs_indices == nullptr && qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
-        if ((static_cast<int64_t>(a.M) * a.N) % 4 == 0) {
-          const int k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, a.L);
-          if (k_splits > 1) {
-            return run_k_split(a, gs, bits, dtype, k_splits, s, false);
-          }
-        }
-        return launch_qmm_mfma_n(a, gs, bits, dtype, 1, s);
+        return run_qmm_n(a, gs, bits, dtype, s);
       }
       return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
     case Family::QmmNaive:

@@ -114,7 +114,19 @@ int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s, int
 int qmm_mfma_k_splits(int M, int N, int K, int L);
 // transpose=false (w [K, N*bits/32]), 4/8-bit, 16-bit types, K % 64 == 0; with
 // k_splits > 1 `a.out` points at k_splits fp32 planes as for the k-split launch.
+// `a.scales` / `a.biases` must point at [group][k] images (transpose_sb_for_qmm_n).
 int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
+size_t qmm_n_sb_bytes(int K, int G, int batches, int dtype);
+int transpose_sb_for_qmm_n(
+    const void* scales,
+    const void* biases,
+    void* out,
+    int K,
+    int G,
+    int batches,
+    int64_t src_stride,
+    int dtype,
+    hipStream_t s);
 // 1..8 rows of x on the 4x4x4 matrix instruction: transpose=true, 16-bit types,
 // 4-bit, K a multiple of 512 codes and at most 16384, an even number of groups.
 bool qmv_quad_supported(const QmmArgs& a, int gs, int bits, int dtype);

@@ -190,8 +190,10 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const int ncol = (n0 + 8 * ng < N) ? n0 + 8 * ng : N - 8; // clamp: stay in bounds
     wsrc = reinterpret_cast<const uint32_t*>(p.w) +
         static_cast<size_t>(4 * kg) * row_words + ncol / 8 * kWPR;
-    ssrc = p.scales + static_cast<size_t>(4 * kg) * groups + (ncol >> gs_shift);
-    bsrc = p.biases + static_cast<size_t>(4 * kg) * groups + (ncol >> gs_shift);
+    // scales / biases arrive transposed, [group][k] (the launcher's pre-pass): the
+    // four rows' values are 8 contiguous bytes
+    ssrc = p.scales + static_cast<size_t>(ncol >> gs_shift) * K + 4 * kg;
+    bsrc = p.biases + static_cast<size_t>(ncol >> gs_shift) * K + 4 * kg;
   } else {
     const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
     wsrc = reinterpret_cast<const uint32_t*>(p.w) +
@@ -229,7 +231,13 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 // scratch memory
 #define QMM_XQ(set, i) (*((kXSets == 2 && (set) == 1) ? &xb##i : &xa##i))
   uint32_t wreg[BITS], wnext[BITS];
-  TS sreg[kSB], breg[kSB], snext[kSB], bnext[kSB]; // converted when used, so the loads are not waited for early
+  TS sreg[1], breg[1], snext[1], bnext[1]; // converted when used, so the loads are not waited for early
+  uint2 swn, bwn, swn_next, bwn_next;      // WN: four 16-bit values each, kept raw for the same reason
+  auto wn_value = [](const uint2& v, int j) {
+    const uint32_t word = j < 2 ? v.x : v.y;
+    return to_f32(__builtin_bit_cast(TS, static_cast<
+        std::conditional_t<sizeof(TS) == 2, uint16_t, uint32_t>>(word >> (16 * (j & 1)))));
+  };
 
 #define QMM_LOAD_X(set, k0)                                                      \
   do {                                                                           \
@@ -243,14 +251,13 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   do {                                                                           \
     if constexpr (WN) {                                                          \
       const uint32_t* wp__ = wsrc + static_cast<size_t>(k0) * row_words;         \
-      const size_t g__ = static_cast<size_t>(k0) * groups;                       \
       _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
         _Pragma("unroll") for (int u__ = 0; u__ < kWPR; ++u__) {                 \
           wnext[j__ * kWPR + u__] = wp__[static_cast<size_t>(j__) * row_words + u__]; \
         }                                                                        \
-        snext[j__] = ssrc[g__ + static_cast<size_t>(j__) * groups];              \
-        bnext[j__] = bsrc[g__ + static_cast<size_t>(j__) * groups];              \
       }                                                                          \
+      swn_next = *reinterpret_cast<const uint2*>(ssrc + (k0));                   \
+      bwn_next = *reinterpret_cast<const uint2*>(bsrc + (k0));                   \
     } else {                                                                     \
       /* split mode: blocks 3t, 3t+1, 3t+2 of x all meet block t of W */         \
       const int kw__ = kSplit ? ((k0) / (3 * kBK)) * kBK : (k0);                 \
@@ -269,9 +276,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
       wreg[j__] = wnext[j__];                                                    \
     }                                                                            \
-    _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
-      sreg[j__] = snext[j__];                                                    \
-      breg[j__] = bnext[j__];                                                    \
+    sreg[0] = snext[0];                                                          \
+    breg[0] = bnext[0];                                                          \
+    if constexpr (WN) {                                                          \
+      swn = swn_next;                                                            \
+      bwn = bwn_next;                                                            \
     }                                                                            \
   } while (0)
 
@@ -291,8 +300,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     if constexpr (WN) {                                                          \
       float sf__[4], bf__[4];                                                    \
       _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
-        sf__[j__] = to_f32(sreg[j__]);                                           \
-        bf__[j__] = to_f32(breg[j__]);                                           \
+        sf__[j__] = wn_value(swn, j__);                                          \
+        bf__[j__] = wn_value(bwn, j__);                                          \
       }                                                                          \
       dequant_cols<T, BITS>(wreg, sf__, bf__, dq__);                             \
       T* col__ = &ws__[(8 * ng) * kLdsStride + 4 * kg];                          \
@@ -485,8 +494,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     T* wcol = &xs[kXTile + (8 * ng) * kLdsStride + 4 * kg];                      \
     float sf[kSB], bf[kSB];                                                      \
     _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
-      sf[j__] = to_f32(sreg[j__]);                                               \
-      bf[j__] = to_f32(breg[j__]);                                               \
+      sf[j__] = WN ? wn_value(swn, j__) : to_f32(sreg[0]);                       \
+      bf[j__] = WN ? wn_value(bwn, j__) : to_f32(breg[0]);                       \
     }                                                                            \
     /* the tile prepared in step tt is tile tt + 1: block (tt + 1) % 3 of its   \
        group of three takes the weights' low parts */                           \
@@ -680,7 +689,83 @@ int launch_wn(const QmmArgs& a, int gs_shift, int bits, dim3 grid, hipStream_t s
 
 } // namespace
 
-// transpose=false on the matrix cores: same tiles, column loader for W.
+namespace {
+
+// [K][G] -> [G][K] for scales and biases (blockIdx.z: which of the two, then
+// which batch entry), 32 x 32 tiles through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_sb_kernel(
+    const T* scales,
+    const T* biases,
+    T* out,
+    int K,
+    int G,
+    int64_t src_stride) {
+  __shared__ T tile[32][33];
+  const int which = blockIdx.z & 1;
+  const int l = blockIdx.z >> 1;
+  const T* src = (which == 0 ? scales : biases) + l * src_stride;
+  T* dst = out + (static_cast<size_t>(l) * 2 + which) * K * G;
+  const int tx = threadIdx.x & 31;
+  const int ty = threadIdx.x >> 5; // 0..7
+  const int g0 = blockIdx.x * 32;
+  const int k0 = blockIdx.y * 32;
+#pragma unroll
+  for (int r = ty; r < 32; r += 8) {
+    const int k = k0 + r;
+    const int g = g0 + tx;
+    if (k < K && g < G) {
+      tile[r][tx] = src[static_cast<size_t>(k) * G + g];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = ty; r < 32; r += 8) {
+    const int g = g0 + r;
+    const int k = k0 + tx;
+    if (k < K && g < G) {
+      dst[static_cast<size_t>(g) * K + k] = tile[tx][r];
+    }
+  }
+}
+
+} // namespace
+
+// Scratch bytes of the transposed scale / bias image of `batches` weight matrices.
+size_t qmm_n_sb_bytes(int K, int G, int batches, int dtype) {
+  return static_cast<size_t>(2) * batches * K * G * dtype_size(dtype);
+}
+
+// out: per batch entry the [G][K] scales followed by the [G][K] biases.
+int transpose_sb_for_qmm_n(
+    const void* scales,
+    const void* biases,
+    void* out,
+    int K,
+    int G,
+    int batches,
+    int64_t src_stride,
+    int dtype,
+    hipStream_t s) {
+  const dim3 grid((G + 31) / 32, (K + 31) / 32, 2 * batches);
+  if (grid.y > 65535u || grid.z > 65535u) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmm] K=%d or batch=%d exceed the grid", K, batches);
+  }
+  if (dtype == MLXROCM_BFLOAT16) {
+    transpose_sb_kernel<bf16_t><<<grid, 256, 0, s>>>(
+        static_cast<const bf16_t*>(scales), static_cast<const bf16_t*>(biases),
+        static_cast<bf16_t*>(out), K, G, src_stride);
+  } else {
+    transpose_sb_kernel<f16_t><<<grid, 256, 0, s>>>(
+        static_cast<const f16_t*>(scales), static_cast<const f16_t*>(biases),
+        static_cast<f16_t*>(out), K, G, src_stride);
+  }
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return MLXROCM_OK;
+}
+
+// transpose=false on the matrix cores: same tiles, column loader for W.  a.scales
+// / a.biases point at the transposed images made by transpose_sb_for_qmm_n.
 int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
   const int gs_shift = shift_of(gs);
   if (k_splits > 1) {

@@ -411,13 +411,21 @@ struct QuadPlan {
   int s;
 };
 
-QuadPlan quad_plan(int K, int bits) {
+QuadPlan quad_plan(int K, int bits, int M = 1) {
   const int slot_codes = 16 * (128 / bits);
   QuadPlan pl{0, 0};
   if (K % slot_codes != 0) {
     return pl;
   }
   const int need = K / slot_codes;
+  if (M > 4 && need >= 8 && need <= 32) {
+    // two operand sets of x: all eight wavefronts split K, so that a wave holds
+    // as few slices of x as possible (registers decide the occupancy here)
+    const int s8 = (need + 7) / 8;
+    pl.kw = 8;
+    pl.s = s8 == 3 ? 4 : s8;
+    return pl;
+  }
   // as many k-waves as keep at most 4 slots per wave; few slots per wave keep x
   // in few registers
   for (int kw = 1; kw <= 8; kw *= 2) {
@@ -451,7 +459,7 @@ bool qmv_quad_supported(const QmmArgs& a, int gs, int bits, int dtype) {
 }
 
 int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
-  const QuadPlan pl = quad_plan(a.K, bits);
+  const QuadPlan pl = quad_plan(a.K, bits, a.M);
   if (pl.kw == 0) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] K=%d is not covered by the quad kernel", a.K);
   }
