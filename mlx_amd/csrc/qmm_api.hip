@@ -238,6 +238,50 @@ int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hip
   return reduce_k_splits(scratch, a.out, plane, k_splits, dtype, s);
 }
 
+// Prefill (transpose=true, 16-bit types) from 512 rows of x on: the tile kernel
+// reads one scale and one bias per thread and K-step, and with the caller's
+// [N][K / group] layout every lane of such a load touches a line of its own
+// (measured: 15 % of the kernel's time).  A pre-pass transposes both arrays to
+// [K / group][N] in the stream's scratch buffer (a few MB, ~5 us), after which
+// a wavefront's 32 rows read 64 contiguous bytes.
+constexpr int kTransposeSbMinM = 512;
+
+int run_qmm_t_transposed_sb(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
+  const int G = a.K / gs;
+  const int batches = a.sb_batch_stride == 0 ? 1 : a.L;
+  const size_t sb_bytes = (qmm_n_sb_bytes(a.N, G, batches, dtype) + 255) / 256 * 256;
+  const size_t plane = static_cast<size_t>(a.M) * a.N;
+  const size_t partial_bytes = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  void* scratch = nullptr;
+  int rc = stream_scratch(s, sb_bytes + partial_bytes, &scratch);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  // rows of the source are the N rows of W, columns its G groups
+  rc = transpose_sb_for_qmm_n(
+      a.scales, a.biases, scratch, a.N, G, batches, a.sb_batch_stride, dtype, s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  const size_t image = static_cast<size_t>(a.N) * G;
+  QmmArgs part = a;
+  part.scales = scratch;
+  part.biases = static_cast<char*>(scratch) + image * dtype_size(dtype);
+  part.sb_batch_stride = batches == 1 ? 0 : static_cast<int64_t>(2 * image);
+  part.sb_transposed = 1;
+  if (k_splits <= 1) {
+    return launch_qmm_mfma(part, gs, bits, dtype, s);
+  }
+  void* partial = static_cast<char*>(scratch) + sb_bytes;
+  part.out = partial;
+  rc = launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  return reduce_k_splits(partial, a.out, plane, k_splits, dtype, s);
+}
+
 // transpose=false on the matrix cores.  The column loader wants the four
 // scales of four consecutive rows of W side by side, so scales and biases are
 // first transposed to [group][k] in the stream's scratch buffer (a few MB, a
@@ -323,11 +367,15 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   switch (choose_family(a.M, a.N, a.K, a.L, bits, dtype, transpose)) {
     case Family::QmmT:
       if (qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
+        int k_splits = 1;
         if (a.lhs_indices == nullptr && (static_cast<int64_t>(a.M) * a.N) % 4 == 0) {
-          const int k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, a.L);
-          if (k_splits > 1) {
-            return run_k_split(a, gs, bits, dtype, k_splits, s);
-          }
+          k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, a.L);
+        }
+        if (a.lhs_indices == nullptr && a.M >= kTransposeSbMinM) {
+          return run_qmm_t_transposed_sb(a, gs, bits, dtype, k_splits, s);
+        }
+        if (k_splits > 1) {
+          return run_k_split(a, gs, bits, dtype, k_splits, s);
         }
         return launch_qmm_mfma(a, gs, bits, dtype, s);
       }

@@ -34,6 +34,11 @@ struct QmmArgs {
   const int32_t* group_perm;
   const int32_t* group_ntiles;
   int group_tile_rows;
+  // Prefill tile kernel only: scales / biases point at a transposed image
+  // [K / group][N] (made by transpose_sb_for_qmm_n with the roles of K and N
+  // swapped), so that the lanes of a wavefront, which own consecutive rows of
+  // W, read consecutive values.  0: the caller's [N][K / group] arrays.
+  int sb_transposed;
 };
 
 // Resolved operand pointers of problem l.  `valid` is false when a gathered

@@ -198,9 +198,13 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
     wsrc = reinterpret_cast<const uint32_t*>(p.w) +
         static_cast<size_t>(w_row) * row_words + wh * BITS;
-    ssrc = p.scales + static_cast<size_t>(w_row) * groups;
-    bsrc = p.biases + static_cast<size_t>(w_row) * groups;
+    // group g of row w_row: [row][g], or [g][row] in the transposed image
+    const size_t sb_row = a.sb_transposed ? static_cast<size_t>(w_row)
+                                          : static_cast<size_t>(w_row) * groups;
+    ssrc = p.scales + sb_row;
+    bsrc = p.biases + sb_row;
   }
+  const size_t sb_gstride = a.sb_transposed ? static_cast<size_t>(N) : 1;
   // Rows of x past M are never stored, so they may read any valid row: the
   // loads then need no predicate.  32-bit element offsets from p.x.
   uint32_t xoff0, xoff1, xoff2, xoff3;
@@ -265,7 +269,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
       _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                   \
         wnext[j__] = wp__[j__];                                                  \
       }                                                                          \
-      const int g__ = (kw__ + 32 * wh) >> gs_shift;                              \
+      const size_t g__ = static_cast<size_t>((kw__ + 32 * wh) >> gs_shift) * sb_gstride; \
       snext[0] = ssrc[g__];                                                      \
       bnext[0] = bsrc[g__];                                                      \
     }                                                                            \
