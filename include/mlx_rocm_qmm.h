@@ -137,13 +137,15 @@ int mlxrocm_gguf_repack(
  * 0 when one weight matrix is shared by every batch (w.ndim() == 2 in MLX).
  * The kernel is picked from M, N, K, bits, group_size and dtype.
  *
- * Two kinds of call keep device scratch inside the library -- one buffer per
- * stream, allocated (hipMalloc) or grown on the first call that needs it and
- * kept until the process ends: float32 operands with M > 8 (x is split into two
- * bfloat16 parts for the matrix cores) and 16-bit calls whose tile grid would
- * leave compute units idle (K is split; fp32 partial results).  Every other
- * call allocates nothing.  A call that needs a larger buffer than the stream
- * holds synchronizes that stream before replacing it.
+ * Some calls keep device scratch inside the library -- one buffer per stream,
+ * allocated (hipMalloc) or grown on the first call that needs it and kept until
+ * the process ends: float32 operands with M > 8 (x is split into two bfloat16
+ * parts for the matrix cores); 16-bit calls whose tile grid would leave compute
+ * units idle (K is split; fp32 partial results); 16-bit prefill calls with
+ * M >= 512 and every transpose == 0 call on the matrix cores (a transposed copy
+ * of scales and biases, 4 * N * K / group_size bytes).  Decode calls (M <= 32)
+ * with transpose != 0 allocate nothing.  A call that needs a larger buffer than
+ * the stream holds synchronizes that stream before replacing it.
  */
 int mlxrocm_qmm(
     const void* x,
