@@ -5,14 +5,18 @@
 // mlx/backend/metal/quantized.cpp:1905-1923).
 //
 // Three small kernels fill a caller-provided workspace:
-//   count    one atomic per pair into counts[expert]; pairs with an index out of
-//            range are left out and their output rows are zero-filled here;
+//   count    a histogram per workgroup in LDS, then one global atomic per
+//            workgroup and expert into counts[expert] (one global atomic per
+//            pair serializes on the few counters, worst for sorted indices);
+//            pairs with an index out of range are left out and their output
+//            rows are zero-filled here;
 //   plan     one workgroup: exclusive scan of the counts -> first sorted
 //            position of every expert, and the list of tiles {expert, first
 //            position, rows} of up to tile_rows rows (256 for the tile GEMM, 32
 //            for the few-row kernel when the groups are small); the tile count
 //            stays on the device;
-//   scatter  perm[position] = pair, position handed out by a per-expert cursor.
+//   scatter  perm[position] = pair: rank inside the workgroup from an LDS
+//            counter, the workgroup's base from one atomic on a per-expert cursor.
 // The order inside an expert's run is arbitrary; every output row depends on
 // its own x row only, so the result does not depend on it.
 #include "qmm_args.h"
@@ -33,18 +37,28 @@ __global__ __launch_bounds__(256) void group_count_kernel(
     int32_t* counts,
     T* out,
     int N) {
-  const int l = blockIdx.x * blockDim.x + threadIdx.x;
-  if (l >= n_indices) {
-    return;
+  __shared__ int32_t hist[kMaxExperts];
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    hist[e] = 0;
   }
-  const uint32_t xi = lhs[l];
-  const uint32_t wi = rhs[l];
-  if (xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts)) {
-    atomicAdd(&counts[wi], 1);
-  } else {
-    T* row = out + static_cast<size_t>(l) * N;
-    for (int n = 0; n < N; ++n) {
-      row[n] = static_cast<T>(0.0f);
+  __syncthreads();
+  const int l = blockIdx.x * blockDim.x + threadIdx.x;
+  if (l < n_indices) {
+    const uint32_t xi = lhs[l];
+    const uint32_t wi = rhs[l];
+    if (xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts)) {
+      atomicAdd(&hist[wi], 1);
+    } else {
+      T* row = out + static_cast<size_t>(l) * N;
+      for (int n = 0; n < N; ++n) {
+        row[n] = static_cast<T>(0.0f);
+      }
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    if (hist[e] != 0) {
+      atomicAdd(&counts[e], hist[e]);
     }
   }
 }
@@ -96,15 +110,33 @@ __global__ __launch_bounds__(256) void group_scatter_kernel(
     const int32_t* offsets,
     int32_t* cursor,
     int32_t* perm) {
-  const int l = blockIdx.x * blockDim.x + threadIdx.x;
-  if (l >= n_indices) {
-    return;
+  __shared__ int32_t hist[kMaxExperts]; // pairs of this workgroup per expert, then its base
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    hist[e] = 0;
   }
-  const uint32_t xi = lhs[l];
-  const uint32_t wi = rhs[l];
-  if (xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts)) {
-    const int pos = offsets[wi] + atomicAdd(&cursor[wi], 1);
-    perm[pos] = l;
+  __syncthreads();
+  const int l = blockIdx.x * blockDim.x + threadIdx.x;
+  bool live = false;
+  uint32_t wi = 0;
+  int rank = 0;
+  if (l < n_indices) {
+    const uint32_t xi = lhs[l];
+    wi = rhs[l];
+    live = xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts);
+    if (live) {
+      rank = atomicAdd(&hist[wi], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    const int c = hist[e];
+    if (c != 0) {
+      hist[e] = atomicAdd(&cursor[e], c);
+    }
+  }
+  __syncthreads();
+  if (live) {
+    perm[offsets[wi] + hist[wi] + rank] = l;
   }
 }
 

@@ -350,7 +350,10 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
       return launch_qmv_quad(a, gs, bits, dtype, s);
     }
   }
-  const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype);
+  // (two rows of 8-bit codes over a long K: the streaming kernel's dot products
+  // are issue-bound there, 28 us against 20 us for the wide kernel at K = 14336)
+  const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype) ||
+      (a.M == 2 && bits == 8 && a.K > 8192);
   const bool staged = a.M > 16 || (a.M > 8 && a.N >= 8192);
   if (few_rows && !staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
     const bool gemv_better = a.M <= 8 && a.K <= 8192 && qmv_mfma_supported(a, gs, bits, dtype);
