@@ -151,6 +151,10 @@ int stream_scratch(hipStream_t s, size_t bytes, void** out) {
   return MLXROCM_OK;
 }
 
+// Rows of x from which the prefill paths transpose scales and biases first (see
+// run_qmm_t_transposed_sb).
+constexpr int kTransposeSbMinM = 512;
+
 // fp32 prefill: x is split into bf16 high/low parts in scratch, at most
 // kSplitScratchBytes of it at a time (row blocks of one batch entry), and each
 // block runs on the bf16 matrix path with fp32 scales, biases and output.
@@ -176,14 +180,29 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
   }
   const size_t x_bytes = (split_x_bytes(rows_per_block, a.K) + 255) / 256 * 256;
   const size_t plane = static_cast<size_t>(a.M) * a.N;
-  const size_t partial_bytes = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
+  const size_t partial_raw = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
+  const size_t partial_bytes = (partial_raw + 255) / 256 * 256;
+  // scales / biases transposed to [K / group][N], as for the 16-bit prefill
+  const int G = a.K / gs;
+  const int sb_batches = a.sb_batch_stride == 0 ? 1 : a.L;
+  const bool sb_t = a.M >= kTransposeSbMinM;
+  const size_t sb_bytes = sb_t ? qmm_n_sb_bytes(a.N, G, sb_batches, MLXROCM_FLOAT32) : 0;
   std::lock_guard<std::mutex> lock(g_scratch_mu);
   void* scratch = nullptr;
-  int rc = stream_scratch(s, x_bytes + partial_bytes, &scratch);
+  int rc = stream_scratch(s, x_bytes + partial_bytes + sb_bytes, &scratch);
   if (rc != MLXROCM_OK) {
     return rc;
   }
   void* partial = static_cast<char*>(scratch) + x_bytes;
+  float* sb_image = reinterpret_cast<float*>(static_cast<char*>(scratch) + x_bytes + partial_bytes);
+  const size_t image = static_cast<size_t>(a.N) * G;
+  if (sb_t) {
+    rc = transpose_sb_for_qmm_n(
+        a.scales, a.biases, sb_image, a.N, G, sb_batches, a.sb_batch_stride, MLXROCM_FLOAT32, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+  }
   for (int l = 0; l < a.L; ++l) {
     for (int m_begin = 0; m_begin < a.M; m_begin += rows_per_block) {
       const int rows = (a.M - m_begin < rows_per_block) ? a.M - m_begin : rows_per_block;
@@ -199,8 +218,15 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
       part.L = 1;
       part.x_batch_stride = static_cast<int64_t>(rows) * 3 * a.K;
       part.w = a.w + l * a.w_batch_stride;
-      part.scales = static_cast<const float*>(a.scales) + l * a.sb_batch_stride;
-      part.biases = static_cast<const float*>(a.biases) + l * a.sb_batch_stride;
+      if (sb_t) {
+        const size_t lb = sb_batches == 1 ? 0 : static_cast<size_t>(l) * 2 * image;
+        part.scales = sb_image + lb;
+        part.biases = sb_image + lb + image;
+        part.sb_transposed = 1;
+      } else {
+        part.scales = static_cast<const float*>(a.scales) + l * a.sb_batch_stride;
+        part.biases = static_cast<const float*>(a.biases) + l * a.sb_batch_stride;
+      }
       float* out = static_cast<float*>(a.out) +
           (static_cast<int64_t>(l) * a.M + m_begin) * static_cast<int64_t>(a.N);
       part.out = k_splits > 1 ? partial : out;
@@ -244,8 +270,6 @@ int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hip
 // (measured: 15 % of the kernel's time).  A pre-pass transposes both arrays to
 // [K / group][N] in the stream's scratch buffer (a few MB, ~5 us), after which
 // a wavefront's 32 rows read 64 contiguous bytes.
-constexpr int kTransposeSbMinM = 512;
-
 int run_qmm_t_transposed_sb(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
   const int G = a.K / gs;
   const int batches = a.sb_batch_stride == 0 ? 1 : a.L;

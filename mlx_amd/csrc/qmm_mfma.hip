@@ -755,7 +755,11 @@ int transpose_sb_for_qmm_n(
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] K=%d or batch=%d exceed the grid", K, batches);
   }
-  if (dtype == MLXROCM_BFLOAT16) {
+  if (dtype == MLXROCM_FLOAT32) {
+    transpose_sb_kernel<float><<<grid, 256, 0, s>>>(
+        static_cast<const float*>(scales), static_cast<const float*>(biases),
+        static_cast<float*>(out), K, G, src_stride);
+  } else if (dtype == MLXROCM_BFLOAT16) {
     transpose_sb_kernel<bf16_t><<<grid, 256, 0, s>>>(
         static_cast<const bf16_t*>(scales), static_cast<const bf16_t*>(biases),
         static_cast<bf16_t*>(out), K, G, src_stride);
