@@ -417,6 +417,9 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
       if (qmv_mfma_supported(a, gs, bits, dtype)) {
         return launch_qmv_mfma(a, gs, bits, dtype, s);
       }
+      if (qmv_f32_supported(a, gs, bits, dtype)) {
+        return launch_qmv_f32(a, gs, bits, s);
+      }
       return launch_qmv_generic(a, gs, bits, dtype, s);
     case Family::QmmN:
       if (a.lhs_indices == nullptr && qmm_mfma_supported(a, gs, bits, dtype, transpose)) {

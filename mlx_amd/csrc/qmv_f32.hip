@@ -1,0 +1,228 @@
+// qmv_f32.hip -- decode GEMV (transpose=true) for float32 operands, every code
+// width, one row of x: a streaming kernel in plain fp32 arithmetic.
+//
+// A lane owns 32 consecutive codes of a row (= `bits` whole dwords for every
+// width, and never more than one quantization group), so a wavefront covers a
+// "chunk" of 2048 codes with `bits` dword loads per lane whose addresses are
+// contiguous across the lanes.  The K axis is split over KW wavefronts of the
+// workgroup, CPW chunks each; every wavefront keeps its slices of x in
+// registers (fetched once, straight from global memory: x is small and shared by
+// every workgroup, so it stays in the caches) and walks over kRowsInFlight rows
+// of W at a time with all their loads issued before the first is consumed.  Per
+// lane and chunk the affine part is applied once: y += s * dot(q, x) + b * sum(x).
+// Lanes are added with DPP / permutes, k-waves through LDS.
+#include "mfma_dequant.h"
+#include "qmm_args.h"
+
+namespace mlxrocm {
+
+namespace {
+
+constexpr int kF32ChunkCodes = 64 * 32;
+constexpr int kF32RowsInFlight = 4;
+constexpr int kF32Threads = 256;
+
+template <int BITS, int MROWS, int CPW, int KW>
+__global__ __launch_bounds__(kF32Threads) void qmv_f32_kernel(const QmmArgs a, const int gs_shift) {
+  constexpr int RW = kF32Threads / 64 / KW; // row-waves per workgroup
+  __shared__ float red[kF32Threads / 64][kF32RowsInFlight][MROWS];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kw = wave % KW;
+  const int rw = wave / KW;
+  const int K = a.K;
+  const int N = a.N;
+  const QmmProblem<float> p = resolve_problem<float>(a, blockIdx.y);
+  const int groups = K >> gs_shift;
+  const int row_words = K / 32 * BITS;
+
+  // this lane's codes of chunk c: k in [k_of(c), k_of(c) + 32)
+  int kpos[CPW];
+  bool live[CPW];
+#pragma unroll
+  for (int c = 0; c < CPW; ++c) {
+    const int k = (kw * CPW + c) * kF32ChunkCodes + lane * 32;
+    live[c] = k < K; // K is a multiple of 32
+    kpos[c] = live[c] ? k : 0;
+  }
+  // x slices and their sums
+  float xr[MROWS][CPW][32];
+  float sx[MROWS][CPW];
+#pragma unroll
+  for (int m = 0; m < MROWS; ++m) {
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const float* src = p.x + static_cast<size_t>(m < a.M ? m : 0) * K + kpos[c];
+      float s = 0.0f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        float4 v = *reinterpret_cast<const float4*>(src + 4 * u);
+        if (!live[c] || m >= a.M) {
+          v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+        xr[m][c][4 * u + 0] = v.x;
+        xr[m][c][4 * u + 1] = v.y;
+        xr[m][c][4 * u + 2] = v.z;
+        xr[m][c][4 * u + 3] = v.w;
+        s += (v.x + v.y) + (v.z + v.w);
+      }
+      sx[m][c] = s;
+    }
+  }
+
+  const int rows_per_wg = RW * kF32RowsInFlight;
+  const int row0 = blockIdx.x * rows_per_wg + rw * kF32RowsInFlight;
+  uint32_t wv[kF32RowsInFlight][CPW][BITS];
+  float sv[kF32RowsInFlight][CPW], bv[kF32RowsInFlight][CPW];
+#pragma unroll
+  for (int r = 0; r < kF32RowsInFlight; ++r) {
+    const int row = row0 + r < N ? row0 + r : N - 1; // clamp: stay in bounds
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const int g = kpos[c] >> gs_shift;
+      sv[r][c] = p.scales[static_cast<size_t>(row) * groups + g];
+      bv[r][c] = p.biases[static_cast<size_t>(row) * groups + g];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < kF32RowsInFlight; ++r) {
+    const int row = row0 + r < N ? row0 + r : N - 1;
+    const uint32_t* wrow = reinterpret_cast<const uint32_t*>(p.w) +
+        static_cast<size_t>(row) * row_words;
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const uint32_t* src = wrow + kpos[c] / 32 * BITS;
+#pragma unroll
+      for (int j = 0; j < BITS; ++j) {
+        wv[r][c][j] = __builtin_nontemporal_load(src + j);
+      }
+    }
+  }
+
+  float y[kF32RowsInFlight][MROWS];
+#pragma unroll
+  for (int r = 0; r < kF32RowsInFlight; ++r) {
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+      y[r][m] = 0.0f;
+    }
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      float dot[MROWS];
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) {
+        dot[m] = 0.0f;
+      }
+#pragma unroll
+      for (int e = 0; e < 32; ++e) {
+        const float q = static_cast<float>(code32<BITS>(wv[r][c], e));
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) {
+          dot[m] = fmaf(q, xr[m][c][e], dot[m]);
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) {
+        y[r][m] = fmaf(sv[r][c], dot[m], y[r][m]);
+        y[r][m] = fmaf(bv[r][c], sx[m][c], y[r][m]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < kF32RowsInFlight; ++r) {
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+      const float total = wave_sum(y[r][m]);
+      if (lane == 0) {
+        red[wave][r][m] = total;
+      }
+    }
+  }
+  __syncthreads();
+  if (tid < RW * kF32RowsInFlight * MROWS) {
+    const int m = tid % MROWS;
+    const int r = (tid / MROWS) % kF32RowsInFlight;
+    const int w = tid / (MROWS * kF32RowsInFlight);
+    float total = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KW; ++k) {
+      total += red[w * KW + k][r][m];
+    }
+    const int row = blockIdx.x * rows_per_wg + w * kF32RowsInFlight + r;
+    if (row < N && m < a.M) {
+      p.out[static_cast<size_t>(m) * N + row] = p.valid ? total : 0.0f;
+    }
+  }
+}
+
+struct F32Plan {
+  int kw; // 0: not covered
+  int cpw;
+};
+
+F32Plan f32_plan(int K) {
+  const int need = (K + kF32ChunkCodes - 1) / kF32ChunkCodes;
+  F32Plan pl{0, 0};
+  if (need <= 1) {
+    pl = {1, 1};
+  } else if (need <= 2) {
+    pl = {1, 2};
+  } else if (need <= 4) {
+    pl = {2, 2};
+  } else if (need <= 8) {
+    pl = {4, 2};
+  }
+  return pl;
+}
+
+} // namespace
+
+bool qmv_f32_supported(const QmmArgs& a, int gs, int bits, int dtype) {
+  (void)gs;
+  (void)bits;
+  // one row of x: a second one doubles the registers that hold x (the kernel is
+  // written for it, the dispatch is not)
+  if (dtype != MLXROCM_FLOAT32 || a.M != 1) {
+    return false;
+  }
+  return f32_plan(a.K).kw != 0; // K <= 16384
+}
+
+int launch_qmv_f32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
+  const F32Plan pl = f32_plan(a.K);
+  if (pl.kw == 0) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmv] K=%d is not covered by the fp32 GEMV", a.K);
+  }
+  const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
+  const int rows_per_wg = (kF32Threads / 64 / pl.kw) * kF32RowsInFlight;
+  const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.L);
+  if (grid.y > 65535u) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmv] batch=%d exceeds the grid", a.L);
+  }
+  auto go = [&](auto bval, auto mval, auto cval, auto kval) -> int {
+    constexpr int B = decltype(bval)::value;
+    constexpr int M = decltype(mval)::value;
+    constexpr int C = decltype(cval)::value;
+    constexpr int KWv = decltype(kval)::value;
+    qmv_f32_kernel<B, M, C, KWv><<<grid, kF32Threads, 0, s>>>(a, gs_shift);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
+  };
+  auto by_plan = [&](auto bval, auto mval) -> int {
+    if (pl.kw == 1 && pl.cpw == 1) {
+      return go(bval, mval, IntC<1>{}, IntC<1>{});
+    }
+    if (pl.kw == 1) {
+      return go(bval, mval, IntC<2>{}, IntC<1>{});
+    }
+    if (pl.kw == 2) {
+      return go(bval, mval, IntC<2>{}, IntC<2>{});
+    }
+    return go(bval, mval, IntC<2>{}, IntC<4>{});
+  };
+  return dispatch_bits(bits, [&](auto bval) { return by_plan(bval, IntC<1>{}); });
+}
+
+} // namespace mlxrocm

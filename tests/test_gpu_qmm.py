@@ -253,3 +253,13 @@ def test_qmv_matrix_instruction_gemv_batched(oracle, gpu):
         exact = x[l].double() @ w_hat.T
         tol = matmul_tolerance(dtype, K, x[l], w_hat) + float((ref.double() - exact).abs().max())
         assert float((got[l].double() - ref.double()).abs().max()) <= tol
+
+
+@pytest.mark.parametrize("bits", ALL_BITS)
+def test_qmv_float32_streaming(oracle, gpu, bits):
+    """One row of float32 x runs on the fp32 streaming GEMV: K of a partial chunk,
+    of several k-waves with an unused tail (11008), ragged N, every group size."""
+    for gs, N, K in ((32, 67, 2080), (64, 40, 11008), (128, 130, 4096), (32, 9, 16384)):
+        w = normal_weights((N, K), torch.float32, seed=bits + gs)
+        x = activations((1, K), torch.float32, seed=K)
+        _check_qmm(oracle, gpu, x, w, gs, bits)
