@@ -379,6 +379,11 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype) ||
       (a.M == 2 && bits == 8 && a.K > 8192);
   const bool staged = a.M > 16 || (a.M > 8 && a.N >= 8192);
+  // one row at a width the row-streaming GEMV does not cover (2/3/5/6 bits): the
+  // fp32-arithmetic streaming kernel
+  if (transpose && a.M == 1 && few_rows && qmv_f32_supported(a, gs, bits, dtype)) {
+    return launch_qmv_f32(a, gs, bits, dtype, s);
+  }
   if (few_rows && !staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
     const bool gemv_better = a.M <= 8 && a.K <= 8192 && qmv_mfma_supported(a, gs, bits, dtype);
     if (!gemv_better) {
@@ -418,7 +423,7 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
         return launch_qmv_mfma(a, gs, bits, dtype, s);
       }
       if (qmv_f32_supported(a, gs, bits, dtype)) {
-        return launch_qmv_f32(a, gs, bits, s);
+        return launch_qmv_f32(a, gs, bits, dtype, s);
       }
       return launch_qmv_generic(a, gs, bits, dtype, s);
     case Family::QmmN:

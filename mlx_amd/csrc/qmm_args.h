@@ -132,9 +132,10 @@ int transpose_sb_for_qmm_n(
     int64_t src_stride,
     int dtype,
     hipStream_t s);
-// float32 decode GEMV (transpose=true), every width, one row of x, K <= 16384.
+// decode GEMV in fp32 arithmetic (transpose=true): every width and element type,
+// one row of x, K <= 16384.
 bool qmv_f32_supported(const QmmArgs& a, int gs, int bits, int dtype);
-int launch_qmv_f32(const QmmArgs& a, int gs, int bits, hipStream_t s);
+int launch_qmv_f32(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 // 1..8 rows of x on the 4x4x4 matrix instruction: transpose=true, 16-bit types,
 // 4-bit, K a multiple of 512 codes and at most 16384, an even number of groups.
 bool qmv_quad_supported(const QmmArgs& a, int gs, int bits, int dtype);

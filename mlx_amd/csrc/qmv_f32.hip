@@ -1,5 +1,6 @@
-// qmv_f32.hip -- decode GEMV (transpose=true) for float32 operands, every code
-// width, one row of x: a streaming kernel in plain fp32 arithmetic.
+// qmv_f32.hip -- decode GEMV (transpose=true) in plain fp32 arithmetic, every
+// code width and element type, one row of x: the streaming kernel for float32
+// operands and for the 16-bit types at widths 2/3/5/6.
 //
 // A lane owns 32 consecutive codes of a row (= `bits` whole dwords for every
 // width, and never more than one quantization group), so a wavefront covers a
@@ -22,7 +23,34 @@ constexpr int kF32ChunkCodes = 64 * 32;
 constexpr int kF32RowsInFlight = 4;
 constexpr int kF32Threads = 256;
 
-template <int BITS, int MROWS, int CPW, int KW>
+// 32 consecutive elements of x as floats.
+__device__ __forceinline__ void load_x32(const float* src, float (&out)[32]) {
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const float4 v = *reinterpret_cast<const float4*>(src + 4 * u);
+    out[4 * u + 0] = v.x;
+    out[4 * u + 1] = v.y;
+    out[4 * u + 2] = v.z;
+    out[4 * u + 3] = v.w;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void load_x32(const T* src, float (&out)[32]) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    union {
+      uint4 v;
+      T h[8];
+    } r;
+    r.v = *reinterpret_cast<const uint4*>(src + 8 * u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      out[8 * u + e] = to_f32(r.h[e]);
+    }
+  }
+}
+
+template <typename T, int BITS, int MROWS, int CPW, int KW>
 __global__ __launch_bounds__(kF32Threads) void qmv_f32_kernel(const QmmArgs a, const int gs_shift) {
   constexpr int RW = kF32Threads / 64 / KW; // row-waves per workgroup
   __shared__ float red[kF32Threads / 64][kF32RowsInFlight][MROWS];
@@ -33,7 +61,7 @@ __global__ __launch_bounds__(kF32Threads) void qmv_f32_kernel(const QmmArgs a, c
   const int rw = wave / KW;
   const int K = a.K;
   const int N = a.N;
-  const QmmProblem<float> p = resolve_problem<float>(a, blockIdx.y);
+  const QmmProblem<T> p = resolve_problem<T>(a, blockIdx.y);
   const int groups = K >> gs_shift;
   const int row_words = K / 32 * BITS;
 
@@ -53,19 +81,14 @@ __global__ __launch_bounds__(kF32Threads) void qmv_f32_kernel(const QmmArgs a, c
   for (int m = 0; m < MROWS; ++m) {
 #pragma unroll
     for (int c = 0; c < CPW; ++c) {
-      const float* src = p.x + static_cast<size_t>(m < a.M ? m : 0) * K + kpos[c];
+      load_x32(p.x + static_cast<size_t>(m < a.M ? m : 0) * K + kpos[c], xr[m][c]);
       float s = 0.0f;
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        float4 v = *reinterpret_cast<const float4*>(src + 4 * u);
+      for (int e = 0; e < 32; ++e) {
         if (!live[c] || m >= a.M) {
-          v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          xr[m][c][e] = 0.0f;
         }
-        xr[m][c][4 * u + 0] = v.x;
-        xr[m][c][4 * u + 1] = v.y;
-        xr[m][c][4 * u + 2] = v.z;
-        xr[m][c][4 * u + 3] = v.w;
-        s += (v.x + v.y) + (v.z + v.w);
+        s += xr[m][c][e];
       }
       sx[m][c] = s;
     }
@@ -74,7 +97,7 @@ __global__ __launch_bounds__(kF32Threads) void qmv_f32_kernel(const QmmArgs a, c
   const int rows_per_wg = RW * kF32RowsInFlight;
   const int row0 = blockIdx.x * rows_per_wg + rw * kF32RowsInFlight;
   uint32_t wv[kF32RowsInFlight][CPW][BITS];
-  float sv[kF32RowsInFlight][CPW], bv[kF32RowsInFlight][CPW];
+  T sv[kF32RowsInFlight][CPW], bv[kF32RowsInFlight][CPW];
 #pragma unroll
   for (int r = 0; r < kF32RowsInFlight; ++r) {
     const int row = row0 + r < N ? row0 + r : N - 1; // clamp: stay in bounds
@@ -124,8 +147,8 @@ __global__ __launch_bounds__(kF32Threads) void qmv_f32_kernel(const QmmArgs a, c
       }
 #pragma unroll
       for (int m = 0; m < MROWS; ++m) {
-        y[r][m] = fmaf(sv[r][c], dot[m], y[r][m]);
-        y[r][m] = fmaf(bv[r][c], sx[m][c], y[r][m]);
+        y[r][m] = fmaf(to_f32(sv[r][c]), dot[m], y[r][m]);
+        y[r][m] = fmaf(to_f32(bv[r][c]), sx[m][c], y[r][m]);
       }
     }
   }
@@ -152,7 +175,7 @@ __global__ __launch_bounds__(kF32Threads) void qmv_f32_kernel(const QmmArgs a, c
     }
     const int row = blockIdx.x * rows_per_wg + w * kF32RowsInFlight + r;
     if (row < N && m < a.M) {
-      p.out[static_cast<size_t>(m) * N + row] = p.valid ? total : 0.0f;
+      p.out[static_cast<size_t>(m) * N + row] = from_f32<T>(p.valid ? total : 0.0f);
     }
   }
 }
@@ -184,13 +207,14 @@ bool qmv_f32_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   (void)bits;
   // one row of x: a second one doubles the registers that hold x (the kernel is
   // written for it, the dispatch is not)
-  if (dtype != MLXROCM_FLOAT32 || a.M != 1) {
+  (void)dtype;
+  if (a.M != 1) {
     return false;
   }
   return f32_plan(a.K).kw != 0; // K <= 16384
 }
 
-int launch_qmv_f32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
+int launch_qmv_f32(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
   const F32Plan pl = f32_plan(a.K);
   if (pl.kw == 0) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] K=%d is not covered by the fp32 GEMV", a.K);
@@ -201,28 +225,31 @@ int launch_qmv_f32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] batch=%d exceeds the grid", a.L);
   }
-  auto go = [&](auto bval, auto mval, auto cval, auto kval) -> int {
+  auto go = [&](auto tval, auto bval, auto mval, auto cval, auto kval) -> int {
+    using T = decltype(tval);
     constexpr int B = decltype(bval)::value;
     constexpr int M = decltype(mval)::value;
     constexpr int C = decltype(cval)::value;
     constexpr int KWv = decltype(kval)::value;
-    qmv_f32_kernel<B, M, C, KWv><<<grid, kF32Threads, 0, s>>>(a, gs_shift);
+    qmv_f32_kernel<T, B, M, C, KWv><<<grid, kF32Threads, 0, s>>>(a, gs_shift);
     MLXROCM_HIP_TRY(hipGetLastError());
     return static_cast<int>(MLXROCM_OK);
   };
-  auto by_plan = [&](auto bval, auto mval) -> int {
+  auto by_plan = [&](auto tval, auto bval, auto mval) -> int {
     if (pl.kw == 1 && pl.cpw == 1) {
-      return go(bval, mval, IntC<1>{}, IntC<1>{});
+      return go(tval, bval, mval, IntC<1>{}, IntC<1>{});
     }
     if (pl.kw == 1) {
-      return go(bval, mval, IntC<2>{}, IntC<1>{});
+      return go(tval, bval, mval, IntC<2>{}, IntC<1>{});
     }
     if (pl.kw == 2) {
-      return go(bval, mval, IntC<2>{}, IntC<2>{});
+      return go(tval, bval, mval, IntC<2>{}, IntC<2>{});
     }
-    return go(bval, mval, IntC<2>{}, IntC<4>{});
+    return go(tval, bval, mval, IntC<2>{}, IntC<4>{});
   };
-  return dispatch_bits(bits, [&](auto bval) { return by_plan(bval, IntC<1>{}); });
+  return dispatch_dtype(dtype, [&](auto tval) {
+    return dispatch_bits(bits, [&](auto bval) { return by_plan(tval, bval, IntC<1>{}); });
+  });
 }
 
 } // namespace mlxrocm
