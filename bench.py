@@ -252,6 +252,31 @@ def sweep(torch, mlx_amd, dev) -> list:
         ms = timed(lambda i: mlx_amd.gather_qmm(xs, wq, sc, bi, rhs_indices=fs, transpose=True,
                                                 group_size=64, bits=4, sorted_indices=True))
         add("cfg4", f"gather T={T} top-2 of 8, sorted", ms, flops=4.0 * T * n * k)
+        # the same unsorted call through the C ABI (no Python operator in the loop)
+        from mlx_amd import _lib
+        lib = _lib.load()
+        n_idx = 2 * T
+        lhs_u = torch.arange(T, device=dev).repeat_interleave(2).to(torch.uint32).contiguous()
+        rhs_u = idx.reshape(-1).to(torch.uint32).contiguous()
+        xb = x.reshape(T, 1, k).contiguous()
+        out = torch.empty((n_idx, 1, n), dtype=bf16, device=dev)
+        ws_bytes = lib.mlxrocm_gather_qmm_workspace_size(1, n, k, n_idx, E, 64, 4, 2, 1, 0)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+
+        def gstep(i, stream):
+            rc = lib.mlxrocm_gather_qmm(
+                xb.data_ptr(), wq.data_ptr(), sc.data_ptr(), bi.data_ptr(), lhs_u.data_ptr(),
+                rhs_u.data_ptr(), out.data_ptr(), 1, n, k, n_idx, T, E, k, wq.stride(0),
+                sc.stride(0), 64, 4, 2, 1, 0, ws.data_ptr() if ws_bytes else None, ws_bytes, stream)
+            if rc != 0:
+                raise RuntimeError(_lib.last_error())
+
+        small = T <= 64
+        launcher = Launcher(torch, gstep, 4, small)
+        launcher.run(4)
+        torch.cuda.synchronize()
+        ms = hip_event_ms(lib, launcher, 40 if small else 10)
+        add("cfg4", f"gather T={T} top-2 of 8, unsorted, C ABI" + (" (2 experts, cache-resident)" if T == 1 else ""), ms, flops=4.0 * T * n * k)
     del wq, sc, bi
     # Cfg5: odd code widths, group 32, Llama-2-7B MLP shapes
     for dtype in (bf16, f32):
