@@ -144,4 +144,17 @@ int launch_qmm_mfma_ksplit(const QmmArgs& a, int gs, int bits, int dtype, int k_
 int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int dtype, hipStream_t s);
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 
+// Compute units of the current device (read once).
+inline int compute_units() {
+  static int cus = [] {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+      return 256;
+    }
+    return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }();
+  return cus;
+}
+
 } // namespace mlxrocm

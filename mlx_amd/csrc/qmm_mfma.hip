@@ -612,18 +612,6 @@ constexpr size_t qmm_smem_bytes() {
   return stages > out ? stages : out;
 }
 
-int compute_units() {
-  static int cus = [] {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
-      return 256;
-    }
-    return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-  }();
-  return cus;
-}
-
 // Tile width (in units of 32 columns) that finishes first: a workgroup needs
 // time ~ NT per tile and the tiles run in ceil(tiles / CUs) rounds.
 int choose_nt(int M, int N, int L) {

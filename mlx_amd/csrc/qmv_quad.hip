@@ -105,15 +105,16 @@ __device__ __forceinline__ float sum_blocks(float v, int lane) {
   return v;
 }
 
-constexpr int kQuadsPerWave = 4; // row quads whose loads are in flight together
 
 // MB: operand sets of x (rows 0..3, 4..7).  S: slots (one 16-byte load per lane
 // each) of K per wavefront.  KW: wavefronts that split K.
 // XLDS: x reaches the lanes through one coalesced read per workgroup and LDS
 // (4 MB K elements of LDS); otherwise every lane fetches its slices itself.
 // MC: columns of an operand set that are live (rows of x: M = 1, 2, or more).
-template <typename T, int BITS, int MB, int S, int KW, int kSbLoads, bool XLDS, int MC>
+// QPW: row quads per wave, whose loads are in flight together.
+template <typename T, int BITS, int MB, int S, int KW, int kSbLoads, bool XLDS, int MC, int QPW>
 __global__ __launch_bounds__(512) void qmv_quad_kernel(const QmmArgs a, const int gs_shift) {
+  constexpr int kQuadsPerWave = QPW;
   constexpr int RW = 8 / KW;
   constexpr int kLaneCodes = 128 / BITS;      // codes in a lane's 16 bytes
   constexpr int kSlotCodes = 16 * kLaneCodes; // 512 or 256 codes of k per load instruction
@@ -465,17 +466,28 @@ int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
   }
   const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
   const int rw = 8 / pl.kw;
-  const int rows_per_wg = rw * kQuadsPerWave * 4;
+  const int mb = a.M <= 4 ? 1 : 2;
+  const size_t x_bytes = static_cast<size_t>(4 * mb) * a.K * 2;
+  // x through LDS while a few workgroups still fit a compute unit
+  const bool xlds = x_bytes + 8 * 4 * mb * 16 * sizeof(float) <= 64 * 1024 &&
+      static_cast<size_t>(a.M) * (a.K / 8) <= static_cast<size_t>(4 * mb) * 512;
+  // Row quads per wave: four keep the most loads in flight, but a small N then
+  // leaves compute units without a workgroup.  Measured at K = 4096 (two
+  // row-waves): 1024 rows 5.6 -> 3.4 us, 4096 rows 6.2 -> 4.7, 11008 rows
+  // 9.3 -> 8.1 with fewer quads; from ~1.5 workgroups per unit on four quads win.
+  int qpw = 4;
+  if (mb == 1 && xlds && pl.kw <= 4) {
+    const long want = compute_units() * 3L / 2;
+    while (qpw > 1 && static_cast<long>((a.N + rw * qpw * 4 - 1) / (rw * qpw * 4)) * a.L < want) {
+      qpw /= 2;
+    }
+  }
+  const int rows_per_wg = rw * qpw * 4;
   const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.L);
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] batch=%d exceeds the grid", a.L);
   }
-  const int mb = a.M <= 4 ? 1 : 2;
-  const size_t red_bytes = static_cast<size_t>(8) * kQuadsPerWave * mb * 16 * sizeof(float);
-  const size_t x_bytes = static_cast<size_t>(4 * mb) * a.K * 2;
-  // x through LDS while a few workgroups still fit a compute unit
-  const bool xlds = x_bytes + red_bytes <= 64 * 1024 &&
-      static_cast<size_t>(a.M) * (a.K / 8) <= static_cast<size_t>(4 * mb) * 512;
+  const size_t red_bytes = static_cast<size_t>(8) * qpw * mb * 16 * sizeof(float);
   const size_t smem = red_bytes + (xlds ? x_bytes : 0);
   // dwords of scales per row and wave, eight per load
   const int sb_words = pl.s * 16 * (128 / bits) / gs / 2;
@@ -498,21 +510,32 @@ int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
       MLXROCM_HIP_TRY(hipGetLastError());
       return static_cast<int>(MLXROCM_OK);
     };
+    auto by_qpw = [&](auto f) -> int {
+      if constexpr (MB == 1 && KW <= 4) {
+        if (qpw == 1) {
+          return f(IntC<1>{});
+        }
+        if (qpw == 2) {
+          return f(IntC<2>{});
+        }
+      }
+      return f(IntC<4>{});
+    };
     if (xlds) {
       // the x image needs whole slots: S * KW covers K exactly or x is zero there
       if (sb_loads == 1) {
-        return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, true, MC>);
+        return by_qpw([&](auto qv) { return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, true, MC, decltype(qv)::value>); });
       } else if (sb_loads == 2) {
-        return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, true, MC>);
+        return by_qpw([&](auto qv) { return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, true, MC, decltype(qv)::value>); });
       }
-      return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, true, MC>);
+      return by_qpw([&](auto qv) { return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, true, MC, decltype(qv)::value>); });
     }
     if (sb_loads == 1) {
-      return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, false, MC>);
+      return launch(qmv_quad_kernel<T, B, MB, S, KW, 1, false, MC, 4>);
     } else if (sb_loads == 2) {
-      return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, false, MC>);
+      return launch(qmv_quad_kernel<T, B, MB, S, KW, 2, false, MC, 4>);
     }
-    return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, false, MC>);
+    return launch(qmv_quad_kernel<T, B, MB, S, KW, 4, false, MC, 4>);
   };
   auto by_mc = [&](auto tval, auto bval, auto mbv, auto sval, auto kwv) -> int {
     if constexpr (decltype(mbv)::value == 1) {

@@ -30,6 +30,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kChunkBytes = 1024; // 64 lanes x 16 bytes
+constexpr int kChains = 2; // independent accumulators per 16-byte load
 
 template <typename T>
 struct Dot;
@@ -130,6 +131,14 @@ __device__ __forceinline__ uint4 load_streaming(const uint8_t* p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// x + the value of the lane that a quad permutation pairs this lane with.
+template <int CTRL>
+__device__ __forceinline__ float quad_add(float x) {
+  const int moved = __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false);
+  return x + __builtin_bit_cast(float, moved);
+}
+
 // Sum of all 64 lanes, valid in lane 63 (DPP: two quad swaps, two mirrors,
 // then row broadcasts across the four rows of 16).
 __device__ __forceinline__ float wave_sum_dpp(float v) {
@@ -152,11 +161,11 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 // KW: waves that split K between them; RW: row-waves; the workgroup owns
 // RW * kRowsPerWave rows.  M is 1 or 2.  FULL: K is exactly KW * CPW chunks, so
 // no lane ever falls outside a row and the loads carry no predicate.
-template <typename T, int BITS, int GS, int M, int RW, int KW, bool FULL>
+template <typename T, int BITS, int GS, int M, int RW, int KW, bool FULL, int RM = 1>
 __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs a) {
   using S = StreamShape<BITS, GS>;
   constexpr int CPW = S::kChunksPerWave;
-  constexpr int kRowsPerWave = S::kRowsPerWave;
+  constexpr int kRowsPerWave = S::kRowsPerWave * RM;
   constexpr int kThreads = RW * KW * 64;
   constexpr float kOffset = (BITS == 4) ? Dot<T>::kOffset4 : Dot<T>::kOffset8;
   static_assert(GS >= S::kLaneCodes, "a lane's 16 bytes stay inside one group");
@@ -180,8 +189,12 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
   const int x_units = M * (K / 8); // 16-byte units
   const uint8_t* xbytes = reinterpret_cast<const uint8_t*>(p.x);
   uint4 xv0 = make_uint4(0, 0, 0, 0);
+  uint4 xv1 = make_uint4(0, 0, 0, 0);
   if (tid < x_units) {
     xv0 = *reinterpret_cast<const uint4*>(xbytes + static_cast<uint32_t>(tid) * 16);
+  }
+  if (tid + kThreads < x_units) {
+    xv1 = *reinterpret_cast<const uint4*>(xbytes + static_cast<uint32_t>(tid + kThreads) * 16);
   }
 
   // ---- 2. every weight / scale / bias load of this wave ----
@@ -250,6 +263,7 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
   constexpr int P = S::kLaneCodes / 8;
   const int nchunks = (K + S::kChunkCodes - 1) / S::kChunkCodes;
   const uint32_t xrow_bytes = static_cast<uint32_t>(nchunks) * P * 64 * 16;
+  float* sx_lds = reinterpret_cast<float*>(smem + M * xrow_bytes); // [M][nchunks][64]
   auto stage_x = [&](int idx, const uint4& v) {
     const int m = idx / (K / 8);
     const int e = idx - m * (K / 8); // 8-element unit index inside the row
@@ -266,13 +280,30 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
     }
     *reinterpret_cast<uint4*>(
         smem + m * xrow_bytes + ((static_cast<uint32_t>(c) * P + t) * 64 + l) * 16) = o;
+    // sum of the P pieces that one lane of a chunk will hold: the P threads
+    // that stage them are neighbours (idx % P == tid % P), so two quad swaps
+    // finish it, and every wave reads the sum instead of recomputing it
+    float part = Dot<T>::dot2(v.x, Dot<T>::kOnes, 0.0f);
+    part = Dot<T>::dot2(v.y, Dot<T>::kOnes, part);
+    part = Dot<T>::dot2(v.z, Dot<T>::kOnes, part);
+    part = Dot<T>::dot2(v.w, Dot<T>::kOnes, part);
+    part = quad_add<0xB1>(part); // quad_perm [1,0,3,2]
+    if constexpr (P == 4) {
+      part = quad_add<0x4E>(part); // quad_perm [2,3,0,1]
+    }
+    if (t == 0) {
+      sx_lds[(m * nchunks + c) * 64 + l] = part;
+    }
   };
   if (tid < x_units) {
     stage_x(tid, xv0);
   }
-  // longer x (K > 4096 elements per 512 threads, or M = 2): the remaining
-  // units follow the weight loads in the queue
-  for (int idx = tid + kThreads; idx < x_units; idx += kThreads) {
+  if (tid + kThreads < x_units) {
+    stage_x(tid + kThreads, xv1);
+  }
+  // longer x (more than 16 bytes x 2 per thread): the remaining units follow
+  // the weight loads in the queue
+  for (int idx = tid + 2 * kThreads; idx < x_units; idx += kThreads) {
     stage_x(idx, *reinterpret_cast<const uint4*>(xbytes + static_cast<uint32_t>(idx) * 16));
   }
   __syncthreads();
@@ -285,7 +316,6 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
     for (int c = 0; c < CPW; ++c) {
       const bool live = FULL ||
           (static_cast<uint32_t>(c0 + c) * kChunkBytes + lane * 16) < row_bytes;
-      float s = 0.0f;
 #pragma unroll
       for (int t = 0; t < P; ++t) {
         uint4 v;
@@ -305,12 +335,8 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
         xr[m][c][4 * t + 1] = v.y;
         xr[m][c][4 * t + 2] = v.z;
         xr[m][c][4 * t + 3] = v.w;
-        s = Dot<T>::dot2(v.x, Dot<T>::kOnes, s);
-        s = Dot<T>::dot2(v.y, Dot<T>::kOnes, s);
-        s = Dot<T>::dot2(v.z, Dot<T>::kOnes, s);
-        s = Dot<T>::dot2(v.w, Dot<T>::kOnes, s);
       }
-      sx[m][c] = s;
+      sx[m][c] = live ? sx_lds[(m * nchunks + c0 + c) * 64 + lane] : 0.0f;
     }
   }
 
@@ -332,7 +358,7 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
       for (int d = 0; d < 4; ++d) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-          dacc[m][d] = 0.0f;
+          dacc[m][d] = (d < kChains) ? 0.0f : dacc[m][d >= kChains ? d - kChains : 0];
         }
         if constexpr (BITS == 4) {
           const uint32_t q0 = (w[d] & w4c.mask) | w4c.magic;
@@ -358,7 +384,13 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
       float dot[M];
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        dot[m] = (dacc[m][0] + dacc[m][1]) + (dacc[m][2] + dacc[m][3]);
+        if constexpr (kChains == 4) {
+          dot[m] = (dacc[m][0] + dacc[m][1]) + (dacc[m][2] + dacc[m][3]);
+        } else if constexpr (kChains == 2) {
+          dot[m] = dacc[m][2] + dacc[m][3];
+        } else {
+          dot[m] = dacc[m][3];
+        }
       }
       const uint32_t s_word = static_cast<uint32_t>(
           __builtin_amdgcn_ds_bpermute(sb_src[c], static_cast<int>(sbw[r])));
@@ -426,11 +458,13 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
 }
 
 template <int BITS, int GS>
-size_t stream_smem_bytes(int M, int K, int rw, int kw) {
+size_t stream_smem_bytes(int M, int K, int rw, int kw, int rm) {
   using S = StreamShape<BITS, GS>;
-  constexpr int kRowsPerWave = S::kRowsPerWave;
+  const int kRowsPerWave = S::kRowsPerWave * rm;
   const int nchunks = (K + S::kChunkCodes - 1) / S::kChunkCodes;
-  const size_t x_bytes = static_cast<size_t>(M) * nchunks * (S::kLaneCodes / 8) * 64 * 16;
+  // the staged x image, then one partial sum of x per lane and chunk
+  const size_t x_bytes = static_cast<size_t>(M) * nchunks * (S::kLaneCodes / 8) * 64 * 16 +
+      static_cast<size_t>(M) * nchunks * 64 * 4;
   const size_t red_bytes = static_cast<size_t>(rw) * kw * kRowsPerWave * M * 4;
   return x_bytes > red_bytes ? x_bytes : red_bytes;
 }
@@ -440,16 +474,45 @@ size_t stream_smem_bytes(int M, int K, int rw, int kw) {
 struct StreamPlan {
   int kw;
   int rw;
+  int rm; // multiple of the shape's rows per wave
 };
 
 template <int BITS, int GS>
-StreamPlan stream_plan(int K) {
+StreamPlan stream_plan(int K, int N, int M) {
   using S = StreamShape<BITS, GS>;
   const int nchunks = (K + S::kChunkCodes - 1) / S::kChunkCodes;
   const int need = (nchunks + S::kChunksPerWave - 1) / S::kChunksPerWave;
   StreamPlan pl;
   pl.kw = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 0)));
   pl.rw = pl.kw == 0 ? 0 : 8 / pl.kw;
+  pl.rm = 1;
+  // Long K (four or eight k-waves): every workgroup stages the whole of x for
+  // the few rows it owns, so give a wave four rows while the grid still covers
+  // the compute units 1.5 times (4096 x 14336 8-bit: 17.8 -> 15.9 us, 4096 x 11008
+  // 4-bit: 10.7 -> 9.9 us).
+  if (pl.kw >= 4) {
+    const long want = compute_units() * 3L / 2;
+    int rm = 4 / S::kRowsPerWave;
+    while (rm > 1 && (N + pl.rw * S::kRowsPerWave * rm - 1) / (pl.rw * S::kRowsPerWave * rm) < want) {
+      rm /= 2;
+    }
+    pl.rm = rm;
+  }
+  // One k-wave, one row of x, 4-bit: workgroups of four waves when that lowers
+  // the number of rows the busiest compute unit ends up with (14336 rows on 256
+  // units: 7 x 8 rows instead of 4 x 16); measured 3-6 % faster when it does
+  // and slower when it does not, and slower for 8-bit codes either way.
+  if (pl.kw == 1 && M == 1 && BITS == 4) {
+    const long cus = compute_units();
+    auto busiest = [&](int rw) {
+      const long rows = static_cast<long>(rw) * S::kRowsPerWave * pl.rm;
+      const long wgs = (N + rows - 1) / rows;
+      return (wgs + cus - 1) / cus * rows;
+    };
+    if (busiest(4) < busiest(8)) {
+      pl.rw = 4;
+    }
+  }
   return pl;
 }
 
@@ -466,13 +529,13 @@ bool qmv_stream_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   if ((a.K / gs) % 2 != 0 || a.sb_batch_stride % 2 != 0) {
     return false;
   }
-  StreamPlan pl{0, 0};
+  StreamPlan pl{0, 0, 1};
   size_t smem = 0;
   auto probe = [&](auto bval, auto gval) {
     constexpr int B = decltype(bval)::value;
     constexpr int G = decltype(gval)::value;
-    pl = stream_plan<B, G>(a.K);
-    smem = pl.kw == 0 ? 0 : stream_smem_bytes<B, G>(a.M, a.K, pl.rw, pl.kw);
+    pl = stream_plan<B, G>(a.K, a.N, a.M);
+    smem = pl.kw == 0 ? 0 : stream_smem_bytes<B, G>(a.M, a.K, pl.rw, pl.kw, pl.rm);
   };
   auto by_group = [&](auto bval) {
     if (gs == 32) {
@@ -491,7 +554,7 @@ bool qmv_stream_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   if (pl.kw == 0) {
     return false; // K beyond 8 k-waves
   }
-  return smem <= 64 * 1024;
+  return smem <= 72 * 1024; // x image of 64 KiB (M = 2, K = 16384, 4-bit) + its sums
 }
 
 int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
@@ -500,20 +563,21 @@ int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t
     constexpr int B = decltype(bval)::value;
     constexpr int G = decltype(gval)::value;
     using S = StreamShape<B, G>;
-    const StreamPlan pl = stream_plan<B, G>(a.K);
-    const size_t smem = stream_smem_bytes<B, G>(a.M, a.K, pl.rw, pl.kw);
-    const int rows_per_wg = pl.rw * S::kRowsPerWave;
+    const StreamPlan pl = stream_plan<B, G>(a.K, a.N, a.M);
+    const size_t smem = stream_smem_bytes<B, G>(a.M, a.K, pl.rw, pl.kw, pl.rm);
+    const int rows_per_wg = pl.rw * S::kRowsPerWave * pl.rm;
     const bool full = a.K == pl.kw * S::kChunksPerWave * S::kChunkCodes;
     const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.L);
     if (grid.y > 65535u) {
       return fail(MLXROCM_UNSUPPORTED, "[qmv] batch=%d exceeds the grid", a.L);
     }
-    auto go = [&](auto mval, auto rwv, auto kwv) -> int {
+    auto go = [&](auto mval, auto rwv, auto kwv, auto rmv) -> int {
       constexpr int M = decltype(mval)::value;
       constexpr int RW = decltype(rwv)::value;
       constexpr int KW = decltype(kwv)::value;
-      auto kern = full ? qmv_stream_kernel<T, B, G, M, RW, KW, true>
-                       : qmv_stream_kernel<T, B, G, M, RW, KW, false>;
+      constexpr int RM = decltype(rmv)::value;
+      auto kern = full ? qmv_stream_kernel<T, B, G, M, RW, KW, true, RM>
+                       : qmv_stream_kernel<T, B, G, M, RW, KW, false, RM>;
       if (smem > 48 * 1024) {
         MLXROCM_HIP_TRY(hipFuncSetAttribute(
             reinterpret_cast<const void*>(kern),
@@ -524,16 +588,30 @@ int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t
       MLXROCM_HIP_TRY(hipGetLastError());
       return static_cast<int>(MLXROCM_OK);
     };
+    auto by_rm = [&](auto mval, auto rwv, auto kwv) -> int {
+      if constexpr (decltype(kwv)::value >= 4) {
+        if (pl.rm == 2) {
+          return go(mval, rwv, kwv, IntC<2>{});
+        }
+        if (pl.rm == 4) {
+          return go(mval, rwv, kwv, IntC<4>{});
+        }
+      }
+      return go(mval, rwv, kwv, IntC<1>{});
+    };
     auto by_plan = [&](auto mval) -> int {
       switch (pl.kw) {
         case 1:
-          return go(mval, IntC<8>{}, IntC<1>{});
+          if (pl.rw == 4) {
+            return by_rm(mval, IntC<4>{}, IntC<1>{});
+          }
+          return by_rm(mval, IntC<8>{}, IntC<1>{});
         case 2:
-          return go(mval, IntC<4>{}, IntC<2>{});
+          return by_rm(mval, IntC<4>{}, IntC<2>{});
         case 4:
-          return go(mval, IntC<2>{}, IntC<4>{});
+          return by_rm(mval, IntC<2>{}, IntC<4>{});
         default:
-          return go(mval, IntC<1>{}, IntC<8>{});
+          return by_rm(mval, IntC<1>{}, IntC<8>{});
       }
     };
     return a.M == 1 ? by_plan(IntC<1>{}) : by_plan(IntC<2>{});
