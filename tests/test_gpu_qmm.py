@@ -237,6 +237,24 @@ def test_qmv_matrix_instruction_gemv(oracle, gpu, dtype, gs):
         _check_qmm(oracle, gpu, x, w, gs, 4)
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+def test_qmv_launch_plans(oracle, gpu, dtype):
+    """Shapes that select each launch plan of the decode kernels: workgroups of
+    four and of eight waves with the dot products on the matrix instruction
+    (one row of x, 4-bit, groups of 64 / 128), four rows per wave for a long K
+    that is not a whole number of chunks (11008, one and two rows of x; 8-bit at
+    14336), and two row quads per wave on the 4x4x4 GEMV (8192 rows)."""
+    cases = (
+        (1, 6144, 4096, 4, 64), (1, 8192, 4096, 4, 128), (1, 4104, 2048, 4, 64),
+        (1, 4096, 11008, 4, 64), (2, 4096, 11008, 4, 64), (1, 4096, 14336, 8, 128),
+        (2, 4096, 8192, 8, 64), (3, 8192, 4096, 4, 64), (2, 8200, 4096, 4, 32),
+    )
+    for M, N, K, bits, gs in cases:
+        w = normal_weights((N, K), dtype, seed=M + N + K)
+        x = activations((M, K), dtype, seed=N + bits)
+        _check_qmm(oracle, gpu, x, w, gs, bits)
+
+
 def test_qmv_matrix_instruction_gemv_batched(oracle, gpu):
     # a batch of problems, each with its own weights: blockIdx.y walks the batch
     dtype, gs, L, M, N, K = torch.bfloat16, 64, 3, 3, 48, 1024
