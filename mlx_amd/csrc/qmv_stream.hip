@@ -206,13 +206,17 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
   // ---- 1. x: one coalesced read per workgroup (issued first) ----
   const int x_units = M * (K / 8); // 16-byte units
   const uint8_t* xbytes = reinterpret_cast<const uint8_t*>(p.x);
-  uint4 xv0 = make_uint4(0, 0, 0, 0);
-  uint4 xv1 = make_uint4(0, 0, 0, 0);
-  if (tid < x_units) {
-    xv0 = *reinterpret_cast<const uint4*>(xbytes + static_cast<uint32_t>(tid) * 16);
-  }
-  if (tid + kThreads < x_units) {
-    xv1 = *reinterpret_cast<const uint4*>(xbytes + static_cast<uint32_t>(tid + kThreads) * 16);
+  // up to kUpfront units per thread are fetched ahead of the weight stream (a
+  // long K split over four or eight k-waves needs up to four per row of x)
+  constexpr int kUpfront = KW >= 4 ? 4 : 2;
+  uint4 xv[kUpfront];
+#pragma unroll
+  for (int u = 0; u < kUpfront; ++u) {
+    xv[u] = make_uint4(0, 0, 0, 0);
+    if (tid + u * kThreads < x_units) {
+      xv[u] = *reinterpret_cast<const uint4*>(
+          xbytes + static_cast<uint32_t>(tid + u * kThreads) * 16);
+    }
   }
 
   // ---- 2. every weight / scale / bias load of this wave ----
@@ -316,15 +320,14 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
       sx_lds[(m * nchunks + c) * 64 + l] = part;
     }
   };
-  if (tid < x_units) {
-    stage_x(tid, xv0);
+#pragma unroll
+  for (int u = 0; u < kUpfront; ++u) {
+    if (tid + u * kThreads < x_units) {
+      stage_x(tid + u * kThreads, xv[u]);
+    }
   }
-  if (tid + kThreads < x_units) {
-    stage_x(tid + kThreads, xv1);
-  }
-  // longer x (more than 16 bytes x 2 per thread): the remaining units follow
-  // the weight loads in the queue
-  for (int idx = tid + 2 * kThreads; idx < x_units; idx += kThreads) {
+  // longer x: the remaining units follow the weight loads in the queue
+  for (int idx = tid + kUpfront * kThreads; idx < x_units; idx += kThreads) {
     stage_x(idx, *reinterpret_cast<const uint4*>(xbytes + static_cast<uint32_t>(idx) * 16));
   }
   __syncthreads();
