@@ -311,6 +311,27 @@ int run_qmm_t_transposed_sb(const QmmArgs& a, int gs, int bits, int dtype, int k
 // first transposed to [group][k] in the stream's scratch buffer (a few MB, a
 // few microseconds); few-row shapes also cut K and keep their fp32 partial
 // planes there.
+// transpose=false, 1..4 rows of x: the streaming kernel, its K ranges added up
+// from fp32 planes in the stream's scratch buffer.
+int run_qmv_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  const QmvNPlan pl = qmv_n_plan(a, bits);
+  if (pl.splits <= 1) {
+    return launch_qmv_n(a, gs, bits, dtype, nullptr, s);
+  }
+  const size_t plane = static_cast<size_t>(a.L) * a.M * a.N;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  void* scratch = nullptr;
+  int rc = stream_scratch(s, plane * pl.splits * sizeof(float), &scratch);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  rc = launch_qmv_n(a, gs, bits, dtype, static_cast<float*>(scratch), s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  return reduce_planes(static_cast<const float*>(scratch), a.out, plane, pl.splits, dtype, s);
+}
+
 int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
   const int G = a.N / gs;
   const int batches = a.sb_batch_stride == 0 ? 1 : a.L;
@@ -350,6 +371,11 @@ int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
 }
 
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
+  // w [K, N] with a few rows of x: the streaming kernel (the tile kernel
+  // needs 60-70 us for one row of a 4096 x 14336 weight)
+  if (!transpose && qmv_n_supported(a, gs, bits, dtype)) {
+    return run_qmv_n(a, gs, bits, dtype, s);
+  }
   // A few rows of x, beyond what the row-streaming GEMV keeps in registers.
   // Measured on gate/up and down projection shapes (4- and 8-bit):
   //   3..8 rows   the 32-row MFMA GEMV up to K = 8192, the wide kernel (K split

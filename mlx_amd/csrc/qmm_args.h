@@ -132,6 +132,19 @@ int transpose_sb_for_qmm_n(
     int64_t src_stride,
     int dtype,
     hipStream_t s);
+// transpose=false with 1..4 rows of x, 4/8-bit, every element type: a streaming
+// kernel over the packed rows of W.  K is cut into `splits` ranges of `range`
+// rows; with more than one range `partial` receives `splits` fp32 planes of
+// [L, M, N] for reduce_planes.
+struct QmvNPlan {
+  int range;
+  int splits;
+};
+bool qmv_n_supported(const QmmArgs& a, int gs, int bits, int dtype);
+QmvNPlan qmv_n_plan(const QmmArgs& a, int bits);
+int launch_qmv_n(const QmmArgs& a, int gs, int bits, int dtype, float* partial, hipStream_t s);
+// y (n elements, n % 4 == 0) = sum of `splits` fp32 planes; built for many planes.
+int reduce_planes(const float* partial, void* out, size_t n, int splits, int dtype, hipStream_t s);
 // decode GEMV in fp32 arithmetic (transpose=true): every width and element type,
 // one row of x, K <= 16384.
 bool qmv_f32_supported(const QmmArgs& a, int gs, int bits, int dtype);

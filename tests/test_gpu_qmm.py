@@ -199,6 +199,36 @@ def test_qmm_n_on_the_matrix_path(oracle, gpu, dtype, bits, gs):
         _check_qmm(oracle, gpu, x, w, gs, bits, transpose=False)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits,gs", ((4, 32), (4, 64), (4, 128), (8, 32), (8, 64), (8, 128)))
+def test_qvm_streaming_kernel(oracle, gpu, dtype, bits, gs):
+    """transpose=False with 1..4 rows of x (cpu/quantized.cpp:96-152, the "qvm"
+    case) runs on the row-streaming kernel: one K range and many, a K that is
+    not a multiple of the four wavefronts or of the eight rows in flight, an N
+    that leaves lanes (and whole wavefronts of the last column block) idle."""
+    for M, K, N in ((1, 40, 128), (2, 260, 1152), (3, 1024, 640), (4, 4096, 2048), (1, 2056, 4096)):
+        w = normal_weights((K, N), dtype, seed=bits + gs + M)
+        x = activations((M, K), dtype, seed=K)
+        _check_qmm(oracle, gpu, x, w, gs, bits, transpose=False)
+
+
+def test_qvm_streaming_kernel_batched(oracle, gpu):
+    dtype, gs, bits, L, M, K, N = torch.bfloat16, 64, 4, 3, 2, 1536, 256
+    ws = [normal_weights((K, N), dtype, seed=20 + l) for l in range(L)]
+    qs = [oracle.quantize(w, gs, bits) for w in ws]
+    wq = torch.stack([q[0] for q in qs]).to(gpu)
+    s = torch.stack([q[1] for q in qs]).to(gpu)
+    b = torch.stack([q[2] for q in qs]).to(gpu)
+    x = activations((L, M, K), dtype, seed=5)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq, s, b, False, gs, bits).cpu()
+    for l in range(L):
+        ref = oracle.qmm(x[l], *qs[l], False, gs, bits)
+        w_hat = exact_affine_weights(*qs[l], gs, bits)
+        exact = x[l].double() @ w_hat
+        tol = matmul_tolerance(dtype, K, x[l], w_hat) + float((ref.double() - exact).abs().max())
+        assert float((got[l].double() - ref.double()).abs().max()) <= tol
+
+
 def test_qmm_n_batched_and_full_size(oracle, gpu):
     # a batch of problems with one shared weight matrix, and the benchmark's
     # gate/up shape read the other way round, checked on sampled rows
