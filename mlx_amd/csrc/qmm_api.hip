@@ -102,7 +102,10 @@ int check_alignment(const char* who, const QmmArgs& a, int dtype) {
         who);
   }
   const int64_t x_vec = 16 / static_cast<int64_t>(dtype_size(dtype));
-  if (a.x_batch_stride % x_vec != 0 || a.w_batch_stride % 4 != 0) {
+  // one problem without indices never applies a batch stride (transpose=false
+  // allows any K, so M * K need not be a multiple of 16 bytes there)
+  const bool strided = a.L > 1 || a.lhs_indices != nullptr;
+  if (strided && (a.x_batch_stride % x_vec != 0 || a.w_batch_stride % 4 != 0)) {
     return fail(
         MLXROCM_UNSUPPORTED,
         "[%s] batch strides must keep 16-byte alignment (x stride %lld, w "

@@ -206,10 +206,20 @@ def test_qvm_streaming_kernel(oracle, gpu, dtype, bits, gs):
     case) runs on the row-streaming kernel: one K range and many, a K that is
     not a multiple of the four wavefronts or of the eight rows in flight, an N
     that leaves lanes (and whole wavefronts of the last column block) idle."""
-    for M, K, N in ((1, 40, 128), (2, 260, 1152), (3, 1024, 640), (4, 4096, 2048), (1, 2056, 4096)):
+    for M, K, N in ((1, 40, 128), (2, 257, 1152), (3, 1024, 640), (4, 4096, 2048), (1, 2050, 4096)):
         w = normal_weights((K, N), dtype, seed=bits + gs + M)
         x = activations((M, K), dtype, seed=K)
         _check_qmm(oracle, gpu, x, w, gs, bits, transpose=False)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_transpose_false_odd_k(oracle, gpu, dtype):
+    # K need not be a multiple of anything when w is [K, N]: rows of x then start
+    # at unaligned addresses (7 rows: the generic kernel; 3 rows: the streaming one)
+    for M, K, N in ((7, 257, 128), (3, 101, 96)):
+        w = normal_weights((K, N), dtype, seed=K)
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, w, 32, 4, transpose=False)
 
 
 def test_qvm_streaming_kernel_batched(oracle, gpu):
