@@ -391,14 +391,25 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   // 4-bit decode with a few rows of x: the 4x4x4 matrix-instruction GEMV.
   // Measured against the kernels below on gate/up, down-projection and group-32
   // shapes: it wins for 2..4 rows everywhere; for one row only where the
-  // row-streaming GEMV splits a long K over all eight wavefronts (K > 8192);
-  // for 5..8 rows (two operand sets, half the occupancy) only there and with
-  // 32-wide groups.
+  // row-streaming GEMV splits a long K over all eight wavefronts (K > 8192).
+  // With 5..8 rows (two operand sets, one workgroup per compute unit at a time)
+  // it wins by 10-60 % from K = 8192 on, with 32-wide groups, and wherever its
+  // workgroups fill their last round of compute units (4096, 11008, 12288 or
+  // 28672 rows at K = 4096); at 6144 or 14336 rows the last round is half
+  // empty and the 32-row MFMA GEMV is 4-12 % ahead.
   if (transpose && a.M <= 8 && qmv_quad_supported(a, gs, bits, dtype)) {
     const bool long_k = a.K > 8192;
+    bool many_rows = false;
+    if (a.M >= 5) {
+      const long cus = compute_units();
+      const long wgs = qmv_quad_workgroups_two_sets(a, bits);
+      const long rounds = (wgs + cus - 1) / cus;
+      // a single round, or more than 7/8 of the slots of all rounds in use
+      many_rows = long_k || a.K >= 8192 || gs == 32 ||
+          (wgs > 0 && (rounds <= 1 || wgs * 8 > rounds * cus * 7));
+    }
     const bool use = (a.M >= 2 && a.M <= 4) ||
-        (a.M == 1 && (long_k || !qmv_stream_supported(a, gs, bits, dtype))) ||
-        (a.M >= 5 && (long_k || gs == 32));
+        (a.M == 1 && (long_k || !qmv_stream_supported(a, gs, bits, dtype))) || many_rows;
     if (use) {
       return launch_qmv_quad(a, gs, bits, dtype, s);
     }

@@ -153,6 +153,7 @@ int launch_qmv_f32(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s)
 // 4-bit, K a multiple of 512 codes and at most 16384, an even number of groups.
 bool qmv_quad_supported(const QmmArgs& a, int gs, int bits, int dtype);
 int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+long qmv_quad_workgroups_two_sets(const QmmArgs& a, int bits);
 int launch_qmm_mfma_ksplit(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
 int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int dtype, hipStream_t s);
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);

@@ -459,6 +459,17 @@ bool qmv_quad_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   return quad_plan(a.K, bits).kw != 0;
 }
 
+// Workgroups of a launch with 5..8 rows of x (two operand sets: one workgroup
+// per compute unit at a time, so the launch runs in rounds of that many).
+long qmv_quad_workgroups_two_sets(const QmmArgs& a, int bits) {
+  const QuadPlan pl = quad_plan(a.K, bits, 8);
+  if (pl.kw == 0) {
+    return 0;
+  }
+  const int rows_per_wg = (8 / pl.kw) * 4 * 4;
+  return static_cast<long>((a.N + rows_per_wg - 1) / rows_per_wg) * a.L;
+}
+
 int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
   const QuadPlan pl = quad_plan(a.K, bits, a.M);
   if (pl.kw == 0) {

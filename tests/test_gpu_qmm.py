@@ -288,6 +288,9 @@ def test_qmv_launch_plans(oracle, gpu, dtype):
         (1, 6144, 4096, 4, 64), (1, 8192, 4096, 4, 128), (1, 4104, 2048, 4, 64),
         (1, 4096, 11008, 4, 64), (2, 4096, 11008, 4, 64), (1, 4096, 14336, 8, 128),
         (2, 4096, 8192, 8, 64), (3, 8192, 4096, 4, 64), (2, 8200, 4096, 4, 32),
+        # 5..8 rows: the 4x4x4 GEMV with two operand sets (K = 8192; a single
+        # round of workgroups) and the 32-row MFMA GEMV (a half-empty last round)
+        (6, 4096, 8192, 4, 64), (8, 1024, 4096, 4, 128), (5, 6144, 4096, 4, 64),
     )
     for M, N, K, bits, gs in cases:
         w = normal_weights((N, K), dtype, seed=M + N + K)
