@@ -146,7 +146,7 @@ int launch_qmv_n(const QmmArgs& a, int gs, int bits, int dtype, float* partial, 
 // y (n elements, n % 4 == 0) = sum of `splits` fp32 planes; built for many planes.
 int reduce_planes(const float* partial, void* out, size_t n, int splits, int dtype, hipStream_t s);
 // decode GEMV in fp32 arithmetic (transpose=true): every width and element type,
-// one row of x, K <= 16384.
+// one row of x at K <= 16384, two to four rows at K <= 8192.
 bool qmv_f32_supported(const QmmArgs& a, int gs, int bits, int dtype);
 int launch_qmv_f32(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 // 1..8 rows of x on the 4x4x4 matrix instruction: transpose=true, 16-bit types,

@@ -1,6 +1,6 @@
 // qmv_f32.hip -- decode GEMV (transpose=true) in plain fp32 arithmetic, every
-// code width and element type, one row of x: the streaming kernel for float32
-// operands and for the 16-bit types at widths 2/3/5/6.
+// code width and element type, one to four rows of x: the streaming kernel for
+// float32 operands and for the 16-bit types at widths 2/3/5/6.
 //
 // A lane owns 32 consecutive codes of a row (= `bits` whole dwords for every
 // width, and never more than one quantization group), so a wavefront covers a
@@ -202,22 +202,35 @@ F32Plan f32_plan(int K) {
 
 } // namespace
 
+// Rows of x in one launch: one for every K up to 16384; two to four while a
+// lane keeps a single 32-code slice of each row of x (K <= 8192).
 bool qmv_f32_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   (void)gs;
   (void)bits;
-  // one row of x: a second one doubles the registers that hold x (the kernel is
-  // written for it, the dispatch is not)
   (void)dtype;
-  if (a.M != 1) {
+  if (a.M < 1 || a.M > 4) {
     return false;
   }
-  return f32_plan(a.K).kw != 0; // K <= 16384
+  const F32Plan pl = f32_plan(a.K);
+  if (pl.kw == 0) {
+    return false; // K > 16384
+  }
+  return a.M == 1 || (a.K + kF32ChunkCodes - 1) / kF32ChunkCodes <= 4;
 }
 
 int launch_qmv_f32(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
-  const F32Plan pl = f32_plan(a.K);
-  if (pl.kw == 0) {
-    return fail(MLXROCM_UNSUPPORTED, "[qmv] K=%d is not covered by the fp32 GEMV", a.K);
+  F32Plan pl = f32_plan(a.K);
+  if (pl.kw == 0 || a.M < 1 || a.M > 4) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmv] M=%d K=%d is not covered by the fp32 GEMV", a.M, a.K);
+  }
+  if (a.M > 1) {
+    // one chunk per wave: the registers go to the rows of x
+    const int need = (a.K + kF32ChunkCodes - 1) / kF32ChunkCodes;
+    if (need > 4) {
+      return fail(MLXROCM_UNSUPPORTED, "[qmv] K=%d is not covered by the fp32 GEMV at M=%d", a.K, a.M);
+    }
+    pl.cpw = 1;
+    pl.kw = need <= 1 ? 1 : (need <= 2 ? 2 : 4);
   }
   const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
   const int rows_per_wg = (kF32Threads / 64 / pl.kw) * kF32RowsInFlight;
@@ -236,19 +249,36 @@ int launch_qmv_f32(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s)
     return static_cast<int>(MLXROCM_OK);
   };
   auto by_plan = [&](auto tval, auto bval, auto mval) -> int {
-    if (pl.kw == 1 && pl.cpw == 1) {
-      return go(tval, bval, mval, IntC<1>{}, IntC<1>{});
+    if (pl.cpw == 1) {
+      if (pl.kw == 1) {
+        return go(tval, bval, mval, IntC<1>{}, IntC<1>{});
+      }
+      if (pl.kw == 2) {
+        return go(tval, bval, mval, IntC<1>{}, IntC<2>{});
+      }
+      return go(tval, bval, mval, IntC<1>{}, IntC<4>{});
     }
-    if (pl.kw == 1) {
-      return go(tval, bval, mval, IntC<2>{}, IntC<1>{});
+    if constexpr (decltype(mval)::value == 1) {
+      if (pl.kw == 1) {
+        return go(tval, bval, mval, IntC<2>{}, IntC<1>{});
+      }
+      if (pl.kw == 2) {
+        return go(tval, bval, mval, IntC<2>{}, IntC<2>{});
+      }
+      return go(tval, bval, mval, IntC<2>{}, IntC<4>{});
     }
-    if (pl.kw == 2) {
-      return go(tval, bval, mval, IntC<2>{}, IntC<2>{});
-    }
-    return go(tval, bval, mval, IntC<2>{}, IntC<4>{});
+    return fail(MLXROCM_UNSUPPORTED, "[qmv] no fp32 GEMV plan for M=%d K=%d", a.M, a.K);
   };
   return dispatch_dtype(dtype, [&](auto tval) {
-    return dispatch_bits(bits, [&](auto bval) { return by_plan(tval, bval, IntC<1>{}); });
+    return dispatch_bits(bits, [&](auto bval) {
+      if (a.M == 1) {
+        return by_plan(tval, bval, IntC<1>{});
+      }
+      if (a.M == 2) {
+        return by_plan(tval, bval, IntC<2>{});
+      }
+      return by_plan(tval, bval, IntC<4>{});
+    });
   });
 }
 

@@ -324,3 +324,30 @@ def test_qmv_float32_streaming(oracle, gpu, bits):
         w = normal_weights((N, K), torch.float32, seed=bits + gs)
         x = activations((1, K), torch.float32, seed=K)
         _check_qmm(oracle, gpu, x, w, gs, bits)
+
+
+@pytest.mark.parametrize("bits", ALL_BITS)
+def test_qmv_float32_few_rows(oracle, gpu, bits):
+    """2..4 rows of float32 x in one launch of the fp32 streaming GEMV (K up to
+    8192), and the shapes beyond it (5..16 rows, K > 8192 with two rows, a batch
+    of problems with five rows) on the generic kernels and the matrix path."""
+    cases = ((64, 2, 100, 512), (32, 3, 70, 4096), (128, 4, 33, 8192), (64, 7, 64, 2048),
+             (64, 16, 48, 4096), (32, 13, 40, 6144), (64, 2, 24, 10240))
+    for gs, M, N, K in cases:
+        w = normal_weights((N, K), torch.float32, seed=bits + gs + M)
+        x = activations((M, K), torch.float32, seed=K + M)
+        _check_qmm(oracle, gpu, x, w, gs, bits)
+    # batched, five rows
+    L, M, N, K, gs = 2, 5, 40, 1024, 64
+    ws = [normal_weights((N, K), torch.float32, seed=30 + l) for l in range(L)]
+    qs = [oracle.quantize(w, gs, bits) for w in ws]
+    wq = torch.stack([q[0] for q in qs]).to(gpu)
+    s = torch.stack([q[1] for q in qs]).to(gpu)
+    b = torch.stack([q[2] for q in qs]).to(gpu)
+    x = activations((L, M, K), torch.float32, seed=6)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq, s, b, True, gs, bits).cpu()
+    for l in range(L):
+        ref = oracle.qmm(x[l], *qs[l], True, gs, bits)
+        w_hat = exact_affine_weights(*qs[l], gs, bits)
+        tol = matmul_tolerance(torch.float32, K, x[l], w_hat)
+        assert float((got[l].double() - ref.double()).abs().max()) <= tol
