@@ -418,7 +418,32 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   // are issue-bound there, 28 us against 20 us for the wide kernel at K = 14336)
   const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype) ||
       (a.M == 2 && bits == 8 && a.K > 8192);
-  const bool staged = a.M > 16 || (a.M > 8 && a.N >= 8192);
+  // 17..32 rows over a narrow N (fewer 64-row workgroups than half the compute
+  // units): the wide kernel twice, 16 rows each; the second pass finds the
+  // weights in the Infinity Cache (4096 x 4096: 24 -> 16 us, 4096 x 14336: 56 -> 45 us)
+  if (transpose && a.M > 16 && a.M <= 32 && a.L == 1 && a.lhs_indices == nullptr &&
+      a.group_tiles == nullptr && (a.N + 63) / 64 < compute_units() / 2) {
+    QmmArgs part = a;
+    part.M = 16;
+    if (qmv_wide_supported(part, gs, bits, dtype, transpose)) {
+      int rc = launch_qmv_wide(part, gs, bits, dtype, s);
+      if (rc != MLXROCM_OK) {
+        return rc;
+      }
+      const size_t esize = dtype_size(dtype);
+      part.M = a.M - 16;
+      part.x = static_cast<const char*>(a.x) + static_cast<size_t>(16) * a.K * esize;
+      part.out = static_cast<char*>(a.out) + static_cast<size_t>(16) * a.N * esize;
+      return launch_qmv_wide(part, gs, bits, dtype, s);
+    }
+  }
+  // (17..32 rows: the staged kernel walks K serially with N / 64 workgroups, so
+  // a narrow N with a long K goes to the tile kernel and its K split instead:
+  // 4096 x 14336, 32 rows: 78 us against 57 us)
+  const bool narrow_long = a.M > 16 && a.K > 8192 &&
+      static_cast<long>((a.N + 63) / 64) * a.L < compute_units() / 2 &&
+      a.lhs_indices == nullptr && a.group_tiles == nullptr;
+  const bool staged = (a.M > 16 || (a.M > 8 && a.N >= 8192)) && !narrow_long;
   // one row at a width the row-streaming GEMV does not cover (2/3/5/6 bits): the
   // fp32-arithmetic streaming kernel
   if (transpose && a.M == 1 && few_rows && qmv_f32_supported(a, gs, bits, dtype)) {

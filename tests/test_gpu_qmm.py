@@ -174,10 +174,12 @@ def test_qmm_t_fp32_runs_on_the_matrix_path(oracle, gpu):
 @pytest.mark.parametrize("bits", ALL_BITS)
 def test_qmm_few_rows_kernels(oracle, gpu, dtype, bits):
     """3 <= M <= 32 goes to the few-row kernels (K split over wavefronts up to 16
-    rows, 64-row LDS-staged tiles up to 32): ragged N, K of one and of several
-    steps, every group size."""
+    rows and, for a narrow N, twice for up to 32; 64-row LDS-staged tiles for
+    17..32 rows over a wide N): ragged N, K of one and of several steps, every
+    group size."""
     for gs in ALL_GROUPS:
-        for M, N, K in ((5, 67, 128), (12, 130, 1280), (16, 48, 8704), (17, 200, 256), (32, 67, 1792)):
+        for M, N, K in ((5, 67, 128), (12, 130, 1280), (16, 48, 8704), (17, 200, 256), (32, 67, 1792),
+                        (20, 8224, 384), (32, 8192, 128)):
             w = normal_weights((N, K), dtype, seed=bits + gs + M)
             x = activations((M, K), dtype, seed=M)
             _check_qmm(oracle, gpu, x, w, gs, bits)
