@@ -264,8 +264,15 @@ int reduce_planes(const float* partial, void* out, size_t n, int splits, int dty
 bool qmv_n_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   (void)gs;
   (void)dtype;
-  return a.M >= 1 && a.M <= 4 && (bits == 4 || bits == 8) && a.lhs_indices == nullptr &&
-      a.L <= 65535;
+  if (a.M < 1 || a.M > 4 || !(bits == 4 || bits == 8) || a.lhs_indices != nullptr ||
+      a.L > 65535) {
+    return false;
+  }
+  // the K ranges are a grid dimension, and their fp32 planes (K N M / 16 bytes)
+  // stay below 256 MiB of scratch
+  const long splits = (static_cast<long>(a.K) + kNRange - 1) / kNRange;
+  const long plane = static_cast<long>(a.L) * a.M * a.N;
+  return splits <= 65535 && splits * plane <= (64L << 20);
 }
 
 QmvNPlan qmv_n_plan(const QmmArgs& a, int bits) {
