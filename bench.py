@@ -231,6 +231,49 @@ def sweep(torch, mlx_amd, dev) -> list:
         for (bits, gs) in ((4, 64), (8, 128)):
             for M in (512, 2048, 8192):
                 matmul_case("cfg3", M, n, k, bits, gs, bf16)
+    # gated MLP decode (nn callers): silu(gate(x)) * up(x), fused entry point against
+    # two quantized_matmul launches and the elementwise arithmetic
+    def swiglu_case(M, n, k, bits, gs):
+        from mlx_amd import _lib
+        lib = _lib.load()
+        qg = mlx_amd.quantize(weights(n, k, bf16), gs, bits)
+        wbytes = n * k * bits // 8 + 2 * n * (k // gs) * 2
+        ring = ring_of(qg, wbytes)  # entries 2i, 2i+1: gate and up
+        x = torch.randn((M, k), generator=g, dtype=torch.float32).to(bf16).to(dev)
+        out = torch.empty((M, n), dtype=bf16, device=dev)
+        gate = torch.empty((M, n), dtype=bf16, device=dev)
+        up = torch.empty((M, n), dtype=bf16, device=dev)
+        ws = torch.empty(lib.mlxrocm_qmm_swiglu_workspace_size(M, n, 2), dtype=torch.uint8, device=dev)
+        R = len(ring) // 2
+
+        def fused(i, stream):
+            a, b = ring[2 * (i % R)], ring[2 * (i % R) + 1]
+            rc = lib.mlxrocm_qmm_swiglu(x.data_ptr(), a[0].data_ptr(), a[1].data_ptr(), a[2].data_ptr(),
+                                        b[0].data_ptr(), b[1].data_ptr(), b[2].data_ptr(),
+                                        out.data_ptr(), ws.data_ptr(), M, n, k, gs, bits, 2, stream)
+            if rc != 0:
+                raise RuntimeError(_lib.last_error())
+
+        def unfused(i, stream):
+            a, b = ring[2 * (i % R)], ring[2 * (i % R) + 1]
+            for q_, o_ in ((a, gate), (b, up)):
+                rc = lib.mlxrocm_qmm(x.data_ptr(), q_[0].data_ptr(), q_[1].data_ptr(), q_[2].data_ptr(),
+                                     o_.data_ptr(), M, n, k, 1, M * k, 0, 0, gs, bits, 2, 1, stream)
+                if rc != 0:
+                    raise RuntimeError(_lib.last_error())
+            torch.mul(torch.nn.functional.silu(gate), up, out=out)
+
+        nb = 2 * qmv_bytes(M, n, k, bits, gs, 2) - M * k * 2
+        for label, fn in (("fused entry point", fused), ("two launches + elementwise", unfused)):
+            launcher = Launcher(torch, fn, R, True)
+            launcher.run(R)
+            torch.cuda.synchronize()
+            ms = hip_event_ms(lib, launcher, R * 20)
+            add("f1", f"silu(gate(x))*up(x), x bfloat16 [{M},{k}] W 2x[{n},{k}] b{bits} g{gs}, {label}",
+                ms, nbytes=nb)
+
+    for B in (1, 4):
+        swiglu_case(B, 14336, 4096, 4, 64)
     # transpose=False (the vjp of a quantized linear layer): w [k, n] quantized along n
     for M in (1, 512, 2048):
         matmul_case("f3", M, 14336, 4096, 4, 64, bf16, transpose=False)

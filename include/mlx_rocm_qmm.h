@@ -167,6 +167,38 @@ int mlxrocm_qmm(
     mlxrocm_stream_t stream);
 
 /*
+ * Gated-MLP decode: out = silu(x @ dequant(w_gate).T) * (x @ dequant(w_up).T),
+ * both projections in one launch over the shared x, then one elementwise pass.
+ * No single primitive of the reference corresponds to it: it fuses the two
+ * QuantizedMatmul calls and the `nn.silu(gate(x)) * up(x)` arithmetic that
+ * callers of nn.QuantizedLinear (python/mlx/nn/layers/quantized.py:205-307)
+ * issue per MLP block; intermediate results are rounded to the element type
+ * where that chain rounds them.  x [M, K] (M <= 8), both weights [N, K*bits/32]
+ * with scales / biases [N, K/group_size], out [M, N].  `workspace` is device
+ * memory of mlxrocm_qmm_swiglu_workspace_size(M, N, dtype) bytes, 16-byte
+ * aligned, owned by the caller (the two projections before the gate is
+ * applied); the call allocates nothing.
+ */
+size_t mlxrocm_qmm_swiglu_workspace_size(int M, int N, int dtype);
+int mlxrocm_qmm_swiglu(
+    const void* x,
+    const uint32_t* wq_gate,
+    const void* scales_gate,
+    const void* biases_gate,
+    const uint32_t* wq_up,
+    const void* scales_up,
+    const void* biases_up,
+    void* out,
+    void* workspace,
+    int M,
+    int N,
+    int K,
+    int group_size,
+    int bits,
+    int dtype,
+    mlxrocm_stream_t stream);
+
+/*
  * Replaces GatherQMM::eval_gpu (mlx/primitives.h:1698; CPU body
  * mlx/backend/cpu/quantized.cpp:966-1047, loop :700-747):
  *

@@ -3,6 +3,6 @@
 with the reference's operator names and semantics, backed by hand-written HIP
 kernels through the C ABI declared in ``include/mlx_rocm_qmm.h``."""
 from . import nn
-from .ops import dequantize, gather_qmm, quantize, quantized_matmul
+from .ops import dequantize, gather_qmm, quantize, quantized_matmul, quantized_swiglu
 
-__all__ = ["quantize", "dequantize", "quantized_matmul", "gather_qmm", "nn"]
+__all__ = ["quantize", "dequantize", "quantized_matmul", "quantized_swiglu", "gather_qmm", "nn"]

@@ -524,6 +524,110 @@ extern "C" const char* mlxrocm_qmm_kernel_name(
   return family_name(choose_family(M, N, K, L, bits, dtype, transpose != 0));
 }
 
+namespace {
+
+// out[i] = silu(gate[i]) * up[i] with the roundings of the unfused chain
+// (sigmoid, gate * sigmoid and the product are each rounded to T, as
+// x * sigmoid(x) followed by a multiply is in the element type).
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* gate_up, T* out, size_t n) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) {
+    return;
+  }
+  const float g = to_f32(gate_up[i]);
+  const float u = to_f32(gate_up[n + i]);
+  const float sg = to_f32(from_f32<T>(1.0f / (1.0f + __expf(-g))));
+  const float h = to_f32(from_f32<T>(g * sg));
+  out[i] = from_f32<T>(h * u);
+}
+
+} // namespace
+
+extern "C" size_t mlxrocm_qmm_swiglu_workspace_size(int M, int N, int dtype) {
+  if (M <= 0 || N <= 0) {
+    return 0;
+  }
+  return static_cast<size_t>(2) * M * N * dtype_size(dtype);
+}
+
+extern "C" int mlxrocm_qmm_swiglu(
+    const void* x,
+    const uint32_t* wq_gate,
+    const void* scales_gate,
+    const void* biases_gate,
+    const uint32_t* wq_up,
+    const void* scales_up,
+    const void* biases_up,
+    void* out,
+    void* workspace,
+    int M,
+    int N,
+    int K,
+    int group_size,
+    int bits,
+    int dtype,
+    mlxrocm_stream_t stream) {
+  int rc = check_shape("quantized_swiglu", M, N, K, 1, group_size, bits, dtype, 1);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (M > 8) {
+    return fail(
+        MLXROCM_UNSUPPORTED,
+        "[quantized_swiglu] M=%d: the fused gate/up projection covers decode (M <= 8)",
+        M);
+  }
+  if (static_cast<int64_t>(M) * N == 0) {
+    return MLXROCM_OK;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (K == 0) {
+    return launch_zero_fill(out, static_cast<size_t>(M) * N * dtype_size(dtype), s);
+  }
+  if (!x || !wq_gate || !scales_gate || !biases_gate || !wq_up || !scales_up || !biases_up ||
+      !out || !workspace) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[quantized_swiglu] null device pointer");
+  }
+  if (!aligned16(wq_up) || !aligned16(scales_up) || !aligned16(biases_up) ||
+      !aligned16(workspace)) {
+    return fail(MLXROCM_UNSUPPORTED, "[quantized_swiglu] operand pointers must be 16-byte aligned");
+  }
+  QmmArgs a{};
+  a.x = x;
+  a.w = wq_gate;
+  a.scales = scales_gate;
+  a.biases = biases_gate;
+  a.w_alt = wq_up;
+  a.scales_alt = scales_up;
+  a.biases_alt = biases_up;
+  a.out = workspace; // [2, M, N]: gate, up
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.L = 2;
+  a.x_batches = 2;
+  a.n_experts = 2;
+  rc = check_alignment("quantized_swiglu", a, dtype);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  rc = run(a, group_size, bits, dtype, true, s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  const size_t n = static_cast<size_t>(M) * N;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  rc = dispatch_dtype(dtype, [&](auto tval) {
+    using T = decltype(tval);
+    swiglu_kernel<T><<<blocks, 256, 0, s>>>(
+        static_cast<const T*>(workspace), static_cast<T*>(out), n);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
+  });
+  return rc;
+}
+
 extern "C" int mlxrocm_qmm(
     const void* x,
     const uint32_t* wq,

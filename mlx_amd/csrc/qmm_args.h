@@ -39,6 +39,13 @@ struct QmmArgs {
   // swapped), so that the lanes of a wavefront, which own consecutive rows of
   // W, read consecutive values.  0: the caller's [N][K / group] arrays.
   int sb_transposed;
+  // Two weight matrices sharing one x (the gate and up projections of a gated
+  // MLP): with L == 2 and these set, problem 1 reads them instead of w / scales /
+  // biases advanced by a batch stride.  Null otherwise.  Honoured by the kernels
+  // that resolve their operands with resolve_problem (every decode kernel).
+  const uint32_t* w_alt;
+  const void* scales_alt;
+  const void* biases_alt;
 };
 
 // Resolved operand pointers of problem l.  `valid` is false when a gathered
@@ -73,6 +80,11 @@ __device__ __forceinline__ QmmProblem<T> resolve_problem(
   p.w = reinterpret_cast<const uint8_t*>(a.w + wb * a.w_batch_stride);
   p.scales = static_cast<const T*>(a.scales) + wb * a.sb_batch_stride;
   p.biases = static_cast<const T*>(a.biases) + wb * a.sb_batch_stride;
+  if (a.w_alt != nullptr && l == 1) {
+    p.w = reinterpret_cast<const uint8_t*>(a.w_alt);
+    p.scales = static_cast<const T*>(a.scales_alt);
+    p.biases = static_cast<const T*>(a.biases_alt);
+  }
   p.out = static_cast<T*>(a.out) +
       static_cast<int64_t>(l) * a.M * static_cast<int64_t>(a.N);
   return p;

@@ -264,6 +264,59 @@ def _dense_batches(t: torch.Tensor, batch_shape: Tuple[int, ...]):
     return t, t.shape[-1] * t.shape[-2]
 
 
+def quantized_swiglu(
+    x: torch.Tensor,
+    gate: tuple,
+    up: tuple,
+    group_size: Optional[int] = None,
+    bits: Optional[int] = None,
+):
+    """``silu(quantized_matmul(x, *gate)) * quantized_matmul(x, *up)`` for decode
+    (at most 8 rows of x), both projections in one launch.  ``gate`` and ``up``
+    are ``(weight, scales, biases)`` triplets of equal shape, as
+    ``nn.QuantizedLinear`` holds them (python/mlx/nn/layers/quantized.py:205-307);
+    the reference has no fused primitive for the gated MLP, so more rows of x, or
+    a device other than the GPU, raise instead of taking another route."""
+    wg, sg, bg = gate
+    wu, su, bu = up
+    dtype, mode = _validate_mode_with_type("quantized_swiglu", sg, bg, None, "affine")
+    group_size, bits = _params_from_mode(mode, group_size, bits)
+    _, n_gate = _extract_dims("quantized_swiglu", x, wg, sg, bg, True, group_size, bits)
+    _, n_up = _extract_dims("quantized_swiglu", x, wu, su, bu, True, group_size, bits)
+    if n_gate != n_up or wg.shape != wu.shape or wg.dim() != 2:
+        raise ValueError(
+            "[quantized_swiglu] gate and up must be 2-D weights of one shape; got "
+            f"{tuple(wg.shape)} and {tuple(wu.shape)}."
+        )
+    dtype = torch.promote_types(x.dtype, dtype)
+    if dtype not in _FLOATING:
+        raise ValueError(
+            f"[quantized_swiglu] Only real floating types are supported but x.dtype() == {x.dtype}."
+        )
+    _check_affine_params("quantized_swiglu", group_size, bits)
+    _require_gpu("quantized_swiglu", x, wg, sg, bg, wu, su, bu)
+    lib = _lib.load()
+    K = x.shape[-1]
+    M = 1
+    for d in x.shape[:-1]:
+        M *= d
+    xb = x.to(dtype).reshape(M, K).contiguous()
+    sg, bg, su, bu = (t.to(dtype).contiguous() for t in (sg, bg, su, bu))
+    wg, wu = wg.contiguous(), wu.contiguous()
+    code = _DTYPE_CODE[dtype]
+    ws_bytes = lib.mlxrocm_qmm_swiglu_workspace_size(M, n_gate, code)
+    workspace = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=x.device)
+    out = torch.empty(tuple(x.shape[:-1]) + (n_gate,), dtype=dtype, device=x.device)
+    _lib.check(
+        lib.mlxrocm_qmm_swiglu(
+            xb.data_ptr(), wg.data_ptr(), sg.data_ptr(), bg.data_ptr(),
+            wu.data_ptr(), su.data_ptr(), bu.data_ptr(), out.data_ptr(), workspace.data_ptr(),
+            M, n_gate, K, group_size, bits, code, _stream_ptr(x),
+        )
+    )
+    return out
+
+
 def quantized_matmul(
     x: torch.Tensor,
     w: torch.Tensor,

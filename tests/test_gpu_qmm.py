@@ -353,3 +353,49 @@ def test_qmv_float32_few_rows(oracle, gpu, bits):
         w_hat = exact_affine_weights(*qs[l], gs, bits)
         tol = matmul_tolerance(torch.float32, K, x[l], w_hat)
         assert float((got[l].double() - ref.double()).abs().max()) <= tol
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits,gs", ((4, 64), (8, 128), (3, 32)))
+def test_quantized_swiglu_matches_the_unfused_chain(oracle, gpu, dtype, bits, gs):
+    """silu(gate(x)) * up(x) in one call against the same chain built from the
+    oracle's two products, with every intermediate rounded to the element type as
+    `x * sigmoid(x)` and the multiply round it; 1..8 rows of x, ragged N."""
+    for M, N, K in ((1, 200, 512), (2, 96, 4096), (4, 64, 1024), (8, 130, 2048)):
+        wg = normal_weights((N, K), dtype, seed=bits + M)
+        wu = normal_weights((N, K), dtype, seed=bits + M + 100)
+        x = activations((M, K), dtype, seed=K + M)
+        qg = oracle.quantize(wg, gs, bits)
+        qu = oracle.quantize(wu, gs, bits)
+        got = mlx_amd.quantized_swiglu(
+            x.to(gpu), tuple(t.to(gpu) for t in qg), tuple(t.to(gpu) for t in qu), gs, bits
+        ).cpu()
+        assert got.shape == (M, N) and got.dtype == dtype
+        # the chain in fp64 from the exact products, and its unfused form on the GPU
+        eg = x.double() @ exact_affine_weights(*qg, gs, bits).T
+        eu = x.double() @ exact_affine_weights(*qu, gs, bits).T
+        exact = eg * torch.sigmoid(eg) * eu
+        g = mlx_amd.quantized_matmul(x.to(gpu), *(t.to(gpu) for t in qg), True, gs, bits)
+        u = mlx_amd.quantized_matmul(x.to(gpu), *(t.to(gpu) for t in qu), True, gs, bits)
+        unfused = ((g * torch.sigmoid(g)) * u).cpu()
+        eps = {torch.float32: 2.0 ** -22, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+        scale = float(unfused.double().abs().max()) + 1e-30
+        # same products, same roundings: a few units in the last place of T
+        assert float((got.double() - unfused.double()).abs().max()) <= 4 * eps * scale
+        # and within the matmul tolerance (propagated through the gate) of fp64
+        w_hat = exact_affine_weights(*qg, gs, bits)
+        tol = matmul_tolerance(dtype, K, x, w_hat)
+        bound = tol * (float(eu.abs().max()) + 1.1 * float(eg.abs().max()) + tol) + 8 * eps * scale
+        assert float((got.double() - exact).abs().max()) <= bound
+
+
+def test_quantized_swiglu_rejects_prefill_and_mismatched_weights(oracle, gpu):
+    w = normal_weights((64, 256), torch.bfloat16, seed=1)
+    q = tuple(t.to(gpu) for t in oracle.quantize(w, 64, 4))
+    x = activations((9, 256), torch.bfloat16).to(gpu)
+    with pytest.raises(RuntimeError, match="M <= 8"):
+        mlx_amd.quantized_swiglu(x, q, q, 64, 4)
+    w2 = normal_weights((32, 256), torch.bfloat16, seed=2)
+    q2 = tuple(t.to(gpu) for t in oracle.quantize(w2, 64, 4))
+    with pytest.raises(ValueError, match="one shape"):
+        mlx_amd.quantized_swiglu(x[:1], q, q2, 64, 4)
