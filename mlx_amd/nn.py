@@ -121,6 +121,37 @@ class QuantizedEmbedding(torch.nn.Module):
         return ql
 
 
+class SwiGLU(torch.nn.Module):
+    """Gated MLP block ``down(silu(gate(x)) * up(x))`` over three
+    :class:`QuantizedLinear` layers (the MLP of Llama-style models built from
+    ``nn.QuantizedLinear``, python/mlx/nn/layers/quantized.py:205-307).  With at
+    most 8 rows of x and no additive biases the gate and up projections and the
+    gate arithmetic run as one ``quantized_swiglu`` call; otherwise as the three
+    separate products."""
+
+    def __init__(self, input_dims: int, hidden_dims: int, bias: bool = False,
+                 group_size: Optional[int] = None, bits: Optional[int] = None,
+                 device=None, dtype=torch.float32):
+        super().__init__()
+        kw = dict(bias=bias, group_size=group_size, bits=bits, device=device, dtype=dtype)
+        self.gate_proj = QuantizedLinear(input_dims, hidden_dims, **kw)
+        self.up_proj = QuantizedLinear(input_dims, hidden_dims, **kw)
+        self.down_proj = QuantizedLinear(hidden_dims, input_dims, **kw)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        g, u = self.gate_proj, self.up_proj
+        rows = x.numel() // max(x.shape[-1], 1)
+        fused = (0 < rows <= 8 and g.bias is None and u.bias is None
+                 and (g.group_size, g.bits, g.mode) == (u.group_size, u.bits, "affine")
+                 and u.mode == "affine")
+        if fused:
+            h = ops.quantized_swiglu(x, (g.weight, g.scales, g.biases),
+                                     (u.weight, u.scales, u.biases), g.group_size, g.bits)
+        else:
+            h = torch.nn.functional.silu(g(x)) * u(x)
+        return self.down_proj(h)
+
+
 class QuantizedSwitchLinear(torch.nn.Module):
     """A stack of ``num_experts`` quantized linear layers evaluated through
     ``gather_qmm``: ``y[..., i, :, :] = x[..., :, :] @ dequant(weight[indices[..., i]]).T``

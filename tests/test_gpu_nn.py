@@ -156,3 +156,27 @@ def test_switch_linear_bias_and_sorted_flag():
     w1 = mlx_amd.dequantize(layer.weight[1], layer.scales[1], layer.biases[1], group_size=32, bits=8)
     want = x[2, 0].double() @ w1.double().T + layer.bias[1].double()
     assert float((a[2, 0].double() - want).abs().max()) <= 2e-2
+
+
+@pytest.mark.parametrize("rows", (1, 5, 16))
+def test_swiglu_block_matches_dense(rows):
+    # the gated MLP of dequantized weights; up to 8 rows take the fused gate/up
+    # call, 16 rows the three separate products, and both agree with each other
+    torch.manual_seed(rows)
+    D, H, dt = 256, 512, torch.bfloat16
+    mlp = qnn.SwiGLU(D, H, group_size=64, bits=4, dtype=dt)
+    x = torch.randn(rows, D, device="cuda", dtype=dt)
+    y = mlp(x)
+    assert tuple(y.shape) == (rows, D) and y.dtype == dt
+
+    def dense(layer):
+        return mlx_amd.dequantize(layer.weight, layer.scales, layer.biases,
+                                  group_size=64, bits=4).double()
+
+    gate = (x.double() @ dense(mlp.gate_proj).T).to(dt)
+    up = (x.double() @ dense(mlp.up_proj).T).to(dt)
+    h = (torch.nn.functional.silu(gate) * up).double()
+    want = h @ dense(mlp.down_proj).T
+    assert float((y.double() - want).abs().max()) <= 0.05
+    separate = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
+    assert float((y.double() - separate.double()).abs().max()) <= 0.02
