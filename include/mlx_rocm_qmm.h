@@ -177,7 +177,8 @@ int mlxrocm_qmm(
  * with scales / biases [N, K/group_size], out [M, N].  `workspace` is device
  * memory of mlxrocm_qmm_swiglu_workspace_size(M, N, dtype) bytes, 16-byte
  * aligned, owned by the caller (the two projections before the gate is
- * applied); the call allocates nothing.
+ * applied; shapes whose gate is applied inside the GEMV leave it untouched);
+ * the call allocates nothing.
  */
 size_t mlxrocm_qmm_swiglu_workspace_size(int M, int N, int dtype);
 int mlxrocm_qmm_swiglu(

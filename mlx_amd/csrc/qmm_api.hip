@@ -612,6 +612,16 @@ extern "C" int mlxrocm_qmm_swiglu(
   if (rc != MLXROCM_OK) {
     return rc;
   }
+  // one row of x on the row-streaming GEMV: the gate is applied in the kernel's
+  // epilogue and nothing passes through the workspace
+  {
+    QmmArgs one = a;
+    one.L = 1;
+    one.out = out;
+    if (qmv_stream_glu_supported(one, group_size, bits, dtype)) {
+      return launch_qmv_stream_glu(one, group_size, bits, dtype, s);
+    }
+  }
   rc = run(a, group_size, bits, dtype, true, s);
   if (rc != MLXROCM_OK) {
     return rc;

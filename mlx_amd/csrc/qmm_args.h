@@ -157,6 +157,9 @@ QmvNPlan qmv_n_plan(const QmmArgs& a, int bits);
 int launch_qmv_n(const QmmArgs& a, int gs, int bits, int dtype, float* partial, hipStream_t s);
 // y (n elements, n % 4 == 0) = sum of `splits` fp32 planes; built for many planes.
 int reduce_planes(const float* partial, void* out, size_t n, int splits, int dtype, hipStream_t s);
+// gated decode GEMV: y = silu(w . x) * (w_alt . x) in one launch (one row of x)
+bool qmv_stream_glu_supported(const QmmArgs& a, int gs, int bits, int dtype);
+int launch_qmv_stream_glu(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 // decode GEMV in fp32 arithmetic (transpose=true): every width and element type,
 // one row of x at K <= 16384, two to four rows at K <= 8192.
 bool qmv_f32_supported(const QmmArgs& a, int gs, int bits, int dtype);

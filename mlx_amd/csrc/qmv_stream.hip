@@ -178,7 +178,8 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 // KW: waves that split K between them; RW: row-waves; the workgroup owns
 // RW * kRowsPerWave rows.  M is 1 or 2.  FULL: K is exactly KW * CPW chunks, so
 // no lane ever falls outside a row and the loads carry no predicate.
-template <typename T, int BITS, int GS, int M, int RW, int KW, bool FULL, int RM = 1, bool MD = false>
+template <typename T, int BITS, int GS, int M, int RW, int KW, bool FULL, int RM = 1, bool MD = false,
+          bool GLU = false>
 __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs a) {
   using S = StreamShape<BITS, GS>;
   constexpr int CPW = S::kChunksPerWave;
@@ -201,7 +202,14 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
 
   const int groups = K / GS;
   const uint32_t row_bytes = static_cast<uint32_t>(K / 8) * BITS;
-  const int row0 = (blockIdx.x * RW + rw) * kRowsPerWave;
+  // GLU: the wave's two rows are row n of the gate weight (a.w) and row n of the
+  // up weight (a.w_alt); it writes y[n] = silu(gate . x) * (up . x).
+  static_assert(!GLU || (KW == 1 && kRowsPerWave == 2 && M == 1), "gated form: one k-wave, a row pair");
+  const int row0 = GLU ? (blockIdx.x * RW + rw) : (blockIdx.x * RW + rw) * kRowsPerWave;
+  auto row_of = [&](int r) {
+    const int row = GLU ? row0 : row0 + r;
+    return row < N ? row : N - 1; // clamp: stay in bounds
+  };
 
   // ---- 1. x: one coalesced read per workgroup (issued first) ----
   const int x_units = M * (K / 8); // 16-byte units
@@ -237,18 +245,26 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
   const uint8_t* sb_lane_base =
       reinterpret_cast<const uint8_t*>(lane < 32 ? p.scales : p.biases) +
       static_cast<size_t>(sb_group) * 2;
+  const uint8_t* sb_lane_alt = sb_lane_base;
+  const uint8_t* w_alt = p.w;
+  if constexpr (GLU) {
+    sb_lane_alt =
+        reinterpret_cast<const uint8_t*>(lane < 32 ? a.scales_alt : a.biases_alt) +
+        static_cast<size_t>(sb_group) * 2;
+    w_alt = reinterpret_cast<const uint8_t*>(a.w_alt);
+  }
   // The small scale/bias loads go first: loads complete in order, so a scale
   // queued behind the whole weight stream would hold back the first row.
 #pragma unroll
   for (int r = 0; r < kRowsPerWave; ++r) {
-    const int row = (row0 + r < N) ? row0 + r : N - 1; // clamp: stay in bounds
+    const int row = row_of(r);
     sbw[r] = *reinterpret_cast<const uint32_t*>(
-        sb_lane_base + static_cast<size_t>(row) * groups * 2);
+        ((GLU && r == 1) ? sb_lane_alt : sb_lane_base) + static_cast<size_t>(row) * groups * 2);
   }
 #pragma unroll
   for (int r = 0; r < kRowsPerWave; ++r) {
-    const int row = (row0 + r < N) ? row0 + r : N - 1;
-    const uint8_t* wrow = p.w + static_cast<size_t>(row) * row_bytes;
+    const int row = row_of(r);
+    const uint8_t* wrow = ((GLU && r == 1) ? w_alt : p.w) + static_cast<size_t>(row) * row_bytes;
 #pragma unroll
     for (int c = 0; c < CPW; ++c) {
       const uint32_t byte = static_cast<uint32_t>(c0 + c) * kChunkBytes + lane * 16;
@@ -460,7 +476,17 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
       y[r][m] = wave_sum_dpp(y[r][m]);
     }
   }
-  if constexpr (KW == 1) {
+  if constexpr (GLU) {
+    if (lane == 63 && row0 < N) {
+      // the roundings of the unfused chain: both products, the sigmoid, gate *
+      // sigmoid and the final product are each rounded to T
+      const float g = to_f32(from_f32<T>(y[0][0]));
+      const float u = to_f32(from_f32<T>(y[1][0]));
+      const float sg = to_f32(from_f32<T>(1.0f / (1.0f + __expf(-g))));
+      const float h = to_f32(from_f32<T>(g * sg));
+      p.out[row0] = from_f32<T>(h * u);
+    }
+  } else if constexpr (KW == 1) {
     if (lane == 63) {
 #pragma unroll
       for (int r = 0; r < kRowsPerWave; ++r) {
@@ -601,6 +627,70 @@ bool qmv_stream_supported(const QmmArgs& a, int gs, int bits, int dtype) {
     return false; // K beyond 8 k-waves
   }
   return smem <= 72 * 1024; // x image of 64 KiB (M = 2, K = 16384, 4-bit) + its sums
+}
+
+// Gated form (y = silu(gate . x) * (up . x), a.w_alt set): one row of x, one
+// k-wave, shapes whose waves own a pair of rows (4-bit with groups of 64 / 128 up
+// to K = 4096; 8-bit with groups of 32 up to K = 2048).
+bool qmv_stream_glu_supported(const QmmArgs& a, int gs, int bits, int dtype) {
+  if (a.w_alt == nullptr || a.M != 1 || a.L != 1 || a.lhs_indices != nullptr) {
+    return false;
+  }
+  if (!qmv_stream_supported(a, gs, bits, dtype)) {
+    return false;
+  }
+  bool ok = false;
+  auto probe = [&](auto bval, auto gval) {
+    constexpr int B = decltype(bval)::value;
+    constexpr int G = decltype(gval)::value;
+    using S = StreamShape<B, G>;
+    ok = S::kRowsPerWave == 2 && stream_plan<B, G>(a.K, 2 * a.N, 1).kw == 1;
+  };
+  if (bits == 4 && gs == 64) {
+    probe(IntC<4>{}, IntC<64>{});
+  } else if (bits == 4 && gs == 128) {
+    probe(IntC<4>{}, IntC<128>{});
+  } else if (bits == 8 && gs == 32) {
+    probe(IntC<8>{}, IntC<32>{});
+  }
+  return ok;
+}
+
+int launch_qmv_stream_glu(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  if (!qmv_stream_glu_supported(a, gs, bits, dtype)) {
+    return fail(MLXROCM_UNSUPPORTED, "[qmv] shape not covered by the gated GEMV");
+  }
+  auto run = [&](auto tval, auto bval, auto gval) -> int {
+    using T = decltype(tval);
+    constexpr int B = decltype(bval)::value;
+    constexpr int G = decltype(gval)::value;
+    using S = StreamShape<B, G>;
+    if constexpr (S::kRowsPerWave != 2) {
+      return fail(MLXROCM_UNSUPPORTED, "[qmv] shape not covered by the gated GEMV");
+    } else {
+      const StreamPlan pl = stream_plan<B, G>(a.K, 2 * a.N, 1);
+      const size_t smem = stream_smem_bytes<B, G>(1, a.K, pl.rw, 1, 1);
+      const bool full = a.K == S::kChunksPerWave * S::kChunkCodes;
+      const dim3 grid((a.N + pl.rw - 1) / pl.rw, 1);
+      constexpr bool MD = B == 4 && G >= 64;
+      auto go = [&](auto rwv) -> int {
+        constexpr int RW = decltype(rwv)::value;
+        auto kern = full ? qmv_stream_kernel<T, B, G, 1, RW, 1, true, 1, MD, true>
+                         : qmv_stream_kernel<T, B, G, 1, RW, 1, false, 1, MD, true>;
+        kern<<<grid, RW * 64, smem, s>>>(a);
+        MLXROCM_HIP_TRY(hipGetLastError());
+        return static_cast<int>(MLXROCM_OK);
+      };
+      return pl.rw == 4 ? go(IntC<4>{}) : go(IntC<8>{});
+    }
+  };
+  auto by_type = [&](auto bval, auto gval) -> int {
+    return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}, bval, gval) : run(f16_t{}, bval, gval);
+  };
+  if (bits == 4) {
+    return gs == 64 ? by_type(IntC<4>{}, IntC<64>{}) : by_type(IntC<4>{}, IntC<128>{});
+  }
+  return by_type(IntC<8>{}, IntC<32>{});
 }
 
 int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {

@@ -361,7 +361,10 @@ def test_quantized_swiglu_matches_the_unfused_chain(oracle, gpu, dtype, bits, gs
     """silu(gate(x)) * up(x) in one call against the same chain built from the
     oracle's two products, with every intermediate rounded to the element type as
     `x * sigmoid(x)` and the multiply round it; 1..8 rows of x, ragged N."""
-    for M, N, K in ((1, 200, 512), (2, 96, 4096), (4, 64, 1024), (8, 130, 2048)):
+    # one row at 4 bits runs with the gate inside the GEMV (K of a partial chunk,
+    # of exactly one wave's chunks, a grid of four- and of eight-wave workgroups)
+    for M, N, K in ((1, 200, 512), (1, 1000, 4096), (1, 6144, 4096), (2, 96, 4096), (4, 64, 1024),
+                    (8, 130, 2048), (1, 40, 8192)):
         wg = normal_weights((N, K), dtype, seed=bits + M)
         wu = normal_weights((N, K), dtype, seed=bits + M + 100)
         x = activations((M, K), dtype, seed=K + M)
