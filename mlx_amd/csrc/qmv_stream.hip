@@ -630,8 +630,16 @@ bool qmv_stream_supported(const QmmArgs& a, int gs, int bits, int dtype) {
 }
 
 // Gated form (y = silu(gate . x) * (up . x), a.w_alt set): one row of x, one
-// k-wave, shapes whose waves own a pair of rows (4-bit with groups of 64 / 128 up
-// to K = 4096; 8-bit with groups of 32 up to K = 2048).
+// k-wave (4-bit: K <= 4096 with groups of 64 / 128, K <= 2048 with groups of 32;
+// 8-bit: K <= 4096 with groups of 64 / 128, K <= 2048 with groups of 32).  A wave
+// owns one row pair: shapes whose waves own four rows (4-bit, groups of 32) are
+// not covered.
+template <int BITS, int GS>
+constexpr int glu_row_multiple() {
+  // rows per wave must come to two
+  return StreamShape<BITS, GS>::kRowsPerWave == 1 ? 2 : (StreamShape<BITS, GS>::kRowsPerWave == 2 ? 1 : 0);
+}
+
 bool qmv_stream_glu_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   if (a.w_alt == nullptr || a.M != 1 || a.L != 1 || a.lhs_indices != nullptr) {
     return false;
@@ -643,15 +651,21 @@ bool qmv_stream_glu_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   auto probe = [&](auto bval, auto gval) {
     constexpr int B = decltype(bval)::value;
     constexpr int G = decltype(gval)::value;
-    using S = StreamShape<B, G>;
-    ok = S::kRowsPerWave == 2 && stream_plan<B, G>(a.K, 2 * a.N, 1).kw == 1;
+    ok = glu_row_multiple<B, G>() != 0 && stream_plan<B, G>(a.K, 2 * a.N, 1).kw == 1;
   };
-  if (bits == 4 && gs == 64) {
-    probe(IntC<4>{}, IntC<64>{});
-  } else if (bits == 4 && gs == 128) {
-    probe(IntC<4>{}, IntC<128>{});
-  } else if (bits == 8 && gs == 32) {
-    probe(IntC<8>{}, IntC<32>{});
+  auto by_group = [&](auto bval) {
+    if (gs == 32) {
+      probe(bval, IntC<32>{});
+    } else if (gs == 64) {
+      probe(bval, IntC<64>{});
+    } else {
+      probe(bval, IntC<128>{});
+    }
+  };
+  if (bits == 4) {
+    by_group(IntC<4>{});
+  } else {
+    by_group(IntC<8>{});
   }
   return ok;
 }
@@ -665,18 +679,19 @@ int launch_qmv_stream_glu(const QmmArgs& a, int gs, int bits, int dtype, hipStre
     constexpr int B = decltype(bval)::value;
     constexpr int G = decltype(gval)::value;
     using S = StreamShape<B, G>;
-    if constexpr (S::kRowsPerWave != 2) {
+    constexpr int RM = glu_row_multiple<B, G>();
+    if constexpr (RM == 0) {
       return fail(MLXROCM_UNSUPPORTED, "[qmv] shape not covered by the gated GEMV");
     } else {
       const StreamPlan pl = stream_plan<B, G>(a.K, 2 * a.N, 1);
-      const size_t smem = stream_smem_bytes<B, G>(1, a.K, pl.rw, 1, 1);
+      const size_t smem = stream_smem_bytes<B, G>(1, a.K, pl.rw, 1, RM);
       const bool full = a.K == S::kChunksPerWave * S::kChunkCodes;
       const dim3 grid((a.N + pl.rw - 1) / pl.rw, 1);
       constexpr bool MD = B == 4 && G >= 64;
       auto go = [&](auto rwv) -> int {
         constexpr int RW = decltype(rwv)::value;
-        auto kern = full ? qmv_stream_kernel<T, B, G, 1, RW, 1, true, 1, MD, true>
-                         : qmv_stream_kernel<T, B, G, 1, RW, 1, false, 1, MD, true>;
+        auto kern = full ? qmv_stream_kernel<T, B, G, 1, RW, 1, true, RM, MD, true>
+                         : qmv_stream_kernel<T, B, G, 1, RW, 1, false, RM, MD, true>;
         kern<<<grid, RW * 64, smem, s>>>(a);
         MLXROCM_HIP_TRY(hipGetLastError());
         return static_cast<int>(MLXROCM_OK);
@@ -684,13 +699,20 @@ int launch_qmv_stream_glu(const QmmArgs& a, int gs, int bits, int dtype, hipStre
       return pl.rw == 4 ? go(IntC<4>{}) : go(IntC<8>{});
     }
   };
-  auto by_type = [&](auto bval, auto gval) -> int {
-    return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}, bval, gval) : run(f16_t{}, bval, gval);
+  auto by_group = [&](auto tval, auto bval) -> int {
+    switch (gs) {
+      case 32:
+        return run(tval, bval, IntC<32>{});
+      case 64:
+        return run(tval, bval, IntC<64>{});
+      default:
+        return run(tval, bval, IntC<128>{});
+    }
   };
-  if (bits == 4) {
-    return gs == 64 ? by_type(IntC<4>{}, IntC<64>{}) : by_type(IntC<4>{}, IntC<128>{});
-  }
-  return by_type(IntC<8>{}, IntC<32>{});
+  auto by_bits = [&](auto tval) -> int {
+    return bits == 4 ? by_group(tval, IntC<4>{}) : by_group(tval, IntC<8>{});
+  };
+  return dtype == MLXROCM_BFLOAT16 ? by_bits(bf16_t{}) : by_bits(f16_t{});
 }
 
 int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
