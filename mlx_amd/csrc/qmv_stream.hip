@@ -204,7 +204,7 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
   const uint32_t row_bytes = static_cast<uint32_t>(K / 8) * BITS;
   // GLU: the wave's two rows are row n of the gate weight (a.w) and row n of the
   // up weight (a.w_alt); it writes y[n] = silu(gate . x) * (up . x).
-  static_assert(!GLU || (KW == 1 && kRowsPerWave == 2 && M == 1), "gated form: one k-wave, a row pair");
+  static_assert(!GLU || (kRowsPerWave == 2 && M == 1), "gated form: a row pair per wave, one row of x");
   const int row0 = GLU ? (blockIdx.x * RW + rw) : (blockIdx.x * RW + rw) * kRowsPerWave;
   auto row_of = [&](int r) {
     const int row = GLU ? row0 : row0 + r;
@@ -476,15 +476,18 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
       y[r][m] = wave_sum_dpp(y[r][m]);
     }
   }
-  if constexpr (GLU) {
+  // the gate with the roundings of the unfused chain: both products, the sigmoid,
+  // gate * sigmoid and the final product are each rounded to T
+  auto gated = [](float gate, float up) {
+    const float g = to_f32(from_f32<T>(gate));
+    const float u = to_f32(from_f32<T>(up));
+    const float sg = to_f32(from_f32<T>(1.0f / (1.0f + __expf(-g))));
+    const float h = to_f32(from_f32<T>(g * sg));
+    return from_f32<T>(h * u);
+  };
+  if constexpr (GLU && KW == 1) {
     if (lane == 63 && row0 < N) {
-      // the roundings of the unfused chain: both products, the sigmoid, gate *
-      // sigmoid and the final product are each rounded to T
-      const float g = to_f32(from_f32<T>(y[0][0]));
-      const float u = to_f32(from_f32<T>(y[1][0]));
-      const float sg = to_f32(from_f32<T>(1.0f / (1.0f + __expf(-g))));
-      const float h = to_f32(from_f32<T>(g * sg));
-      p.out[row0] = from_f32<T>(h * u);
+      p.out[row0] = gated(y[0][0], y[1][0]);
     }
   } else if constexpr (KW == 1) {
     if (lane == 63) {
@@ -512,7 +515,20 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
       }
     }
     __syncthreads();
-    if (tid < RW * kRowsPerWave * M) {
+    if constexpr (GLU) {
+      if (tid < RW) {
+        float gate = 0.0f, up = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KW; ++k) {
+          gate += red[(tid * KW + k) * 2 + 0];
+          up += red[(tid * KW + k) * 2 + 1];
+        }
+        const int n = blockIdx.x * RW + tid;
+        if (n < N) {
+          p.out[n] = gated(gate, up);
+        }
+      }
+    } else if (tid < RW * kRowsPerWave * M) {
       const int m = tid % M;
       const int r = (tid / M) % kRowsPerWave;
       const int w = tid / (M * kRowsPerWave);
@@ -629,11 +645,9 @@ bool qmv_stream_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   return smem <= 72 * 1024; // x image of 64 KiB (M = 2, K = 16384, 4-bit) + its sums
 }
 
-// Gated form (y = silu(gate . x) * (up . x), a.w_alt set): one row of x, one
-// k-wave (4-bit: K <= 4096 with groups of 64 / 128, K <= 2048 with groups of 32;
-// 8-bit: K <= 4096 with groups of 64 / 128, K <= 2048 with groups of 32).  A wave
-// owns one row pair: shapes whose waves own four rows (4-bit, groups of 32) are
-// not covered.
+// Gated form (y = silu(gate . x) * (up . x), a.w_alt set): one row of x, every K
+// the kernel covers.  A wave owns one row pair: shapes whose waves own four rows
+// (4-bit, groups of 32) are not covered.
 template <int BITS, int GS>
 constexpr int glu_row_multiple() {
   // rows per wave must come to two
@@ -651,7 +665,7 @@ bool qmv_stream_glu_supported(const QmmArgs& a, int gs, int bits, int dtype) {
   auto probe = [&](auto bval, auto gval) {
     constexpr int B = decltype(bval)::value;
     constexpr int G = decltype(gval)::value;
-    ok = glu_row_multiple<B, G>() != 0 && stream_plan<B, G>(a.K, 2 * a.N, 1).kw == 1;
+    ok = glu_row_multiple<B, G>() != 0 && stream_plan<B, G>(a.K, 2 * a.N, 1).kw != 0;
   };
   auto by_group = [&](auto bval) {
     if (gs == 32) {
@@ -684,19 +698,35 @@ int launch_qmv_stream_glu(const QmmArgs& a, int gs, int bits, int dtype, hipStre
       return fail(MLXROCM_UNSUPPORTED, "[qmv] shape not covered by the gated GEMV");
     } else {
       const StreamPlan pl = stream_plan<B, G>(a.K, 2 * a.N, 1);
-      const size_t smem = stream_smem_bytes<B, G>(1, a.K, pl.rw, 1, RM);
-      const bool full = a.K == S::kChunksPerWave * S::kChunkCodes;
+      const size_t smem = stream_smem_bytes<B, G>(1, a.K, pl.rw, pl.kw, RM);
+      const bool full = a.K == pl.kw * S::kChunksPerWave * S::kChunkCodes;
       const dim3 grid((a.N + pl.rw - 1) / pl.rw, 1);
       constexpr bool MD = B == 4 && G >= 64;
-      auto go = [&](auto rwv) -> int {
+      auto go = [&](auto rwv, auto kwv) -> int {
         constexpr int RW = decltype(rwv)::value;
-        auto kern = full ? qmv_stream_kernel<T, B, G, 1, RW, 1, true, RM, MD, true>
-                         : qmv_stream_kernel<T, B, G, 1, RW, 1, false, RM, MD, true>;
-        kern<<<grid, RW * 64, smem, s>>>(a);
+        constexpr int KW = decltype(kwv)::value;
+        auto kern = full ? qmv_stream_kernel<T, B, G, 1, RW, KW, true, RM, MD, true>
+                         : qmv_stream_kernel<T, B, G, 1, RW, KW, false, RM, MD, true>;
+        if (smem > 48 * 1024) {
+          MLXROCM_HIP_TRY(hipFuncSetAttribute(
+              reinterpret_cast<const void*>(kern),
+              hipFuncAttributeMaxDynamicSharedMemorySize,
+              static_cast<int>(smem)));
+        }
+        kern<<<grid, RW * KW * 64, smem, s>>>(a);
         MLXROCM_HIP_TRY(hipGetLastError());
         return static_cast<int>(MLXROCM_OK);
       };
-      return pl.rw == 4 ? go(IntC<4>{}) : go(IntC<8>{});
+      switch (pl.kw) {
+        case 1:
+          return pl.rw == 4 ? go(IntC<4>{}, IntC<1>{}) : go(IntC<8>{}, IntC<1>{});
+        case 2:
+          return go(IntC<4>{}, IntC<2>{});
+        case 4:
+          return go(IntC<2>{}, IntC<4>{});
+        default:
+          return go(IntC<1>{}, IntC<8>{});
+      }
     }
   };
   auto by_group = [&](auto tval, auto bval) -> int {

@@ -364,7 +364,7 @@ def test_quantized_swiglu_matches_the_unfused_chain(oracle, gpu, dtype, bits, gs
     # one row at 4 bits runs with the gate inside the GEMV (K of a partial chunk,
     # of exactly one wave's chunks, a grid of four- and of eight-wave workgroups)
     for M, N, K in ((1, 200, 512), (1, 1000, 4096), (1, 6144, 4096), (2, 96, 4096), (4, 64, 1024),
-                    (8, 130, 2048), (1, 40, 8192)):
+                    (8, 130, 2048), (1, 40, 8192), (1, 48, 14336)):
         wg = normal_weights((N, K), dtype, seed=bits + M)
         wu = normal_weights((N, K), dtype, seed=bits + M + 100)
         x = activations((M, K), dtype, seed=K + M)
