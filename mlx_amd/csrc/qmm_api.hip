@@ -405,7 +405,7 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
       const long wgs = qmv_quad_workgroups_two_sets(a, bits);
       const long rounds = (wgs + cus - 1) / cus;
       // a single round, or more than 7/8 of the slots of all rounds in use
-      many_rows = long_k || a.K >= 8192 || gs == 32 ||
+      many_rows = a.K >= 8192 || gs == 32 ||
           (wgs > 0 && (rounds <= 1 || wgs * 8 > rounds * cus * 7));
     }
     const bool use = (a.M >= 2 && a.M <= 4) ||

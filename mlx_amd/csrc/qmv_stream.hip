@@ -37,7 +37,6 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kChunkBytes = 1024; // 64 lanes x 16 bytes
-constexpr int kChains = 2; // independent accumulators per 16-byte load
 
 template <typename T>
 struct Dot;
@@ -415,12 +414,13 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
         const float d23 = (lane & 1) ? acc[3] : acc[2];
         dot[0] = (lane & 2) ? d23 : d01;
       } else {
+      // two accumulator chains: dwords 0, 2 and dwords 1, 3
       float dacc[M][4];
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-          dacc[m][d] = (d < kChains) ? 0.0f : dacc[m][d >= kChains ? d - kChains : 0];
+          dacc[m][d] = d < 2 ? 0.0f : dacc[m][d >= 2 ? d - 2 : 0];
         }
         if constexpr (BITS == 4) {
           const uint32_t q0 = (w[d] & w4c.mask) | w4c.magic;
@@ -445,13 +445,7 @@ __global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs 
       }
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        if constexpr (kChains == 4) {
-          dot[m] = (dacc[m][0] + dacc[m][1]) + (dacc[m][2] + dacc[m][3]);
-        } else if constexpr (kChains == 2) {
-          dot[m] = dacc[m][2] + dacc[m][3];
-        } else {
-          dot[m] = dacc[m][3];
-        }
+        dot[m] = dacc[m][2] + dacc[m][3];
       }
       }
       const uint32_t s_word = static_cast<uint32_t>(
