@@ -143,8 +143,9 @@ int mlxrocm_gguf_repack(
  * parts for the matrix cores); 16-bit calls whose tile grid would leave compute
  * units idle (K is split; fp32 partial results); 16-bit prefill calls with
  * M >= 512 and every transpose == 0 call on the matrix cores (a transposed copy
- * of scales and biases, 4 * N * K / group_size bytes).  Decode calls (M <= 32)
- * with transpose != 0 allocate nothing.  A call that needs a larger buffer than
+ * of scales and biases, 4 * N * K / group_size bytes); transpose == 0 calls with
+ * 1..4 rows of x and K > 64 (one fp32 plane of the output per 64 rows of K).
+ * Decode calls (M <= 32) with transpose != 0 allocate nothing.  A call that needs a larger buffer than
  * the stream holds synchronizes that stream before replacing it.
  */
 int mlxrocm_qmm(
