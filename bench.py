@@ -29,7 +29,9 @@ BF16_PEAK_TFLOPS = 2500.0
 # a copy of known size (profiles/qmv_stream_4bit_g64_bf16_14336x4096.md and
 # profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md).
 QMV_TRAFFIC_BYTES = 33224063
+QMV_TRAFFIC_SOURCE = "profiles/qmv_stream_4bit_g64_bf16_14336x4096.md"
 QMM_T_TRAFFIC_BYTES = 260219533
+QMM_T_TRAFFIC_SOURCE = "profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md"
 
 N, K = 14336, 4096
 BITS, GS = 4, 64
@@ -43,33 +45,51 @@ def qmv_bytes(M: int, n: int, k: int, bits: int, gs: int, esize: int) -> int:
 
 
 class Launcher:
-    """Issues `steps` launches of fn(i, stream) on one stream, either directly
-    or by replaying a HIP graph that holds one pass over the weight ring (the
-    kernel is a few microseconds long, shorter than a Python-driven launch)."""
+    """Issues launches of fn(i, stream) on one stream, either directly or by
+    replaying HIP graphs: one graph holds a pass over the weight ring (the
+    kernel is a few microseconds long, shorter than a Python-driven launch), a
+    second one the remainder, so that any number of launches can be issued
+    exactly."""
 
     def __init__(self, torch, fn, period: int, use_graph: bool):
         self.torch, self.fn, self.period = torch, fn, period
         self.stream = torch.cuda.Stream()
-        self.graph = None
+        self.use_graph = use_graph
+        self.graphs = {}
         self.stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(self.stream):
             for i in range(period):
                 fn(i, self.stream.cuda_stream)
         self.stream.synchronize()
         if use_graph:
-            self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph, stream=self.stream):
-                for i in range(period):
-                    fn(i, torch.cuda.current_stream().cuda_stream)
+            self._graph(period)
+
+    def _graph(self, count: int):
+        if count not in self.graphs:
+            graph = self.torch.cuda.CUDAGraph()
+            with self.torch.cuda.graph(graph, stream=self.stream):
+                for i in range(count):
+                    self.fn(i, self.torch.cuda.current_stream().cuda_stream)
+            self.graphs[count] = graph
+        return self.graphs[count]
+
+    def prepare(self, steps: int) -> None:
+        """Capture what run(steps) replays, outside any timed region."""
+        if self.use_graph and steps % self.period:
+            self._graph(steps % self.period)
 
     def run(self, steps: int) -> int:
-        """Enqueue at least `steps` launches; returns how many were issued."""
+        """Enqueue exactly `steps` launches."""
         with self.torch.cuda.stream(self.stream):
-            if self.graph is not None:
-                replays = (steps + self.period - 1) // self.period
-                for _ in range(replays):
-                    self.graph.replay()
-                return replays * self.period
+            if self.use_graph:
+                full, rest = divmod(steps, self.period)
+                ring = self._graph(self.period)
+                tail = self._graph(rest) if rest else None
+                for _ in range(full):
+                    ring.replay()
+                if tail is not None:
+                    tail.replay()
+                return steps
             for i in range(steps):
                 self.fn(i, self.stream.cuda_stream)
             return steps
@@ -79,6 +99,7 @@ def hip_event_ms(lib, launcher: "Launcher", steps: int) -> float:
     """Milliseconds per launch, measured with HIP events recorded on the
     stream the kernels are launched on."""
     stream = launcher.stream.cuda_stream
+    launcher.prepare(steps)
     start, stop = ctypes.c_void_p(), ctypes.c_void_p()
     assert lib.mlxrocm_event_create(ctypes.byref(start)) == 0
     assert lib.mlxrocm_event_create(ctypes.byref(stop)) == 0
@@ -91,6 +112,19 @@ def hip_event_ms(lib, launcher: "Launcher", steps: int) -> float:
     lib.mlxrocm_event_destroy(start)
     lib.mlxrocm_event_destroy(stop)
     return ms.value / steps
+
+
+# Timing protocol of the headline figures: after at least MIN_WARMUP untimed
+# launches, REPEATS timed regions of max(--steps, MIN_LAUNCHES) launches each,
+# HIP events around every region; the median region is the figure.
+REPEATS = 7
+MIN_LAUNCHES = 100
+MIN_WARMUP = 10
+
+
+def median_event_ms(lib, launcher: "Launcher", launches: int, repeats: int = REPEATS):
+    samples = sorted(hip_event_ms(lib, launcher, launches) for _ in range(repeats))
+    return samples[len(samples) // 2], samples
 
 
 def cpu_baseline(x_cpu, wq_cpu, s_cpu, b_cpu, nbytes: int) -> dict:
@@ -189,12 +223,14 @@ def sweep(torch, mlx_amd, dev) -> list:
         ring = ring_of(q, wbytes) if small else [q]
         x = torch.randn((M, k), generator=g, dtype=torch.float32).to(dtype).to(dev)
         out = torch.empty((M, n), dtype=dtype, device=dev)
+        ws_bytes = lib.mlxrocm_qmm_workspace_size(M, n, k, 1, 0, gs, bits, code, int(transpose))
+        ws = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=dev)
 
         def step(i, stream):
             wq_, s_, b_ = ring[i % len(ring)]
             rc = lib.mlxrocm_qmm(x.data_ptr(), wq_.data_ptr(), s_.data_ptr(), b_.data_ptr(),
                                  out.data_ptr(), M, n, k, 1, M * k, 0, 0, gs, bits, code,
-                                 int(transpose), stream)
+                                 int(transpose), ws.data_ptr(), ws_bytes, stream)
             if rc != 0:
                 raise RuntimeError(_lib.last_error())
 
@@ -258,7 +294,8 @@ def sweep(torch, mlx_amd, dev) -> list:
             a, b = ring[2 * (i % R)], ring[2 * (i % R) + 1]
             for q_, o_ in ((a, gate), (b, up)):
                 rc = lib.mlxrocm_qmm(x.data_ptr(), q_[0].data_ptr(), q_[1].data_ptr(), q_[2].data_ptr(),
-                                     o_.data_ptr(), M, n, k, 1, M * k, 0, 0, gs, bits, 2, 1, stream)
+                                     o_.data_ptr(), M, n, k, 1, M * k, 0, 0, gs, bits, 2, 1,
+                                     None, 0, stream)
                 if rc != 0:
                     raise RuntimeError(_lib.last_error())
             torch.mul(torch.nn.functional.silu(gate), up, out=out)
@@ -410,32 +447,32 @@ def main() -> int:
     def qmv_step(i, stream):
         wq_p, s_p, b_p = ptrs[i % RING]
         rc = lib.mlxrocm_qmm(x.data_ptr(), wq_p, s_p, b_p, out.data_ptr(),
-                             1, N, K, 1, K, 0, 0, GS, BITS, code, 1, stream)
+                             1, N, K, 1, K, 0, 0, GS, BITS, code, 1, None, 0, stream)
         if rc != 0:
             raise RuntimeError(_lib.last_error())
 
     if args.only in (None, "qmv"):
         launcher = Launcher(torch, qmv_step, RING, not args.no_graph)
-        launcher.run(args.warmup)
+        warmup = max(args.warmup, MIN_WARMUP)
+        launches = max(args.steps, MIN_LAUNCHES)
+        launcher.prepare(warmup)
+        launcher.prepare(launches)
+        launcher.run(warmup)
         torch.cuda.synchronize()
-        steps = (args.steps + RING - 1) // RING * RING if not args.no_graph else args.steps
-        t0 = time.perf_counter()
-        ev_ms = hip_event_ms(lib, launcher, steps)
-        torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-        args.steps = steps
+        ev_ms, samples = median_event_ms(lib, launcher, launches)
         # single hot buffer: served from the Infinity Cache, reported separately
         hot = Launcher(torch, lambda i, st: qmv_step(0, st), RING, not args.no_graph)
-        llc_ms = hip_event_ms(lib, hot, steps)
+        hot.run(warmup)
+        llc_ms, _ = median_event_ms(lib, hot, launches)
         gbps = nbytes / (ev_ms * 1e-3) / 1e9
         result.update({
             "metric": "4-bit qmv HBM GB/s (%peak) at 14336x4096; qmm_t TFLOP/s (%peak) at M=2048",
-            "value": round(nbytes / (wall_ms * 1e-3) / 1e9, 2),
+            "value": round(gbps, 2),
             "unit": "GB/s",
             "n_gpus": 1,
             "steps": args.steps,
             "warmup": args.warmup,
-            "ms_per_step": round(wall_ms, 6),
+            "ms_per_step": round(ev_ms, 6),
             "higher_is_better": True,
             "scaling": "weak",
             "vs_baseline": None,
@@ -448,6 +485,14 @@ def main() -> int:
                 "launch": "direct" if args.no_graph else f"hip graph of {RING} launches",
                 "kernel": lib.mlxrocm_qmm_kernel_name(1, N, K, 1, GS, BITS, code, 1).decode(),
             },
+            "timing": {
+                "method": "HIP events on the launch stream; median of the timed regions",
+                "launches_timed": launches,
+                "repeats": len(samples),
+                "warmup_launches": warmup,
+                "us_per_launch_min_median_max": [round(samples[0] * 1e3, 3), round(ev_ms * 1e3, 3),
+                                                 round(samples[-1] * 1e3, 3)],
+            },
             "roofline": {
                 "bound": "hbm",
                 "achieved": round(gbps, 2),
@@ -455,6 +500,7 @@ def main() -> int:
                 "unit": "GB/s",
                 "frac": round(gbps / HBM_PEAK_GBPS, 4),
                 "traffic": QMV_TRAFFIC_BYTES,
+                "traffic_source": QMV_TRAFFIC_SOURCE,
                 "kernel_us": round(ev_ms * 1e3, 3),
                 "bytes_per_launch": nbytes,
                 "llc_resident_gbps": round(nbytes / (llc_ms * 1e-3) / 1e9, 2),
@@ -466,27 +512,33 @@ def main() -> int:
         xm = torch.randn((QMM_M, K), generator=g, dtype=torch.float32).to(dt).to(dev)
         outm = torch.empty((QMM_M, N), dtype=dt, device=dev)
         flops = 2.0 * QMM_M * N * K
+        ws_bytes = lib.mlxrocm_qmm_workspace_size(QMM_M, N, K, 1, 0, GS, BITS, code, 1)
+        ws = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=dev)
 
         def qmm_step(i, stream):
             wq_p, s_p, b_p = ptrs[i % RING]
             rc = lib.mlxrocm_qmm(xm.data_ptr(), wq_p, s_p, b_p, outm.data_ptr(),
-                                 QMM_M, N, K, 1, QMM_M * K, 0, 0, GS, BITS, code, 1, stream)
+                                 QMM_M, N, K, 1, QMM_M * K, 0, 0, GS, BITS, code, 1,
+                                 ws.data_ptr(), ws_bytes, stream)
             if rc != 0:
                 raise RuntimeError(_lib.last_error())
 
-        steps = max(RING, args.steps // 20)
+        launches = max(args.steps // 20, MIN_LAUNCHES)
         mm = Launcher(torch, qmm_step, RING, False)
-        mm.run(max(3, args.warmup // 20))
+        mm.run(max(args.warmup // 20, MIN_WARMUP))
         torch.cuda.synchronize()
-        ms = hip_event_ms(lib, mm, steps)
+        ms, samples = median_event_ms(lib, mm, launches, repeats=5)
         tflops = flops / (ms * 1e-3) / 1e12
         result["qmm_t"] = {
             "workload": f"qmm_t prefill GEMM: x bf16 [{QMM_M},{K}], W [{N},{K}] 4-bit group 64",
             "kernel": lib.mlxrocm_qmm_kernel_name(QMM_M, N, K, 1, GS, BITS, code, 1).decode(),
             "value": round(tflops, 2),
             "unit": "TFLOP/s",
-            "steps": steps,
+            "launches_timed": launches,
+            "repeats": len(samples),
             "ms_per_step": round(ms, 5),
+            "us_per_launch_min_median_max": [round(samples[0] * 1e3, 2), round(ms * 1e3, 2),
+                                             round(samples[-1] * 1e3, 2)],
             "roofline": {
                 "bound": "mfma",
                 "achieved": round(tflops, 2),
@@ -494,6 +546,7 @@ def main() -> int:
                 "unit": "TFLOP/s",
                 "frac": round(tflops / BF16_PEAK_TFLOPS, 4),
                 "traffic": QMM_T_TRAFFIC_BYTES,
+                "traffic_source": QMM_T_TRAFFIC_SOURCE,
             },
         }
 

@@ -4,7 +4,9 @@
  *
  * This is the thin layer the C++ `eval_gpu` bodies of a `mlx/backend/rocm` tree
  * call: plain pointers and sizes, a HIP stream handle, an int status.  Nothing
- * here allocates or frees device memory except the mlxrocm_malloc family.
+ * here allocates or frees device memory except the mlxrocm_malloc family:
+ * entry points that need device scratch take it from a workspace the caller
+ * provides (its size comes from the matching *_workspace_size function).
  *
  * Conventions
  *   - All data pointers are DEVICE pointers (or host-visible pinned memory).
@@ -28,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MLXROCM_ABI_VERSION 1
+#define MLXROCM_ABI_VERSION 2
 
 typedef enum {
   MLXROCM_OK = 0,
@@ -137,17 +139,31 @@ int mlxrocm_gguf_repack(
  * 0 when one weight matrix is shared by every batch (w.ndim() == 2 in MLX).
  * The kernel is picked from M, N, K, bits, group_size and dtype.
  *
- * Some calls keep device scratch inside the library -- one buffer per stream,
- * allocated (hipMalloc) or grown on the first call that needs it and kept until
- * the process ends: float32 operands with M > 8 (x is split into two bfloat16
- * parts for the matrix cores); 16-bit calls whose tile grid would leave compute
- * units idle (K is split; fp32 partial results); 16-bit prefill calls with
- * M >= 512 and every transpose == 0 call on the matrix cores (a transposed copy
- * of scales and biases, 4 * N * K / group_size bytes); transpose == 0 calls with
- * 1..4 rows of x and K > 64 (one fp32 plane of the output per 64 rows of K).
- * Decode calls (M <= 32) with transpose != 0 allocate nothing.  A call that needs a larger buffer than
- * the stream holds synchronizes that stream before replacing it.
+ * `workspace` is device memory of at least mlxrocm_qmm_workspace_size(...)
+ * bytes, 256-byte aligned, owned by the caller (an eval_gpu body allocates it
+ * like any other temporary and keeps it until the stream has passed the call);
+ * it may be NULL when that size is 0.  Shapes that use it: float32 operands
+ * with M > 8 and transpose != 0 (x split into two bfloat16 parts for the
+ * matrix cores); 16-bit calls whose tile grid would leave compute units idle (K
+ * is split; fp32 partial results); 16-bit prefill calls with M >= 512 and every
+ * transpose == 0 call on the matrix cores (a transposed copy of scales and
+ * biases, 4 * N * K / group_size bytes); transpose == 0 calls with 1..4 rows of
+ * x and K > 64 (one fp32 plane of the output per 64 rows of K).  Decode calls
+ * (M <= 32) with transpose != 0 never use one, except 17..32 rows over a K
+ * beyond 8192 and a narrow N.  The call only enqueues work: it allocates
+ * nothing, takes no lock and does not synchronize, so it can be captured in a
+ * HIP graph.  A workspace that is too small is MLXROCM_INVALID_ARGUMENT.
  */
+size_t mlxrocm_qmm_workspace_size(
+    int M,
+    int N,
+    int K,
+    int L,
+    int batched_weights, /* != 0: one weight matrix per batch entry */
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose);
 int mlxrocm_qmm(
     const void* x,
     const uint32_t* wq,
@@ -165,6 +181,8 @@ int mlxrocm_qmm(
     int bits,
     int dtype,
     int transpose,
+    void* workspace,
+    size_t workspace_bytes,
     mlxrocm_stream_t stream);
 
 /*

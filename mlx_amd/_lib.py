@@ -29,9 +29,10 @@ SIGNATURES = {
     "mlxrocm_affine_quantize": (_i, [_p, _p, _p, _p, _sz, _i, _i, _i, _p]),
     "mlxrocm_affine_dequantize": (_i, [_p, _p, _p, _p, _sz, _i, _i, _i, _p]),
     "mlxrocm_gguf_repack": (_i, [_p, _p, _p, _p, _sz, _i, _p]),
+    "mlxrocm_qmm_workspace_size": (_sz, [_i] * 9),
     "mlxrocm_qmm": (
         _i,
-        [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p],
+        [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p, _sz, _p],
     ),
     "mlxrocm_qmm_swiglu_workspace_size": (_sz, [_i, _i, _i]),
     "mlxrocm_qmm_swiglu": (_i, [_p] * 9 + [_i] * 6 + [_p]),
@@ -92,7 +93,7 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
-    if lib.mlxrocm_abi_version() != 1:
+    if lib.mlxrocm_abi_version() != 2:
         raise ImportError("libmlx_rocm_qmm.so ABI version mismatch")
     _lib = lib
     return lib

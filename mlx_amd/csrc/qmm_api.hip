@@ -1,8 +1,5 @@
 // qmm_api.hip -- C entry points of quantized_matmul / gather_qmm: argument
 // checks, kernel choice, launch.
-#include <mutex>
-#include <unordered_map>
-
 #include "qmm_args.h"
 
 namespace mlxrocm {
@@ -117,42 +114,38 @@ int check_alignment(const char* who, const QmmArgs& a, int dtype) {
   return MLXROCM_OK;
 }
 
-// Device scratch that outlives a call: one buffer per stream, grown on demand
-// and kept until the process ends.  Work that uses it is ordered by the stream;
-// the mutex is held while that work is enqueued so that two host threads cannot
-// interleave their kernels on one buffer.
-struct StreamScratch {
-  void* ptr = nullptr;
+// Device scratch of one call: the caller's workspace.  In a dry run nothing is
+// launched and `need` receives the bytes the same call would claim, so that
+// mlxrocm_qmm_workspace_size walks exactly the code the call itself walks.
+struct Scratch {
+  char* base = nullptr;
   size_t bytes = 0;
+  bool dry = false;
+  size_t need = 0;
 };
-std::mutex g_scratch_mu;
-std::unordered_map<hipStream_t, StreamScratch> g_scratch;
 
-int stream_scratch(hipStream_t s, size_t bytes, void** out) {
-  StreamScratch& sc = g_scratch[s];
-  if (sc.bytes < bytes) {
-    if (sc.ptr != nullptr) {
-      MLXROCM_HIP_TRY(hipStreamSynchronize(s)); // earlier users are done
-      MLXROCM_HIP_TRY(hipFree(sc.ptr));
-      sc.ptr = nullptr;
-      sc.bytes = 0;
-    }
-    const size_t want = (bytes + (size_t(1) << 21) - 1) >> 21 << 21;
-    hipError_t err = hipMalloc(&sc.ptr, want);
-    if (err != hipSuccess) {
-      (void)hipGetLastError();
-      sc.ptr = nullptr;
-      return fail(
-          err == hipErrorOutOfMemory ? MLXROCM_OUT_OF_MEMORY : MLXROCM_HIP_ERROR,
-          "[qmm] unable to allocate %zu bytes of scratch: %s",
-          want,
-          hipGetErrorString(err));
-    }
-    sc.bytes = want;
+constexpr size_t kScratchAlign = 256;
+
+int claim(Scratch& sc, size_t bytes, void** out) {
+  *out = nullptr;
+  if (sc.dry) {
+    sc.need = bytes;
+    return MLXROCM_OK;
   }
-  *out = sc.ptr;
+  if (sc.base == nullptr || sc.bytes < bytes) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[quantized_matmul] this shape needs a workspace of %zu bytes "
+        "(mlxrocm_qmm_workspace_size); got %zu",
+        bytes,
+        sc.base == nullptr ? size_t(0) : sc.bytes);
+  }
+  *out = sc.base;
   return MLXROCM_OK;
 }
+
+// Launch unless this is a dry run.
+#define MLXROCM_LAUNCH(sc, call) ((sc).dry ? static_cast<int>(MLXROCM_OK) : (call))
 
 // Rows of x from which the prefill paths transpose scales and biases first (see
 // run_qmm_t_transposed_sb).
@@ -163,7 +156,7 @@ constexpr int kTransposeSbMinM = 512;
 // block runs on the bf16 matrix path with fp32 scales, biases and output.
 constexpr size_t kSplitScratchBytes = size_t(256) << 20;
 
-int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
+int run_split_fp32(const QmmArgs& a, int gs, int bits, Scratch& sc, hipStream_t s) {
   const size_t row_bytes = split_x_bytes(1, a.K);
   int rows_per_block = static_cast<int>(kSplitScratchBytes / row_bytes / 256 * 256);
   if (rows_per_block < 256) {
@@ -174,7 +167,7 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
   }
   // the kernel addresses x with 32-bit element offsets
   if (static_cast<uint64_t>(rows_per_block) * 3u * static_cast<uint64_t>(a.K) >= (uint64_t(1) << 32)) {
-    return launch_qmm_naive(a, gs, bits, MLXROCM_FLOAT32, true, s);
+    return MLXROCM_LAUNCH(sc, launch_qmm_naive(a, gs, bits, MLXROCM_FLOAT32, true, s));
   }
   // few tiles: also cut K (one row block, one batch entry only)
   int k_splits = 1;
@@ -190,14 +183,13 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
   const int sb_batches = a.sb_batch_stride == 0 ? 1 : a.L;
   const bool sb_t = a.M >= kTransposeSbMinM;
   const size_t sb_bytes = sb_t ? qmm_n_sb_bytes(a.N, G, sb_batches, MLXROCM_FLOAT32) : 0;
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  void* scratch = nullptr;
-  int rc = stream_scratch(s, x_bytes + partial_bytes + sb_bytes, &scratch);
-  if (rc != MLXROCM_OK) {
+  void* region = nullptr;
+  int rc = claim(sc, x_bytes + partial_bytes + sb_bytes, &region);
+  if (rc != MLXROCM_OK || sc.dry) {
     return rc;
   }
-  void* partial = static_cast<char*>(scratch) + x_bytes;
-  float* sb_image = reinterpret_cast<float*>(static_cast<char*>(scratch) + x_bytes + partial_bytes);
+  void* partial = static_cast<char*>(region) + x_bytes;
+  float* sb_image = reinterpret_cast<float*>(static_cast<char*>(region) + x_bytes + partial_bytes);
   const size_t image = static_cast<size_t>(a.N) * G;
   if (sb_t) {
     rc = transpose_sb_for_qmm_n(
@@ -211,12 +203,12 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
       const int rows = (a.M - m_begin < rows_per_block) ? a.M - m_begin : rows_per_block;
       const float* x = static_cast<const float*>(a.x) + l * a.x_batch_stride +
           static_cast<int64_t>(m_begin) * a.K;
-      rc = split_x_for_mfma(x, scratch, static_cast<size_t>(rows), a.K, s);
+      rc = split_x_for_mfma(x, region, static_cast<size_t>(rows), a.K, s);
       if (rc != MLXROCM_OK) {
         return rc;
       }
       QmmArgs part = a;
-      part.x = scratch;
+      part.x = region;
       part.M = rows;
       part.L = 1;
       part.x_batch_stride = static_cast<int64_t>(rows) * 3 * a.K;
@@ -249,58 +241,57 @@ int run_split_fp32(const QmmArgs& a, int gs, int bits, hipStream_t s) {
 }
 
 // 16-bit prefill whose tiles would leave most compute units idle: K is cut into
-// ranges, the fp32 partial tiles go to scratch and are added up.
-int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
+// ranges, the fp32 partial tiles go to the workspace and are added up.
+int run_k_split(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, Scratch& sc, hipStream_t s) {
   const size_t plane = static_cast<size_t>(a.M) * a.N;
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  void* scratch = nullptr;
-  int rc = stream_scratch(s, plane * k_splits * sizeof(float), &scratch);
-  if (rc != MLXROCM_OK) {
+  void* region = nullptr;
+  int rc = claim(sc, plane * k_splits * sizeof(float), &region);
+  if (rc != MLXROCM_OK || sc.dry) {
     return rc;
   }
   QmmArgs part = a;
-  part.out = scratch;
+  part.out = region;
   rc = launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
-  return reduce_k_splits(scratch, a.out, plane, k_splits, dtype, s);
+  return reduce_k_splits(region, a.out, plane, k_splits, dtype, s);
 }
 
 // Prefill (transpose=true, 16-bit types) from 512 rows of x on: the tile kernel
 // reads one scale and one bias per thread and K-step, and with the caller's
 // [N][K / group] layout every lane of such a load touches a line of its own
 // (measured: 15 % of the kernel's time).  A pre-pass transposes both arrays to
-// [K / group][N] in the stream's scratch buffer (a few MB, ~5 us), after which
+// [K / group][N] in the workspace (a few MB, ~5 us), after which
 // a wavefront's 32 rows read 64 contiguous bytes.
-int run_qmm_t_transposed_sb(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
+int run_qmm_t_transposed_sb(
+    const QmmArgs& a, int gs, int bits, int dtype, int k_splits, Scratch& sc, hipStream_t s) {
   const int G = a.K / gs;
   const int batches = a.sb_batch_stride == 0 ? 1 : a.L;
   const size_t sb_bytes = (qmm_n_sb_bytes(a.N, G, batches, dtype) + 255) / 256 * 256;
   const size_t plane = static_cast<size_t>(a.M) * a.N;
   const size_t partial_bytes = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  void* scratch = nullptr;
-  int rc = stream_scratch(s, sb_bytes + partial_bytes, &scratch);
-  if (rc != MLXROCM_OK) {
+  void* region = nullptr;
+  int rc = claim(sc, sb_bytes + partial_bytes, &region);
+  if (rc != MLXROCM_OK || sc.dry) {
     return rc;
   }
   // rows of the source are the N rows of W, columns its G groups
   rc = transpose_sb_for_qmm_n(
-      a.scales, a.biases, scratch, a.N, G, batches, a.sb_batch_stride, dtype, s);
+      a.scales, a.biases, region, a.N, G, batches, a.sb_batch_stride, dtype, s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
   const size_t image = static_cast<size_t>(a.N) * G;
   QmmArgs part = a;
-  part.scales = scratch;
-  part.biases = static_cast<char*>(scratch) + image * dtype_size(dtype);
+  part.scales = region;
+  part.biases = static_cast<char*>(region) + image * dtype_size(dtype);
   part.sb_batch_stride = batches == 1 ? 0 : static_cast<int64_t>(2 * image);
   part.sb_transposed = 1;
   if (k_splits <= 1) {
     return launch_qmm_mfma(part, gs, bits, dtype, s);
   }
-  void* partial = static_cast<char*>(scratch) + sb_bytes;
+  void* partial = static_cast<char*>(region) + sb_bytes;
   part.out = partial;
   rc = launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s);
   if (rc != MLXROCM_OK) {
@@ -311,31 +302,30 @@ int run_qmm_t_transposed_sb(const QmmArgs& a, int gs, int bits, int dtype, int k
 
 // transpose=false on the matrix cores.  The column loader wants the four
 // scales of four consecutive rows of W side by side, so scales and biases are
-// first transposed to [group][k] in the stream's scratch buffer (a few MB, a
+// first transposed to [group][k] in the workspace (a few MB, a
 // few microseconds); few-row shapes also cut K and keep their fp32 partial
 // planes there.
 // transpose=false, 1..4 rows of x: the streaming kernel, its K ranges added up
-// from fp32 planes in the stream's scratch buffer.
-int run_qmv_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+// from fp32 planes in the workspace.
+int run_qmv_n(const QmmArgs& a, int gs, int bits, int dtype, Scratch& sc, hipStream_t s) {
   const QmvNPlan pl = qmv_n_plan(a, bits);
   if (pl.splits <= 1) {
-    return launch_qmv_n(a, gs, bits, dtype, nullptr, s);
+    return MLXROCM_LAUNCH(sc, launch_qmv_n(a, gs, bits, dtype, nullptr, s));
   }
   const size_t plane = static_cast<size_t>(a.L) * a.M * a.N;
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  void* scratch = nullptr;
-  int rc = stream_scratch(s, plane * pl.splits * sizeof(float), &scratch);
+  void* region = nullptr;
+  int rc = claim(sc, plane * pl.splits * sizeof(float), &region);
+  if (rc != MLXROCM_OK || sc.dry) {
+    return rc;
+  }
+  rc = launch_qmv_n(a, gs, bits, dtype, static_cast<float*>(region), s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
-  rc = launch_qmv_n(a, gs, bits, dtype, static_cast<float*>(scratch), s);
-  if (rc != MLXROCM_OK) {
-    return rc;
-  }
-  return reduce_planes(static_cast<const float*>(scratch), a.out, plane, pl.splits, dtype, s);
+  return reduce_planes(static_cast<const float*>(region), a.out, plane, pl.splits, dtype, s);
 }
 
-int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, Scratch& sc, hipStream_t s) {
   const int G = a.N / gs;
   const int batches = a.sb_batch_stride == 0 ? 1 : a.L;
   int k_splits = 1;
@@ -345,26 +335,25 @@ int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
   const size_t sb_bytes = (qmm_n_sb_bytes(a.K, G, batches, dtype) + 255) / 256 * 256;
   const size_t plane = static_cast<size_t>(a.M) * a.N;
   const size_t partial_bytes = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  void* scratch = nullptr;
-  int rc = stream_scratch(s, sb_bytes + partial_bytes, &scratch);
-  if (rc != MLXROCM_OK) {
+  void* region = nullptr;
+  int rc = claim(sc, sb_bytes + partial_bytes, &region);
+  if (rc != MLXROCM_OK || sc.dry) {
     return rc;
   }
   rc = transpose_sb_for_qmm_n(
-      a.scales, a.biases, scratch, a.K, G, batches, a.sb_batch_stride, dtype, s);
+      a.scales, a.biases, region, a.K, G, batches, a.sb_batch_stride, dtype, s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
   const size_t image = static_cast<size_t>(a.K) * G; // elements of one [G][K] image
   QmmArgs part = a;
-  part.scales = scratch;
-  part.biases = static_cast<char*>(scratch) + image * dtype_size(dtype);
+  part.scales = region;
+  part.biases = static_cast<char*>(region) + image * dtype_size(dtype);
   part.sb_batch_stride = batches == 1 ? 0 : static_cast<int64_t>(2 * image);
   if (k_splits <= 1) {
     return launch_qmm_mfma_n(part, gs, bits, dtype, 1, s);
   }
-  void* partial = static_cast<char*>(scratch) + sb_bytes;
+  void* partial = static_cast<char*>(region) + sb_bytes;
   part.out = partial;
   rc = launch_qmm_mfma_n(part, gs, bits, dtype, k_splits, s);
   if (rc != MLXROCM_OK) {
@@ -373,11 +362,11 @@ int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
   return reduce_k_splits(partial, a.out, plane, k_splits, dtype, s);
 }
 
-int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream_t s) {
+int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& sc, hipStream_t s) {
   // w [K, N] with a few rows of x: the streaming kernel (the tile kernel
   // needs 60-70 us for one row of a 4096 x 14336 weight)
   if (!transpose && qmv_n_supported(a, gs, bits, dtype)) {
-    return run_qmv_n(a, gs, bits, dtype, s);
+    return run_qmv_n(a, gs, bits, dtype, sc, s);
   }
   // A few rows of x, beyond what the row-streaming GEMV keeps in registers.
   // Measured on gate/up and down projection shapes (4- and 8-bit):
@@ -411,7 +400,7 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
     const bool use = (a.M >= 2 && a.M <= 4) ||
         (a.M == 1 && (long_k || !qmv_stream_supported(a, gs, bits, dtype))) || many_rows;
     if (use) {
-      return launch_qmv_quad(a, gs, bits, dtype, s);
+      return MLXROCM_LAUNCH(sc, launch_qmv_quad(a, gs, bits, dtype, s));
     }
   }
   // (two rows of 8-bit codes over a long K: the streaming kernel's dot products
@@ -426,6 +415,9 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
     QmmArgs part = a;
     part.M = 16;
     if (qmv_wide_supported(part, gs, bits, dtype, transpose)) {
+      if (sc.dry) {
+        return MLXROCM_OK;
+      }
       int rc = launch_qmv_wide(part, gs, bits, dtype, s);
       if (rc != MLXROCM_OK) {
         return rc;
@@ -447,19 +439,19 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
   // one row at a width the row-streaming GEMV does not cover (2/3/5/6 bits): the
   // fp32-arithmetic streaming kernel
   if (transpose && a.M == 1 && few_rows && qmv_f32_supported(a, gs, bits, dtype)) {
-    return launch_qmv_f32(a, gs, bits, dtype, s);
+    return MLXROCM_LAUNCH(sc, launch_qmv_f32(a, gs, bits, dtype, s));
   }
   if (few_rows && !staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
     const bool gemv_better = a.M <= 8 && a.K <= 8192 && qmv_mfma_supported(a, gs, bits, dtype);
     if (!gemv_better) {
-      return launch_qmv_wide(a, gs, bits, dtype, s);
+      return MLXROCM_LAUNCH(sc, launch_qmv_wide(a, gs, bits, dtype, s));
     }
   }
   if (staged && qmm_skinny_supported(a, gs, bits, dtype, transpose)) {
-    return launch_qmm_skinny(a, gs, bits, dtype, s);
+    return MLXROCM_LAUNCH(sc, launch_qmm_skinny(a, gs, bits, dtype, s));
   }
   if (staged && a.M <= 16 && qmv_wide_supported(a, gs, bits, dtype, transpose)) {
-    return launch_qmv_wide(a, gs, bits, dtype, s);
+    return MLXROCM_LAUNCH(sc, launch_qmv_wide(a, gs, bits, dtype, s));
   }
   switch (choose_family(a.M, a.N, a.K, a.L, bits, dtype, transpose)) {
     case Family::QmmT:
@@ -469,35 +461,35 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, hipStream
           k_splits = qmm_mfma_k_splits(a.M, a.N, a.K, a.L);
         }
         if (a.lhs_indices == nullptr && a.M >= kTransposeSbMinM) {
-          return run_qmm_t_transposed_sb(a, gs, bits, dtype, k_splits, s);
+          return run_qmm_t_transposed_sb(a, gs, bits, dtype, k_splits, sc, s);
         }
         if (k_splits > 1) {
-          return run_k_split(a, gs, bits, dtype, k_splits, s);
+          return run_k_split(a, gs, bits, dtype, k_splits, sc, s);
         }
-        return launch_qmm_mfma(a, gs, bits, dtype, s);
+        return MLXROCM_LAUNCH(sc, launch_qmm_mfma(a, gs, bits, dtype, s));
       }
       if (dtype == MLXROCM_FLOAT32 && a.lhs_indices == nullptr) {
-        return run_split_fp32(a, gs, bits, s);
+        return run_split_fp32(a, gs, bits, sc, s);
       }
-      return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
+      return MLXROCM_LAUNCH(sc, launch_qmm_naive(a, gs, bits, dtype, transpose, s));
     case Family::Qmv:
       if (qmv_stream_supported(a, gs, bits, dtype)) {
-        return launch_qmv_stream(a, gs, bits, dtype, s);
+        return MLXROCM_LAUNCH(sc, launch_qmv_stream(a, gs, bits, dtype, s));
       }
       if (qmv_mfma_supported(a, gs, bits, dtype)) {
-        return launch_qmv_mfma(a, gs, bits, dtype, s);
+        return MLXROCM_LAUNCH(sc, launch_qmv_mfma(a, gs, bits, dtype, s));
       }
       if (qmv_f32_supported(a, gs, bits, dtype)) {
-        return launch_qmv_f32(a, gs, bits, dtype, s);
+        return MLXROCM_LAUNCH(sc, launch_qmv_f32(a, gs, bits, dtype, s));
       }
-      return launch_qmv_generic(a, gs, bits, dtype, s);
+      return MLXROCM_LAUNCH(sc, launch_qmv_generic(a, gs, bits, dtype, s));
     case Family::QmmN:
       if (a.lhs_indices == nullptr && qmm_mfma_supported(a, gs, bits, dtype, transpose)) {
-        return run_qmm_n(a, gs, bits, dtype, s);
+        return run_qmm_n(a, gs, bits, dtype, sc, s);
       }
-      return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
+      return MLXROCM_LAUNCH(sc, launch_qmm_naive(a, gs, bits, dtype, transpose, s));
     case Family::QmmNaive:
-      return launch_qmm_naive(a, gs, bits, dtype, transpose, s);
+      return MLXROCM_LAUNCH(sc, launch_qmm_naive(a, gs, bits, dtype, transpose, s));
   }
   return fail(MLXROCM_UNSUPPORTED, "no kernel");
 }
@@ -622,7 +614,8 @@ extern "C" int mlxrocm_qmm_swiglu(
       return launch_qmv_stream_glu(one, group_size, bits, dtype, s);
     }
   }
-  rc = run(a, group_size, bits, dtype, true, s);
+  Scratch none; // decode shapes with transpose != 0 claim no scratch
+  rc = run(a, group_size, bits, dtype, true, none, s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
@@ -638,7 +631,10 @@ extern "C" int mlxrocm_qmm_swiglu(
   return rc;
 }
 
-extern "C" int mlxrocm_qmm(
+namespace {
+
+// Body of mlxrocm_qmm and, as a dry run, of mlxrocm_qmm_workspace_size.
+int qmm_entry(
     const void* x,
     const uint32_t* wq,
     const void* scales,
@@ -655,7 +651,8 @@ extern "C" int mlxrocm_qmm(
     int bits,
     int dtype,
     int transpose,
-    mlxrocm_stream_t stream) {
+    Scratch& sc,
+    hipStream_t s) {
   int rc = check_shape(
       "quantized_matmul", M, N, K, L, group_size, bits, dtype, transpose);
   if (rc != MLXROCM_OK) {
@@ -664,14 +661,9 @@ extern "C" int mlxrocm_qmm(
   if (static_cast<int64_t>(M) * N * L == 0) {
     return MLXROCM_OK; // empty output
   }
-  hipStream_t s = static_cast<hipStream_t>(stream);
   if (K == 0) {
-    return launch_zero_fill(
-        out, static_cast<size_t>(M) * N * L * dtype_size(dtype), s);
-  }
-  if (!x || !wq || !scales || !biases || !out) {
-    return fail(
-        MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] null device pointer");
+    return MLXROCM_LAUNCH(
+        sc, launch_zero_fill(out, static_cast<size_t>(M) * N * L * dtype_size(dtype), s));
   }
   if (x_batch_stride < 0 || w_batch_stride < 0 || sb_batch_stride < 0) {
     return fail(MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] negative stride");
@@ -693,11 +685,77 @@ extern "C" int mlxrocm_qmm(
   a.rhs_indices = nullptr;
   a.x_batches = L;
   a.n_experts = L;
-  rc = check_alignment("quantized_matmul", a, dtype);
-  if (rc != MLXROCM_OK) {
-    return rc;
+  if (!sc.dry) {
+    if (!x || !wq || !scales || !biases || !out) {
+      return fail(
+          MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] null device pointer");
+    }
+    rc = check_alignment("quantized_matmul", a, dtype);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    if (sc.base != nullptr && (reinterpret_cast<uintptr_t>(sc.base) % kScratchAlign) != 0) {
+      return fail(
+          MLXROCM_INVALID_ARGUMENT,
+          "[quantized_matmul] the workspace must be %zu-byte aligned",
+          kScratchAlign);
+    }
   }
-  return run(a, group_size, bits, dtype, transpose != 0, s);
+  return run(a, group_size, bits, dtype, transpose != 0, sc, s);
+}
+
+} // namespace
+
+extern "C" size_t mlxrocm_qmm_workspace_size(
+    int M,
+    int N,
+    int K,
+    int L,
+    int batched_weights,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose) {
+  Scratch sc;
+  sc.dry = true;
+  // the strides only say "one weight for every batch entry" or "one each"
+  const int64_t w_stride = batched_weights ? 4096 : 0;
+  const int64_t x_stride = static_cast<int64_t>(M) * K;
+  if (qmm_entry(
+          nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, L, x_stride, w_stride,
+          w_stride, group_size, bits, dtype, transpose, sc, nullptr) != MLXROCM_OK) {
+    return 0;
+  }
+  return sc.need;
+}
+
+extern "C" int mlxrocm_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t sb_batch_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream) {
+  Scratch sc;
+  sc.base = static_cast<char*>(workspace);
+  sc.bytes = workspace != nullptr ? workspace_bytes : 0;
+  return qmm_entry(
+      x, wq, scales, biases, out, M, N, K, L, x_batch_stride, w_batch_stride,
+      sb_batch_stride, group_size, bits, dtype, transpose, sc,
+      static_cast<hipStream_t>(stream));
 }
 
 // Grouping by expert pays when every expert's weights are shared by several
@@ -841,7 +899,8 @@ extern "C" int mlxrocm_gather_qmm(
     part.rhs_indices = rhs_indices + first;
     part.out = static_cast<char*>(out) +
         static_cast<size_t>(first) * M * N * dtype_size(dtype);
-    rc = run(part, group_size, bits, dtype, transpose != 0, s);
+    Scratch none; // no launch with index arrays claims scratch
+    rc = run(part, group_size, bits, dtype, transpose != 0, none, s);
     if (rc != MLXROCM_OK) {
       return rc;
     }

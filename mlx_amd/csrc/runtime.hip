@@ -7,8 +7,11 @@
 // memory.  Freed buffers are kept in a size-bucketed cache (the size classes of
 // mlx/backend/cuda/allocator.cpp:22-29: tiny -> 8 B, small -> next power of two,
 // large -> whole 16 KiB pages) and handed back on the next request of the same
-// class; the cache is trimmed, oldest first, above the cache limit and emptied
-// when hipMalloc runs out of memory.
+// class; the cache is trimmed, least recently freed buffer first, above the cache
+// limit, when active + cached + requested bytes would pass the memory limit
+// (95 % of the device's memory unless set; the relief valve of
+// mlx/backend/cuda/allocator.cpp:186-191), and emptied when hipMalloc runs out of
+// memory.  A request larger than the device's memory fails without reaching HIP.
 #include <map>
 #include <mutex>
 #include <unordered_map>
@@ -52,14 +55,31 @@ class DeviceAllocator {
     // not waste more than half of itself.
     auto it = cache_.lower_bound(cls);
     if (it != cache_.end() && it->first <= cls * 2) {
-      void* p = it->second;
+      void* p = it->second.ptr;
       const size_t got = it->first;
+      lru_.erase(it->second.seq);
       cache_.erase(it);
       cached_bytes_ -= got;
       live_[p] = got;
       note_active(got);
       *out = p;
       return MLXROCM_OK;
+    }
+    ask_device();
+    if (cls < size || cls > total_memory_) {
+      return fail(
+          MLXROCM_OUT_OF_MEMORY,
+          "[malloc] unable to allocate %zu bytes: the device holds %zu",
+          size,
+          total_memory_);
+    }
+    // memory pressure: give cached buffers back before asking for more
+    if (cached_bytes_ > 0) {
+      const size_t want = active_bytes_ + cached_bytes_ + cls;
+      if (want > memory_limit_) {
+        const size_t over = want - memory_limit_;
+        release_cache(over >= cached_bytes_ ? 0 : cached_bytes_ - over);
+      }
     }
     void* p = nullptr;
     hipError_t err = hipMalloc(&p, cls);
@@ -95,7 +115,8 @@ class DeviceAllocator {
     const size_t sz = it->second;
     live_.erase(it);
     active_bytes_ -= sz;
-    cache_.emplace(sz, p);
+    const uint64_t seq = next_seq_++;
+    lru_[seq] = cache_.emplace(sz, Cached{p, seq});
     cached_bytes_ += sz;
     if (cached_bytes_ > cache_limit_) {
       release_cache(cache_limit_);
@@ -136,12 +157,14 @@ class DeviceAllocator {
   }
   size_t set_memory_limit(size_t limit) {
     std::lock_guard<std::mutex> lock(mu_);
+    ask_device();
     const size_t prev = memory_limit_;
     memory_limit_ = limit;
     return prev;
   }
   size_t memory_limit() {
     std::lock_guard<std::mutex> lock(mu_);
+    ask_device();
     return memory_limit_;
   }
   void clear_cache() {
@@ -150,6 +173,23 @@ class DeviceAllocator {
   }
 
  private:
+  // The device's memory size and, unless a limit has been set, the default
+  // limit derived from it; asked once, on first use.
+  void ask_device() {
+    if (total_memory_ != 0) {
+      return;
+    }
+    size_t free_now = 0;
+    if (hipMemGetInfo(&free_now, &total_memory_) != hipSuccess || total_memory_ == 0) {
+      (void)hipGetLastError();
+      total_memory_ = static_cast<size_t>(-1);
+      return;
+    }
+    if (memory_limit_ == static_cast<size_t>(-1)) {
+      memory_limit_ = total_memory_ / 100 * 95;
+    }
+  }
+
   void note_active(size_t sz) {
     active_bytes_ += sz;
     if (active_bytes_ > peak_bytes_) {
@@ -157,19 +197,31 @@ class DeviceAllocator {
     }
   }
 
-  // Frees cached buffers, largest first, until at most `target` bytes remain.
+  // Frees cached buffers, least recently freed first, until at most `target`
+  // bytes remain.
   void release_cache(size_t target) {
-    while (cached_bytes_ > target && !cache_.empty()) {
-      auto it = std::prev(cache_.end());
-      (void)hipFree(it->second);
+    while (cached_bytes_ > target && !lru_.empty()) {
+      auto oldest = lru_.begin();
+      auto it = oldest->second;
+      (void)hipFree(it->second.ptr);
       cached_bytes_ -= it->first;
       cache_.erase(it);
+      lru_.erase(oldest);
     }
   }
 
+  struct Cached {
+    void* ptr;
+    uint64_t seq;
+  };
+  using Cache = std::multimap<size_t, Cached>;
+
   std::mutex mu_;
   std::unordered_map<void*, size_t> live_;
-  std::multimap<size_t, void*> cache_;
+  Cache cache_; // by size class
+  std::map<uint64_t, Cache::iterator> lru_; // by time of the free
+  uint64_t next_seq_ = 0;
+  size_t total_memory_ = 0; // 0: not asked yet
   size_t active_bytes_ = 0;
   size_t peak_bytes_ = 0;
   size_t cached_bytes_ = 0;

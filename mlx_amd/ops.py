@@ -364,15 +364,27 @@ def quantized_matmul(
         L *= d
     xb = x.reshape(1, M, K) if x.dim() <= 2 else x.expand(*batch_shape, M, K)
     xb = xb.contiguous()
+    if w.dim() == 2 and L > 1:
+        # one weight matrix for every batch entry: the batch folds into the rows
+        # of x, so W is read once for all of them (the GPU backends do the same,
+        # metal/quantized.cpp:1799-1801, cuda/quantized/qmm/qmm.cu:143-146)
+        M, L = M * L, 1
     wb, w_stride = _dense_batches(w, batch_shape)
     sb, sb_stride = _dense_batches(scales, batch_shape)
     bb, _ = _dense_batches(biases, batch_shape)
     out = torch.empty(out_shape, dtype=dtype, device=x.device)
+    code = _DTYPE_CODE[dtype]
+    ws_bytes = lib.mlxrocm_qmm_workspace_size(
+        M, w_outer, K, L, int(w_stride != 0), group_size, bits, code, int(bool(transpose))
+    )
+    # a temporary of the call, like the ones eval_gpu hands to add_temporary
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     _lib.check(
         lib.mlxrocm_qmm(
             xb.data_ptr(), wb.data_ptr(), sb.data_ptr(), bb.data_ptr(), out.data_ptr(),
             M, w_outer, K, L, M * K, w_stride, sb_stride, group_size, bits,
-            _DTYPE_CODE[dtype], int(bool(transpose)), _stream_ptr(x),
+            code, int(bool(transpose)),
+            ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x),
         )
     )
     return out

@@ -116,13 +116,31 @@ void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
   out.set_data(allocator::malloc(out.nbytes()));
 
   const int K = x.shape(-1);
-  const int M = x.ndim() > 1 ? x.shape(-2) : 1;
+  int M = x.ndim() > 1 ? x.shape(-2) : 1;
   const int N = out.shape(-1);
-  const int L = (M == 0 || K == 0) ? 0 : static_cast<int>(x.size() / (size_t(K) * M));
+  int L = (M == 0 || K == 0) ? 0 : static_cast<int>(x.size() / (size_t(K) * M));
   // w.ndim() == 2: one weight for every batch (mlx/backend/cpu/quantized.cpp:396-397)
   const int64_t w_stride = w.ndim() > 2 ? int64_t(w.shape(-1)) * w.shape(-2) : 0;
   const int64_t sb_stride =
       w.ndim() > 2 ? int64_t(scales.shape(-1)) * scales.shape(-2) : 0;
+  if (w.ndim() == 2 && L > 1) {
+    // x is row-contiguous here, so the batch folds into its rows and the weight
+    // is read once for all of them (mlx/backend/metal/quantized.cpp:1799-1801)
+    M *= L;
+    L = 1;
+  }
+  const int dt = dtype_code(x.dtype(), "quantized_matmul");
+
+  // device scratch of the call: a temporary like any other
+  const size_t ws_bytes = mlxrocm_qmm_workspace_size(
+      M, N, K, L, w.ndim() > 2, group_size_, bits_, dt, transpose_ ? 1 : 0);
+  void* ws_ptr = nullptr;
+  if (ws_bytes > 0) {
+    array ws({static_cast<int>(ws_bytes)}, uint8, nullptr, {});
+    ws.set_data(allocator::malloc(ws_bytes));
+    enc.add_temporary(ws);
+    ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
+  }
 
   rocm::check(mlxrocm_qmm(
       rocm::gpu_ptr<void>(x, enc.stream()),
@@ -139,8 +157,10 @@ void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
       sb_stride,
       group_size_,
       bits_,
-      dtype_code(x.dtype(), "quantized_matmul"),
+      dt,
       transpose_ ? 1 : 0,
+      ws_ptr,
+      ws_bytes,
       enc.stream()));
 }
 

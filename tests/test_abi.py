@@ -35,7 +35,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 
 def test_abi_version(lib):
-    assert lib.mlxrocm_abi_version() == 1
+    assert lib.mlxrocm_abi_version() == 2
 
 
 def test_invalid_arguments_are_reported_not_thrown(lib):
@@ -51,15 +51,15 @@ def test_invalid_arguments_are_reported_not_thrown(lib):
     rc = lib.mlxrocm_affine_dequantize(one, one, one, one, 64, 64, 4, 9, None)
     assert rc == _lib.INVALID_ARGUMENT and b"dtype" in lib.mlxrocm_last_error()
     # quantized axis not a multiple of the group size
-    rc = lib.mlxrocm_qmm(one, one, one, one, one, 1, 32, 96, 1, 96, 0, 0, 64, 4, 0, 1, None)
+    rc = lib.mlxrocm_qmm(one, one, one, one, one, 1, 32, 96, 1, 96, 0, 0, 64, 4, 0, 1, None, 0, None)
     assert rc == _lib.INVALID_ARGUMENT
-    rc = lib.mlxrocm_qmm(None, one, one, one, one, 1, 32, 128, 1, 128, 0, 0, 64, 4, 0, 1, None)
+    rc = lib.mlxrocm_qmm(None, one, one, one, one, 1, 32, 128, 1, 128, 0, 0, 64, 4, 0, 1, None, 0, None)
     assert rc == _lib.INVALID_ARGUMENT and b"null" in lib.mlxrocm_last_error()
     with pytest.raises(ValueError):
         _lib.check(rc)
     # empty problems succeed without touching the device
     assert lib.mlxrocm_affine_quantize(None, None, None, None, 0, 64, 4, 0, None) == 0
-    assert lib.mlxrocm_qmm(None, None, None, None, None, 0, 32, 128, 1, 0, 0, 0, 64, 4, 0, 1, None) == 0
+    assert lib.mlxrocm_qmm(None, None, None, None, None, 0, 32, 128, 1, 0, 0, 0, 64, 4, 0, 1, None, 0, None) == 0
 
 
 def test_kernel_choice(lib):

@@ -4,8 +4,8 @@ import torch
 
 import mlx_amd
 from tests.util import (
-    activations, exact_affine_weights, exact_tolerance, matmul_tolerance,
-    normal_weights,
+    activations, exact_affine_weights, exact_affine_weights_on, exact_tolerance,
+    exact_tolerance_from, matmul_tolerance, normal_weights,
 )
 
 pytestmark = pytest.mark.gpu
@@ -259,3 +259,69 @@ def test_gather_qmm_small_groups(oracle, gpu, bits, gs):
     tol = matmul_tolerance(dtype, K, x, w_hat) + float(
         (ref.reshape(T, N).double() - exact).abs().max())
     assert float((got.double() - ref.double()).abs().max()) <= tol
+
+
+@pytest.fixture(scope="module")
+def mixtral_stack(gpu):
+    """8 experts of [14336, 4096], N(0, 0.02), 4-bit group 64, bf16 scales and
+    biases, quantized on the GPU (that operator is bit-pinned by its own tests),
+    with the fp64 affine weights of every expert beside it."""
+    E, N, K = 8, 14336, 4096
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn((E, N, K), generator=g) * 0.02).to(torch.bfloat16)
+    wq, s, b = mlx_amd.quantize(w.to(gpu), 64, 4)
+    del w
+    w_hat = exact_affine_weights_on(gpu, wq, s, b, 64, 4)
+    yield wq, s, b, w_hat
+    del w_hat
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("T", (1, 64))
+def test_gather_qmm_full_size_moe_few_tokens(oracle, gpu, mixtral_stack, T):
+    """The expert-routed decode shapes at full size: T tokens, top-2 of 8 experts
+    drawn uniformly (seeded), unsorted and pre-sorted by expert.  Every index
+    pair against the fp64 product; a subsample of the pairs against the CPU
+    oracle; sorted and unsorted runs agree bit for bit after un-permuting."""
+    wq, s, b, w_hat = mixtral_stack
+    E, N, K = 8, 14336, 4096
+    x = activations((T, 1, 1, K), torch.bfloat16, seed=T)
+    idx = torch.randint(0, E, (T, 2), generator=torch.Generator().manual_seed(T))
+    gx, gidx = x.to(gpu), idx.to(gpu)
+    unsorted = mlx_amd.gather_qmm(gx, wq, s, b, rhs_indices=gidx, transpose=True,
+                                  group_size=64, bits=4)
+    assert unsorted.shape == (T, 2, 1, N)
+    flat = gidx.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    xs = gx.reshape(T, 1, K)[order // 2].contiguous()
+    ys = mlx_amd.gather_qmm(xs, wq, s, b, rhs_indices=flat[order].contiguous(),
+                            transpose=True, group_size=64, bits=4, sorted_indices=True)
+    torch.cuda.synchronize()
+    assert ys.shape == (2 * T, 1, N)
+    resorted = ys[torch.argsort(order)].reshape(T, 2, 1, N)
+    assert torch.equal(unsorted.view(torch.int16), resorted.view(torch.int16))
+    # every pair against fp64, expert by expert
+    got = unsorted.reshape(2 * T, N).double()
+    xd = gx.reshape(T, K).double()
+    tok = torch.arange(2 * T, device=gpu) // 2
+    x_absmax = float(x.abs().max())
+    for e in range(E):
+        pairs = torch.nonzero(flat == e).reshape(-1)
+        if pairs.numel() == 0:
+            continue
+        exact = xd[tok[pairs]] @ w_hat[e].T
+        err = float((got[pairs] - exact).abs().max())
+        tol = exact_tolerance_from(torch.bfloat16, K, x_absmax, float(w_hat[e].abs().max()),
+                                   float(exact.abs().max()))
+        assert err <= tol, f"expert {e}: {err} > {tol}"
+    # the oracle on a few pairs
+    cq = [t.cpu() for t in (wq, s, b)]
+    for p in sorted({0, (2 * T) // 3, 2 * T - 1}):
+        t, j = p // 2, p % 2
+        e = int(idx[t, j])
+        xr = x[t].reshape(1, K)
+        ref = oracle.qmm(xr, cq[0][e], cq[1][e], cq[2][e], True, 64, 4).double()
+        exact = (xr.to(gpu).double() @ w_hat[e].T).cpu()
+        tol = 2e-2 * (K ** 0.5) * x_absmax * float(w_hat[e].abs().max()) + float(
+            (ref - exact).abs().max())
+        assert float((unsorted[t, j].cpu().double() - ref).abs().max()) <= tol
