@@ -186,6 +186,38 @@ int mlxrocm_qmm(
     mlxrocm_stream_t stream);
 
 /*
+ * mlxrocm_qmm without the workspace argument, for callers that cannot
+ * allocate device memory at all (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  The scratch the shapes listed above need comes from a 64 MiB
+ * array inside the library's device image (one copy per GPU, held until the
+ * process ends); a shape that needs more is refused with MLXROCM_UNSUPPORTED.
+ * The first call on a device looks the array's address up (no allocation; do
+ * it once outside a graph capture -- an empty call, M == 0, is enough).  All
+ * calls on one GPU share the array: calls that may overlap in time (different
+ * streams or host threads without an ordering between them) race on it.
+ * Results are those of mlxrocm_qmm bit for bit.
+ */
+int mlxrocm_qmm_static(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t sb_batch_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    mlxrocm_stream_t stream);
+
+/*
  * Gated-MLP decode: out = silu(x @ dequant(w_gate).T) * (x @ dequant(w_up).T),
  * both projections in one launch over the shared x, then one elementwise pass.
  * No single primitive of the reference corresponds to it: it fuses the two

@@ -34,6 +34,10 @@ SIGNATURES = {
         _i,
         [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p, _sz, _p],
     ),
+    "mlxrocm_qmm_static": (
+        _i,
+        [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p],
+    ),
     "mlxrocm_qmm_swiglu_workspace_size": (_sz, [_i, _i, _i]),
     "mlxrocm_qmm_swiglu": (_i, [_p] * 9 + [_i] * 6 + [_p]),
     "mlxrocm_gather_qmm": (

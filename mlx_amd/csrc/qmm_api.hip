@@ -1,5 +1,7 @@
 // qmm_api.hip -- C entry points of quantized_matmul / gather_qmm: argument
 // checks, kernel choice, launch.
+#include <mutex>
+
 #include "qmm_args.h"
 
 namespace mlxrocm {
@@ -752,6 +754,91 @@ extern "C" int mlxrocm_qmm(
   Scratch sc;
   sc.base = static_cast<char*>(workspace);
   sc.bytes = workspace != nullptr ? workspace_bytes : 0;
+  return qmm_entry(
+      x, wq, scales, biases, out, M, N, K, L, x_batch_stride, w_batch_stride,
+      sb_batch_stride, group_size, bits, dtype, transpose, sc,
+      static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------------------
+// The no-allocation variant of mlxrocm_qmm.
+//
+// Device scratch for callers that cannot allocate: one array in the library's
+// device image, so every GPU the library runs on holds its own copy from the
+// moment the code object is loaded until the process ends.  In host code the
+// name below is only a handle for hipGetSymbolAddress; the address a kernel
+// may use is looked up once per device and kept in g_static_scratch.
+constexpr size_t kStaticScratchBytes = size_t(64) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mu;
+void* g_static_scratch[kMaxDevices] = {};
+
+// Address of the current device's copy of `scratch` (first call on a device
+// resolves it; later calls only read the table).
+int static_scratch(void** out) {
+  int dev = 0;
+  MLXROCM_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) {
+    return fail(MLXROCM_UNSUPPORTED, "[quantized_matmul_static] device %d out of range", dev);
+  }
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (g_static_scratch[dev] == nullptr) {
+    void* ptr = nullptr;
+    MLXROCM_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) {
+      return fail(MLXROCM_HIP_ERROR, "[quantized_matmul_static] no address for the scratch array");
+    }
+    g_static_scratch[dev] = ptr;
+  }
+  *out = g_static_scratch[dev];
+  return MLXROCM_OK;
+}
+
+} // namespace
+
+extern "C" int mlxrocm_qmm_static(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t sb_batch_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    mlxrocm_stream_t stream) {
+  void* region = nullptr;
+  int rc = static_scratch(&region);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  const size_t need = mlxrocm_qmm_workspace_size(
+      M, N, K, L, w_batch_stride != 0 || sb_batch_stride != 0, group_size, bits, dtype, transpose);
+  if (need > kStaticScratchBytes) {
+    return fail(
+        MLXROCM_UNSUPPORTED,
+        "[quantized_matmul_static] this shape needs %zu bytes of scratch, the built-in "
+        "buffer holds %zu; use mlxrocm_qmm with a workspace",
+        need,
+        kStaticScratchBytes);
+  }
+  // Nothing the kernels keep in scratch has to start at zero: the transposed
+  // scale / bias image, the split x and every partial plane are written in
+  // full before they are read, so the previous call's contents need no clearing.
+  Scratch sc;
+  sc.base = static_cast<char*>(region);
+  sc.bytes = kStaticScratchBytes;
   return qmm_entry(
       x, wq, scales, biases, out, M, N, K, L, x_batch_stride, w_batch_stride,
       sb_batch_stride, group_size, bits, dtype, transpose, sc,
