@@ -26,16 +26,126 @@
 // [hi | hi | lo] parts (dequantized in fp32, split on the fly), which sums to
 // x_hi w_hi + x_lo w_hi + x_hi w_lo with fp32 accumulation -- a relative error
 // of about 2^-17 per product, inside the fp32 tolerance of the path.
-// LDS rows are 64 elements + 8 of padding (144 bytes), which makes the 16-byte
-// fragment reads of 16 consecutive rows hit 64 distinct banks.  The finished
-// tile is staged through LDS once more so that y is written in full 16-byte,
-// row-contiguous stores.
+// The x tile never passes through registers: global_load_lds_dwordx4 moves 16
+// bytes per lane straight into LDS (a wavefront's 64 pieces land contiguously,
+// eight 128-byte rows), three stages deep, with the pieces of a row XOR-swizzled
+// by the row number so that the 16-byte fragment reads of 16 consecutive rows
+// spread over the banks (an LDS store from registers costs the matrix pipe
+// about 30 clocks of issue on its SIMD; the x tile was half of them).  W rows in
+// LDS are 64 elements + 8 of padding (144 bytes), conflict free for the same
+// reads.  The finished tile is staged through LDS once more so that y is
+// written in full 16-byte, row-contiguous stores.
 #include "mfma_dequant.h"
 #include "qmm_args.h"
 
 namespace mlxrocm {
 
 namespace {
+
+// ---- global loads issued behind the compiler's back --------------------------
+// The K loop keeps loads of three kinds in flight at once: the direct-to-LDS
+// loads of x (needed two barriers later), and the packed W words with their
+// scale and bias (needed after the next barrier).  The compiler would wait for
+// every outstanding direct-to-LDS load before each LDS read (it cannot tell
+// which LDS bytes they write), and any wait it inserted for the W words would
+// also wait for the younger x loads (vmcnt completes in order).  So all loads
+// of the loop are inline assembly, whose results the compiler believes ready at
+// once, and the loop waits for them itself, once per step, right before the
+// barrier: `s_waitcnt vmcnt(4)` leaves exactly that step's four x loads in
+// flight.  Nothing may read a RawWords / raw value between its load and that
+// wait; every slot of the loop ends in a scheduling barrier, so no use moves up.
+typedef uint32_t raw_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t raw_u32x3 __attribute__((ext_vector_type(3)));
+typedef uint32_t raw_u32x4 __attribute__((ext_vector_type(4)));
+
+
+// K dwords (K = 1..4) exactly as one load instruction fills them: the inline
+// assembly writes the tuple itself, so no copy of a half-arrived value exists.
+template <int K>
+struct RawTuple;
+template <>
+struct RawTuple<1> {
+  uint32_t v;
+  __device__ __forceinline__ void load(const uint32_t* p) {
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p));
+  }
+  __device__ __forceinline__ uint32_t get(int) const { return v; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
+};
+template <>
+struct RawTuple<2> {
+  raw_u32x2 v;
+  __device__ __forceinline__ void load(const uint32_t* p) {
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(p));
+  }
+  __device__ __forceinline__ uint32_t get(int j) const { return v[j]; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
+};
+template <>
+struct RawTuple<3> {
+  raw_u32x3 v;
+  __device__ __forceinline__ void load(const uint32_t* p) {
+    asm volatile("global_load_dwordx3 %0, %1, off" : "=v"(v) : "v"(p));
+  }
+  __device__ __forceinline__ uint32_t get(int j) const { return v[j]; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
+};
+template <>
+struct RawTuple<4> {
+  raw_u32x4 v;
+  __device__ __forceinline__ void load(const uint32_t* p) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p));
+  }
+  __device__ __forceinline__ uint32_t get(int j) const { return v[j]; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
+};
+template <>
+struct RawTuple<0> {
+  __device__ __forceinline__ void load(const uint32_t*) {}
+  __device__ __forceinline__ uint32_t get(int) const { return 0; }
+  __device__ __forceinline__ void pin() {}
+};
+
+// N consecutive dwords (N = 1..8) as the one or two register tuples the loads
+// fill.  pin() marks the place from which the values may be read: it goes right
+// behind the wait that covers the loads, and the compiler treats it as the
+// definition of the registers.
+template <int N>
+struct RawWords {
+  static constexpr int kA = N >= 4 ? 4 : N; // dwords of the first load
+  static constexpr int kB = N - kA;         // of the second (0..4)
+  RawTuple<kA> a;
+  RawTuple<kB> b;
+  __device__ __forceinline__ void load(const uint32_t* p) {
+    a.load(p);
+    b.load(p + 4);
+  }
+  __device__ __forceinline__ uint32_t get(int j) const {
+    return j < 4 ? a.get(j) : b.get(j - 4);
+  }
+  __device__ __forceinline__ void pin() {
+    a.pin();
+    b.pin();
+  }
+};
+
+// One scale or bias value as loaded: 16 bits in the low half, or a float.
+template <typename TS>
+__device__ __forceinline__ void raw_load_value(uint32_t& v, const TS* p) {
+  if constexpr (sizeof(TS) == 2) {
+    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p));
+  } else {
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p));
+  }
+}
+template <typename TS>
+__device__ __forceinline__ float raw_value(uint32_t v) {
+  if constexpr (sizeof(TS) == 2) {
+    return to_f32(__builtin_bit_cast(TS, static_cast<uint16_t>(v)));
+  } else {
+    return __uint_as_float(v);
+  }
+}
 
 constexpr int kBM = 256;
 constexpr int kBK = 64;
@@ -96,10 +206,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   constexpr int kBN = 32 * NT;
   constexpr int kNS = 8 * NT; // MFMAs per wavefront per K-step
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  // two stages, each an x tile followed by a W tile
-  constexpr int kXTile = kBM * kLdsStride; // elements
+  // three unpadded x stages (filled by direct-to-LDS loads), then two W stages
+  constexpr int kXTile = kBM * kBK; // elements
+  constexpr int kXStages = 3;
   constexpr int kWTile = kBN * kLdsStride;
-  constexpr int kStage = kXTile + kWTile;
+  constexpr int kWBase = kXStages * kXTile;
   T* lds = reinterpret_cast<T*>(smem);
 
   const int tid = threadIdx.x;
@@ -166,9 +277,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   const int row_words = (WN ? N : K) / 32 * BITS;
 
   // ---- loader roles ----
-  // x: thread covers 16-byte chunk (tid % 8) of rows tid/8 + 64 i, i < 4.
-  const int xc = tid & 7;
-  const int xr = tid >> 3;
+  // x: wavefront w moves rows 32 w + 8 i .. + 7 of the tile with its i-th load
+  // (i < 4); lane l lands in piece l % 8 of row l / 8 and fetches the row's
+  // logical piece (l % 8) ^ (l / 8).
+  const int xr = wave * 32 + (lane >> 3);
+  const int xc = (lane & 7) ^ (lane >> 3);
   // W: thread (wr, wh) covers codes [32 wh, 32 wh + 32) of tile row wr; the
   // threads past the tile's rows repeat its last row (same values, same place).
   const int wr = (tid >> 1) < kBN ? (tid >> 1) : kBN - 1;
@@ -210,7 +323,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   uint32_t xoff0, xoff1, xoff2, xoff3;
   {
     auto row_off = [&](int i) {
-      const int m = m0 + xr + 64 * i;
+      const int m = m0 + xr + 8 * i;
       const int mc = m < M ? m : M - 1;
       if constexpr (GROUPED) {
         const uint32_t pair = static_cast<uint32_t>(a.group_perm[row0 + mc]);
@@ -225,30 +338,38 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     xoff3 = row_off(3);
   }
 
-  // registers of the tiles in flight: x and the packed W of the next K-step,
-  // and the packed W of the step after that (wnext), fetched a whole step ahead
-  // (x: two sets used by alternate steps, each fetched two steps ahead)
-  constexpr int kXSets = 2;
-  uint4 xa0, xa1, xa2, xa3; // set 0
-  uint4 xb0, xb1, xb2, xb3; // set 1
-// named registers, not an array: an array indexed through macros ends up in
-// scratch memory
-#define QMM_XQ(set, i) (*((kXSets == 2 && (set) == 1) ? &xb##i : &xa##i))
-  uint32_t wreg[BITS], wnext[BITS];
-  TS sreg[1], breg[1], snext[1], bnext[1]; // converted when used, so the loads are not waited for early
-  uint2 swn, bwn, swn_next, bwn_next;      // WN: four 16-bit values each, kept raw for the same reason
+  // registers of the tiles in flight: the packed W of the next K-step and of
+  // the step after that (wnext), fetched a whole step ahead
+  uint32_t wreg[BITS];
+  RawWords<WN ? 1 : BITS> wnext;                 // transpose=true: BITS consecutive words
+  RawWords<(WN ? BITS / 4 : 1)> wnext_row[4];    // WN: the words of each of four rows
+  uint32_t sreg, breg, snext, bnext;             // one scale / bias as loaded
+  uint2 swn, bwn;                                // WN: four 16-bit values each
+  RawTuple<2> swn_next, bwn_next;
   auto wn_value = [](const uint2& v, int j) {
     const uint32_t word = j < 2 ? v.x : v.y;
     return to_f32(__builtin_bit_cast(TS, static_cast<
         std::conditional_t<sizeof(TS) == 2, uint16_t, uint32_t>>(word >> (16 * (j & 1)))));
   };
 
-#define QMM_LOAD_X(set, k0)                                                      \
+// x rows 32 w + 8 i .. + 7 of the tile at k0, straight into LDS stage `xs`
+// (element offset of the stage); completion is counted by vmcnt.
+#define QMM_DMA_X1(xs, k0, i, xoff)                                              \
   do {                                                                           \
-    QMM_XQ(set, 0) = *reinterpret_cast<const uint4*>(p.x + xoff0 + (k0));        \
-    QMM_XQ(set, 1) = *reinterpret_cast<const uint4*>(p.x + xoff1 + (k0));        \
-    QMM_XQ(set, 2) = *reinterpret_cast<const uint4*>(p.x + xoff2 + (k0));        \
-    QMM_XQ(set, 3) = *reinterpret_cast<const uint4*>(p.x + xoff3 + (k0));        \
+    const T* g__ = p.x + (xoff) + (k0);                                          \
+    const uint32_t m0__ = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(     \
+        (__attribute__((address_space(3))) char*)(lds + (xs) + (wave * 32 + 8 * (i)) * kBK))); \
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"           \
+                 :                                                               \
+                 : "v"(g__), "s"(m0__)                                           \
+                 : "memory");                                                    \
+  } while (0)
+#define QMM_DMA_X(xs, k0)                                                        \
+  do {                                                                           \
+    QMM_DMA_X1(xs, k0, 0, xoff0);                                                \
+    QMM_DMA_X1(xs, k0, 1, xoff1);                                                \
+    QMM_DMA_X1(xs, k0, 2, xoff2);                                                \
+    QMM_DMA_X1(xs, k0, 3, xoff3);                                                \
   } while (0)
 
 #define QMM_LOAD_W(k0)                                                           \
@@ -256,50 +377,58 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     if constexpr (WN) {                                                          \
       const uint32_t* wp__ = wsrc + static_cast<size_t>(k0) * row_words;         \
       _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
-        _Pragma("unroll") for (int u__ = 0; u__ < kWPR; ++u__) {                 \
-          wnext[j__ * kWPR + u__] = wp__[static_cast<size_t>(j__) * row_words + u__]; \
-        }                                                                        \
+        wnext_row[j__].load(wp__ + static_cast<size_t>(j__) * row_words);        \
       }                                                                          \
-      swn_next = *reinterpret_cast<const uint2*>(ssrc + (k0));                   \
-      bwn_next = *reinterpret_cast<const uint2*>(bsrc + (k0));                   \
+      swn_next.load(reinterpret_cast<const uint32_t*>(ssrc + (k0)));             \
+      bwn_next.load(reinterpret_cast<const uint32_t*>(bsrc + (k0)));             \
     } else {                                                                     \
       /* split mode: blocks 3t, 3t+1, 3t+2 of x all meet block t of W */         \
       const int kw__ = kSplit ? ((k0) / (3 * kBK)) * kBK : (k0);                 \
-      const uint32_t* wp__ = wsrc + (kw__ / 32) * BITS;                          \
-      _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                   \
-        wnext[j__] = wp__[j__];                                                  \
-      }                                                                          \
+      wnext.load(wsrc + (kw__ / 32) * BITS);                                     \
       const size_t g__ = static_cast<size_t>((kw__ + 32 * wh) >> gs_shift) * sb_gstride; \
-      snext[0] = ssrc[g__];                                                      \
-      bnext[0] = bsrc[g__];                                                      \
+      raw_load_value<TS>(snext, ssrc + g__);                                     \
+      raw_load_value<TS>(bnext, bsrc + g__);                                     \
+    }                                                                            \
+  } while (0)
+
+// Behind the wait that covers the loads of QMM_LOAD_W: from here on the loaded
+// registers may be read (QMM_ROTATE_W).
+#define QMM_PIN_W()                                                              \
+  do {                                                                           \
+    if constexpr (WN) {                                                          \
+      _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
+        wnext_row[j__].pin();                                                    \
+      }                                                                          \
+      swn_next.pin();                                                            \
+      bwn_next.pin();                                                            \
+    } else {                                                                     \
+      wnext.pin();                                                               \
+      asm volatile("" : "+v"(snext), "+v"(bnext));                               \
     }                                                                            \
   } while (0)
 
 #define QMM_ROTATE_W()                                                           \
   do {                                                                           \
-    _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                     \
-      wreg[j__] = wnext[j__];                                                    \
-    }                                                                            \
-    sreg[0] = snext[0];                                                          \
-    breg[0] = bnext[0];                                                          \
     if constexpr (WN) {                                                          \
-      swn = swn_next;                                                            \
-      bwn = bwn_next;                                                            \
+      _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
+        _Pragma("unroll") for (int u__ = 0; u__ < kWPR; ++u__) {                 \
+          wreg[j__ * kWPR + u__] = wnext_row[j__].get(u__);                      \
+        }                                                                        \
+      }                                                                          \
+      swn = make_uint2(swn_next.get(0), swn_next.get(1));                        \
+      bwn = make_uint2(bwn_next.get(0), bwn_next.get(1));                        \
+    } else {                                                                     \
+      _Pragma("unroll") for (int j__ = 0; j__ < BITS; ++j__) {                   \
+        wreg[j__] = wnext.get(j__);                                              \
+      }                                                                          \
+      sreg = snext;                                                              \
+      breg = bnext;                                                              \
     }                                                                            \
-  } while (0)
-
-#define QMM_STORE_X(set, stage)                                                  \
-  do {                                                                           \
-    T* xs__ = lds + (stage) * kStage;                                            \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 0) * kLdsStride + xc * 8]) = QMM_XQ(set, 0);   \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 64) * kLdsStride + xc * 8]) = QMM_XQ(set, 1);  \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 128) * kLdsStride + xc * 8]) = QMM_XQ(set, 2); \
-    *reinterpret_cast<uint4*>(&xs__[(xr + 192) * kLdsStride + xc * 8]) = QMM_XQ(set, 3); \
   } while (0)
 
 #define QMM_STORE_W(stage)                                                       \
   do {                                                                           \
-    T* ws__ = lds + (stage) * kStage + kXTile;                                   \
+    T* ws__ = lds + kWBase + (stage) * kWTile;                                   \
     uint32_t dq__[16];                                                           \
     if constexpr (WN) {                                                          \
       float sf__[4], bf__[4];                                                    \
@@ -314,7 +443,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
             make_uint2(dq__[2 * i__], dq__[2 * i__ + 1]);                        \
       }                                                                          \
     } else {                                                                     \
-      dequant32<T, BITS>(wreg, to_f32(sreg[0]), to_f32(breg[0]), dq__);          \
+      dequant32<T, BITS>(wreg, raw_value<TS>(sreg), raw_value<TS>(breg), dq__);  \
       uint4* dst__ = reinterpret_cast<uint4*>(&ws__[wr * kLdsStride + wh * 32]); \
       _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
         dst__[j__] = make_uint4(                                                 \
@@ -338,8 +467,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 
   const int fi = lane & 15; // fragment row inside a 16-row MFMA tile
   const int fk = lane >> 4; // which 8 of the 32 k of an MFMA step
-  const int xfrag_off = (wm * 64 + fi) * kLdsStride + fk * 8;
-  const int wfrag_off = kXTile + (wn * 16 * NT + fi) * kLdsStride + fk * 8;
+  // x fragment of k slice s: logical piece 4 s + fk of row fi (+ multiples of
+  // 16), which sits at piece (4 s + fk) ^ (fi % 8)
+  const int xfrag_off0 = (wm * 64 + fi) * kBK + ((fk) ^ (fi & 7)) * 8;
+  const int xfrag_off1 = (wm * 64 + fi) * kBK + ((4 + fk) ^ (fi & 7)) * 8;
+  const int wfrag_off = kWBase + (wn * 16 * NT + fi) * kLdsStride + fk * 8;
 
   // MFMA operand fragments.  All four x fragments of a 32-wide k slice stay in
   // registers (two sets, one per slice); the W fragments stream through a ring
@@ -348,13 +480,14 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   // are the first fragments of the next step.
   uint4 bfr[2][4];
   uint4 afr[4];
-  auto read_b = [&](int stage, int s, int b) {
+  // `xs`: element offset of the x stage
+  auto read_b = [&](int xs, int s, int b) {
     bfr[s][b] = *reinterpret_cast<const uint4*>(
-        lds + stage * kStage + xfrag_off + b * 16 * kLdsStride + s * 32);
+        lds + xs + (s == 0 ? xfrag_off0 : xfrag_off1) + b * 16 * kBK);
   };
   auto read_a = [&](int stage, int s, int t, int slot) {
     afr[slot] = *reinterpret_cast<const uint4*>(
-        lds + stage * kStage + wfrag_off + t * 16 * kLdsStride + s * 32);
+        lds + stage * kWTile + wfrag_off + t * 16 * kLdsStride + s * 32);
   };
 
   // ---- software pipeline, one barrier per K-step.  Step t issues 8 NT MFMAs
@@ -386,27 +519,30 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   const int klast = (nk - 1) * kBK;
   // x-image offset of local step t, clamped to the range's last step
   auto kclamp = [&](int t) { return kbeg + (t * kBK < klast ? t * kBK : klast); };
-  QMM_LOAD_X(0, kbeg);
+  // x tiles 0 and 1 on their way into stages 0 and 1, W tile 0 dequantized into
+  // its stage, the packed W of tile 1 in registers
+  QMM_DMA_X(0, kbeg);
   QMM_LOAD_W(kbeg);
+  QMM_DMA_X(kXTile, kclamp(1));
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  QMM_PIN_W();
+  __builtin_amdgcn_sched_barrier(0);
   QMM_ROTATE_W();
-  QMM_STORE_X(0, 0);
   QMM_STORE_W(0);
-  // same order as in the loop (x of one step, packed W, x of the next step): the
-  // compiler's wait counts at the loop head are the stricter of this path's and
-  // the back edge's, and a different order here makes every step wait for loads
-  // it has only just issued
-  QMM_LOAD_X(0, kclamp(1));
   QMM_LOAD_W(kclamp(1));
-  if constexpr (kXSets == 2) {
-    QMM_LOAD_X(1, kclamp(2));
-  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // x tiles 0 and 1 have landed too
+  QMM_PIN_W();
+  __builtin_amdgcn_sched_barrier(0);
   QMM_ROTATE_W();
   __syncthreads();
-  read_b(0, 0, 0);
+  int xs_cur = 0;            // stage of the tile being multiplied
+  int xs_nxt = kXTile;       // stage of the next tile
+  int xs_new = 2 * kXTile;   // free stage: receives the tile after that
+  read_b(xs_cur, 0, 0);
   read_a(0, 0, 0, 0);
-  read_b(0, 0, 1);
-  read_b(0, 0, 2);
-  read_b(0, 0, 3);
+  read_b(xs_cur, 0, 1);
+  read_b(xs_cur, 0, 2);
+  read_b(xs_cur, 0, 3);
   read_a(0, 0, 1, 1);
   read_a(0, 0, 2, 2);
   read_a(0, 0, 3, 3);
@@ -430,11 +566,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
       }                                                                          \
     }                                                                            \
     if constexpr (s__ == 0 && t__ >= NT - 4 && b__ == 1) {                       \
-      read_b(cur, 1, t__ - (NT - 4));                                            \
+      read_b(xs_cur, 1, t__ - (NT - 4));                                         \
     }                                                                            \
     if constexpr ((m) == kNS - 12 || (m) == kNS - 11 || (m) == kNS - 10 ||       \
                   (m) == kNS - 8) {                                              \
-      read_b(nxt, 0, (m) == kNS - 8 ? 3 : (m) - (kNS - 12));                     \
+      read_b(xs_nxt, 0, (m) == kNS - 8 ? 3 : (m) - (kNS - 12));                  \
     }                                                                            \
     if constexpr ((m) == 0) {                                                    \
       QMM_LOAD_W(k2);                                                            \
@@ -460,23 +596,24 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
             dqv[4 * r__], dqv[4 * r__ + 1], dqv[4 * r__ + 2], dqv[4 * r__ + 3]); \
       }                                                                          \
     }                                                                            \
+    /* x tile tt + 2 into the stage that the barrier of the previous step freed; \
+       these are the last loads issued before this step's barrier */            \
     if constexpr ((m) == 1) {                                                    \
-      *reinterpret_cast<uint4*>(&xs[(xr + 0) * kLdsStride + xc * 8]) = QMM_XQ(P, 0);   \
-      QMM_XQ(P, 0) = *reinterpret_cast<const uint4*>(p.x + xoff0 + kx);          \
+      QMM_DMA_X1(xs_new, kx, 0, xoff0);                                          \
     }                                                                            \
     if constexpr ((m) == 5) {                                                    \
-      *reinterpret_cast<uint4*>(&xs[(xr + 64) * kLdsStride + xc * 8]) = QMM_XQ(P, 1);  \
-      QMM_XQ(P, 1) = *reinterpret_cast<const uint4*>(p.x + xoff1 + kx);          \
+      QMM_DMA_X1(xs_new, kx, 1, xoff1);                                          \
     }                                                                            \
     if constexpr ((m) == 9) {                                                    \
-      *reinterpret_cast<uint4*>(&xs[(xr + 128) * kLdsStride + xc * 8]) = QMM_XQ(P, 2); \
-      QMM_XQ(P, 2) = *reinterpret_cast<const uint4*>(p.x + xoff2 + kx);          \
+      QMM_DMA_X1(xs_new, kx, 2, xoff2);                                          \
     }                                                                            \
     if constexpr ((m) == 13) {                                                   \
-      *reinterpret_cast<uint4*>(&xs[(xr + 192) * kLdsStride + xc * 8]) = QMM_XQ(P, 3); \
-      QMM_XQ(P, 3) = *reinterpret_cast<const uint4*>(p.x + xoff3 + kx);          \
+      QMM_DMA_X1(xs_new, kx, 3, xoff3);                                          \
     }                                                                            \
     if constexpr ((m) == kNS - 14) {                                             \
+      /* all but this step's four x loads have completed: x tile tt + 1 is in */ \
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");                           \
+      QMM_PIN_W();                                                               \
       __syncthreads();                                                           \
     }                                                                            \
     __builtin_amdgcn_sched_barrier(0);                                           \
@@ -492,14 +629,14 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const int cur = (P);                                                         \
     const int nxt = (P) ^ 1;                                                     \
     const int k2 = kclamp((tt) + 2);                                             \
-    const int kx = kclamp((tt) + 1 + kXSets);                                    \
-    T* xs = lds + nxt * kStage;                                                  \
-    uint4* wdst = reinterpret_cast<uint4*>(&xs[kXTile + wr * kLdsStride + wh * 32]); \
-    T* wcol = &xs[kXTile + (8 * ng) * kLdsStride + 4 * kg];                      \
+    const int kx = k2;                                                           \
+    T* ws = lds + kWBase + nxt * kWTile;                                         \
+    uint4* wdst = reinterpret_cast<uint4*>(&ws[wr * kLdsStride + wh * 32]);      \
+    T* wcol = &ws[(8 * ng) * kLdsStride + 4 * kg];                               \
     float sf[kSB], bf[kSB];                                                      \
     _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
-      sf[j__] = WN ? wn_value(swn, j__) : to_f32(sreg[0]);                       \
-      bf[j__] = WN ? wn_value(bwn, j__) : to_f32(breg[0]);                       \
+      sf[j__] = WN ? wn_value(swn, j__) : raw_value<TS>(sreg);                   \
+      bf[j__] = WN ? wn_value(bwn, j__) : raw_value<TS>(breg);                   \
     }                                                                            \
     /* the tile prepared in step tt is tile tt + 1: block (tt + 1) % 3 of its   \
        group of three takes the weights' low parts */                           \
@@ -511,6 +648,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     QMM_SLOTS8(0, P) QMM_SLOTS8(8, P) QMM_SLOTS8(16, P) QMM_SLOTS8(24, P)        \
     QMM_SLOTS8(32, P) QMM_SLOTS8(40, P) QMM_SLOTS8(48, P) QMM_SLOTS8(56, P)      \
     QMM_ROTATE_W();                                                              \
+    {                                                                            \
+      const int freed = xs_cur;                                                  \
+      xs_cur = xs_nxt;                                                           \
+      xs_nxt = xs_new;                                                           \
+      xs_new = freed;                                                            \
+    }                                                                            \
   }
 
   int t = 0;
@@ -535,6 +678,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   constexpr int kPiece = 16 / static_cast<int>(sizeof(TO)); // elements per 16 bytes
   constexpr int kOutStride = kBN + kOutPad;
   TO* ys = reinterpret_cast<TO*>(smem);
+  // the last steps' (clamped) loads must not land in LDS after it changes hands,
+  // nor in registers that have been given to something else: their destinations
+  // stay allocated until the wait
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  QMM_PIN_W();
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
     __syncthreads(); // LDS is free: K loop (pass 0) or the previous half is done
@@ -597,16 +745,17 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   }
 }
 
-#undef QMM_XQ
-#undef QMM_LOAD_X
+#undef QMM_DMA_X
+#undef QMM_DMA_X1
 #undef QMM_LOAD_W
 #undef QMM_ROTATE_W
-#undef QMM_STORE_X
+#undef QMM_PIN_W
 #undef QMM_STORE_W
 
 template <int NT>
 constexpr size_t qmm_smem_bytes() {
-  constexpr size_t stages = static_cast<size_t>(2) * (kBM + 32 * NT) * kLdsStride * 2;
+  constexpr size_t stages =
+      (static_cast<size_t>(3) * kBM * kBK + static_cast<size_t>(2) * 32 * NT * kLdsStride) * 2;
   // staged y tile: all 256 rows of a 16-bit tile or 128 rows of an fp32 tile
   constexpr size_t out = static_cast<size_t>(kBM) * (32 * NT + kOutPad) * 2;
   return stages > out ? stages : out;
