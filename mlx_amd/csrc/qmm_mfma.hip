@@ -31,9 +31,9 @@
 // eight 128-byte rows), three stages deep, with the pieces of a row XOR-swizzled
 // by the row number so that the 16-byte fragment reads of 16 consecutive rows
 // spread over the banks (an LDS store from registers costs the matrix pipe
-// about 30 clocks of issue on its SIMD; the x tile was half of them).  W rows in
-// LDS are 64 elements + 8 of padding (144 bytes), conflict free for the same
-// reads.  The finished tile is staged through LDS once more so that y is
+// about 30 clocks of issue on its SIMD; the x tile was half of them).  The W
+// tile uses the same unpadded, swizzled rows (measured: fragment reads of
+// 144-byte padded rows run 20 % slower than swizzled 128-byte rows).  The finished tile is staged through LDS once more so that y is
 // written in full 16-byte, row-contiguous stores.
 #include "mfma_dequant.h"
 #include "qmm_args.h"
@@ -66,8 +66,9 @@ struct RawTuple;
 template <>
 struct RawTuple<1> {
   uint32_t v;
-  __device__ __forceinline__ void load(const uint32_t* p) {
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p));
+  template <int OFF>
+  __device__ __forceinline__ void load(uint32_t voff, const void* sbase) {
+    asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(sbase), "n"(OFF));
   }
   __device__ __forceinline__ uint32_t get(int) const { return v; }
   __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
@@ -75,8 +76,9 @@ struct RawTuple<1> {
 template <>
 struct RawTuple<2> {
   raw_u32x2 v;
-  __device__ __forceinline__ void load(const uint32_t* p) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(p));
+  template <int OFF>
+  __device__ __forceinline__ void load(uint32_t voff, const void* sbase) {
+    asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(sbase), "n"(OFF));
   }
   __device__ __forceinline__ uint32_t get(int j) const { return v[j]; }
   __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
@@ -84,8 +86,9 @@ struct RawTuple<2> {
 template <>
 struct RawTuple<3> {
   raw_u32x3 v;
-  __device__ __forceinline__ void load(const uint32_t* p) {
-    asm volatile("global_load_dwordx3 %0, %1, off" : "=v"(v) : "v"(p));
+  template <int OFF>
+  __device__ __forceinline__ void load(uint32_t voff, const void* sbase) {
+    asm volatile("global_load_dwordx3 %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(sbase), "n"(OFF));
   }
   __device__ __forceinline__ uint32_t get(int j) const { return v[j]; }
   __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
@@ -93,15 +96,17 @@ struct RawTuple<3> {
 template <>
 struct RawTuple<4> {
   raw_u32x4 v;
-  __device__ __forceinline__ void load(const uint32_t* p) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p));
+  template <int OFF>
+  __device__ __forceinline__ void load(uint32_t voff, const void* sbase) {
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(sbase), "n"(OFF));
   }
   __device__ __forceinline__ uint32_t get(int j) const { return v[j]; }
   __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
 };
 template <>
 struct RawTuple<0> {
-  __device__ __forceinline__ void load(const uint32_t*) {}
+  template <int OFF>
+  __device__ __forceinline__ void load(uint32_t, const void*) {}
   __device__ __forceinline__ uint32_t get(int) const { return 0; }
   __device__ __forceinline__ void pin() {}
 };
@@ -116,9 +121,10 @@ struct RawWords {
   static constexpr int kB = N - kA;         // of the second (0..4)
   RawTuple<kA> a;
   RawTuple<kB> b;
-  __device__ __forceinline__ void load(const uint32_t* p) {
-    a.load(p);
-    b.load(p + 4);
+  // dwords at sbase + voff (a uniform 64-bit base plus a per-lane byte offset)
+  __device__ __forceinline__ void load(uint32_t voff, const void* sbase) {
+    a.template load<0>(voff, sbase);
+    b.template load<16>(voff, sbase);
   }
   __device__ __forceinline__ uint32_t get(int j) const {
     return j < 4 ? a.get(j) : b.get(j - 4);
@@ -131,11 +137,11 @@ struct RawWords {
 
 // One scale or bias value as loaded: 16 bits in the low half, or a float.
 template <typename TS>
-__device__ __forceinline__ void raw_load_value(uint32_t& v, const TS* p) {
+__device__ __forceinline__ void raw_load_value(uint32_t& v, uint32_t voff, const void* sbase) {
   if constexpr (sizeof(TS) == 2) {
-    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p));
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
   } else {
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p));
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
   }
 }
 template <typename TS>
@@ -149,7 +155,6 @@ __device__ __forceinline__ float raw_value(uint32_t v) {
 
 constexpr int kBM = 256;
 constexpr int kBK = 64;
-constexpr int kLdsStride = kBK + 8; // elements per LDS row
 constexpr int kThreads = 512;
 constexpr int kOutPad = 8; // elements of padding per row of the staged y tile
 
@@ -209,7 +214,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   // three unpadded x stages (filled by direct-to-LDS loads), then two W stages
   constexpr int kXTile = kBM * kBK; // elements
   constexpr int kXStages = 3;
-  constexpr int kWTile = kBN * kLdsStride;
+  constexpr int kWTile = kBN * kBK; // unpadded rows, pieces XOR-swizzled like x
   constexpr int kWBase = kXStages * kXTile;
   T* lds = reinterpret_cast<T*>(smem);
 
@@ -296,30 +301,43 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   const int wt = tid < 16 * kColBlocks ? tid : 16 * kColBlocks - 1;
   const int kg = wt & 15;
   const int ng = wt >> 4;
-  const uint32_t* wsrc;
-  const TS* ssrc;
-  const TS* bsrc;
+  // Where the dequantized weights go in a W stage (element offsets).  Rows are
+  // 64 elements, eight 16-byte pieces; piece c of row r sits at c ^ (r % 8).
+  // transpose=true: thread (wr, wh) writes pieces 4 wh + j, j < 4, of row wr.
+  int wrow_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    wrow_off[j] = wr * kBK + (((4 * wh + j) ^ (wr & 7)) * 8);
+  }
+  // [K, N] weights: the thread's column i (row 8 ng + i of the tile, so r % 8 == i)
+  // takes 8 bytes at k = 4 kg: half (kg % 2) of piece kg / 2
+  auto wcol_off = [&](int i) { return (8 * ng + i) * kBK + (((kg >> 1) ^ i) * 8) + (kg & 1) * 4; };
+
+  // Per-lane byte offsets from the operands' uniform base pointers (32 bits:
+  // the launcher checks the sizes); the K-step's part of an address is uniform
+  // and goes into the scalar base, so the loop computes no addresses per lane.
+  uint32_t w_voff, sb_voff;
   if constexpr (WN) {
     const int ncol = (n0 + 8 * ng < N) ? n0 + 8 * ng : N - 8; // clamp: stay in bounds
-    wsrc = reinterpret_cast<const uint32_t*>(p.w) +
-        static_cast<size_t>(4 * kg) * row_words + ncol / 8 * kWPR;
+    w_voff = (static_cast<uint32_t>(4 * kg) * row_words + ncol / 8 * kWPR) * 4u;
     // scales / biases arrive transposed, [group][k] (the launcher's pre-pass): the
     // four rows' values are 8 contiguous bytes
-    ssrc = p.scales + static_cast<size_t>(ncol >> gs_shift) * K + 4 * kg;
-    bsrc = p.biases + static_cast<size_t>(ncol >> gs_shift) * K + 4 * kg;
+    sb_voff = (static_cast<uint32_t>(ncol >> gs_shift) * K + 4 * kg) * static_cast<uint32_t>(sizeof(TS));
   } else {
     const int w_row = (n0 + wr < N) ? n0 + wr : N - 1; // clamp: loads stay in bounds
-    wsrc = reinterpret_cast<const uint32_t*>(p.w) +
-        static_cast<size_t>(w_row) * row_words + wh * BITS;
+    w_voff = (static_cast<uint32_t>(w_row) * row_words + wh * BITS) * 4u;
     // group g of row w_row: [row][g], or [g][row] in the transposed image
-    const size_t sb_row = a.sb_transposed ? static_cast<size_t>(w_row)
-                                          : static_cast<size_t>(w_row) * groups;
-    ssrc = p.scales + sb_row;
-    bsrc = p.biases + sb_row;
+    sb_voff = (a.sb_transposed ? static_cast<uint32_t>(w_row)
+                               : static_cast<uint32_t>(w_row) * groups) * static_cast<uint32_t>(sizeof(TS));
   }
   const size_t sb_gstride = a.sb_transposed ? static_cast<size_t>(N) : 1;
+  // thread (wr, wh) needs the group of codes [32 wh, 32 wh + 32) of the step:
+  // group (k0 + 32 wh) >> gs_shift, i.e. one further than the step's first group
+  // only when groups are 32 wide and wh == 1
+  const uint32_t sb_half = (!WN && gs_shift == 5 && wh == 1)
+      ? static_cast<uint32_t>(sb_gstride * sizeof(TS)) : 0u;
   // Rows of x past M are never stored, so they may read any valid row: the
-  // loads then need no predicate.  32-bit element offsets from p.x.
+  // loads then need no predicate.  32-bit byte offsets from p.x.
   uint32_t xoff0, xoff1, xoff2, xoff3;
   {
     auto row_off = [&](int i) {
@@ -327,9 +345,9 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
       const int mc = m < M ? m : M - 1;
       if constexpr (GROUPED) {
         const uint32_t pair = static_cast<uint32_t>(a.group_perm[row0 + mc]);
-        return a.lhs_indices[pair] * static_cast<uint32_t>(a.x_batch_stride) + xc * 8;
+        return (a.lhs_indices[pair] * static_cast<uint32_t>(a.x_batch_stride) + xc * 8) * 2u;
       } else {
-        return static_cast<uint32_t>(mc) * static_cast<uint32_t>(Kx) + xc * 8;
+        return (static_cast<uint32_t>(mc) * static_cast<uint32_t>(Kx) + xc * 8) * 2u;
       }
     };
     xoff0 = row_off(0);
@@ -356,12 +374,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 // (element offset of the stage); completion is counted by vmcnt.
 #define QMM_DMA_X1(xs, k0, i, xoff)                                              \
   do {                                                                           \
-    const T* g__ = p.x + (xoff) + (k0);                                          \
+    const T* g__ = p.x + (k0); /* uniform */                                     \
     const uint32_t m0__ = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(     \
         (__attribute__((address_space(3))) char*)(lds + (xs) + (wave * 32 + 8 * (i)) * kBK))); \
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"           \
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"            \
                  :                                                               \
-                 : "v"(g__), "s"(m0__)                                           \
+                 : "v"(xoff), "s"(g__), "s"(m0__)                                \
                  : "memory");                                                    \
   } while (0)
 #define QMM_DMA_X(xs, k0)                                                        \
@@ -375,19 +393,22 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 #define QMM_LOAD_W(k0)                                                           \
   do {                                                                           \
     if constexpr (WN) {                                                          \
-      const uint32_t* wp__ = wsrc + static_cast<size_t>(k0) * row_words;         \
+      const uint32_t* wp__ = reinterpret_cast<const uint32_t*>(p.w) +            \
+          static_cast<size_t>(k0) * row_words; /* uniform */                     \
       _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
-        wnext_row[j__].load(wp__ + static_cast<size_t>(j__) * row_words);        \
+        wnext_row[j__].load(w_voff, wp__ + static_cast<size_t>(j__) * row_words); \
       }                                                                          \
-      swn_next.load(reinterpret_cast<const uint32_t*>(ssrc + (k0)));             \
-      bwn_next.load(reinterpret_cast<const uint32_t*>(bsrc + (k0)));             \
+      swn_next.template load<0>(sb_voff, p.scales + (k0));                       \
+      bwn_next.template load<0>(sb_voff, p.biases + (k0));                       \
     } else {                                                                     \
       /* split mode: blocks 3t, 3t+1, 3t+2 of x all meet block t of W */         \
       const int kw__ = kSplit ? ((k0) / (3 * kBK)) * kBK : (k0);                 \
-      wnext.load(wsrc + (kw__ / 32) * BITS);                                     \
-      const size_t g__ = static_cast<size_t>((kw__ + 32 * wh) >> gs_shift) * sb_gstride; \
-      raw_load_value<TS>(snext, ssrc + g__);                                     \
-      raw_load_value<TS>(bnext, bsrc + g__);                                     \
+      wnext.load(w_voff, reinterpret_cast<const uint32_t*>(p.w) + (kw__ / 32) * BITS); \
+      /* a K-step lies inside one group when groups are 64 or 128 wide; with    \
+         32-wide groups the two halves of a row differ by one group */          \
+      const size_t g0__ = static_cast<size_t>(kw__ >> gs_shift) * sb_gstride;    \
+      raw_load_value<TS>(snext, sb_voff + sb_half, p.scales + g0__);             \
+      raw_load_value<TS>(bnext, sb_voff + sb_half, p.biases + g0__);             \
     }                                                                            \
   } while (0)
 
@@ -437,16 +458,14 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
         bf__[j__] = wn_value(bwn, j__);                                          \
       }                                                                          \
       dequant_cols<T, BITS>(wreg, sf__, bf__, dq__);                             \
-      T* col__ = &ws__[(8 * ng) * kLdsStride + 4 * kg];                          \
       _Pragma("unroll") for (int i__ = 0; i__ < 8; ++i__) {                      \
-        *reinterpret_cast<uint2*>(col__ + i__ * kLdsStride) =                    \
+        *reinterpret_cast<uint2*>(ws__ + wcol_off(i__)) =                        \
             make_uint2(dq__[2 * i__], dq__[2 * i__ + 1]);                        \
       }                                                                          \
     } else {                                                                     \
       dequant32<T, BITS>(wreg, raw_value<TS>(sreg), raw_value<TS>(breg), dq__);  \
-      uint4* dst__ = reinterpret_cast<uint4*>(&ws__[wr * kLdsStride + wh * 32]); \
       _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
-        dst__[j__] = make_uint4(                                                 \
+        *reinterpret_cast<uint4*>(ws__ + wrow_off[j__]) = make_uint4(            \
             dq__[4 * j__], dq__[4 * j__ + 1], dq__[4 * j__ + 2], dq__[4 * j__ + 3]); \
       }                                                                          \
     }                                                                            \
@@ -471,7 +490,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   // 16), which sits at piece (4 s + fk) ^ (fi % 8)
   const int xfrag_off0 = (wm * 64 + fi) * kBK + ((fk) ^ (fi & 7)) * 8;
   const int xfrag_off1 = (wm * 64 + fi) * kBK + ((4 + fk) ^ (fi & 7)) * 8;
-  const int wfrag_off = kWBase + (wn * 16 * NT + fi) * kLdsStride + fk * 8;
+  const int wfrag_off0 = kWBase + (wn * 16 * NT + fi) * kBK + ((fk) ^ (fi & 7)) * 8;
+  const int wfrag_off1 = kWBase + (wn * 16 * NT + fi) * kBK + ((4 + fk) ^ (fi & 7)) * 8;
 
   // MFMA operand fragments.  All four x fragments of a 32-wide k slice stay in
   // registers (two sets, one per slice); the W fragments stream through a ring
@@ -487,7 +507,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   };
   auto read_a = [&](int stage, int s, int t, int slot) {
     afr[slot] = *reinterpret_cast<const uint4*>(
-        lds + stage * kWTile + wfrag_off + t * 16 * kLdsStride + s * 32);
+        lds + stage * kWTile + (s == 0 ? wfrag_off0 : wfrag_off1) + t * 16 * kBK);
   };
 
   // ---- software pipeline, one barrier per K-step.  Step t issues 8 NT MFMAs
@@ -587,12 +607,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
       constexpr int r__ = wstore_at((m), kNS);                                   \
       if constexpr (WN) {                                                        \
         /* pairs 4r .. 4r+3: columns 2r and 2r+1, four rows (k) each */          \
-        *reinterpret_cast<uint2*>(wcol + (2 * r__) * kLdsStride) =               \
+        *reinterpret_cast<uint2*>(ws + wcol_off(2 * r__)) =                      \
             make_uint2(dqv[4 * r__], dqv[4 * r__ + 1]);                          \
-        *reinterpret_cast<uint2*>(wcol + (2 * r__ + 1) * kLdsStride) =           \
+        *reinterpret_cast<uint2*>(ws + wcol_off(2 * r__ + 1)) =                  \
             make_uint2(dqv[4 * r__ + 2], dqv[4 * r__ + 3]);                      \
       } else {                                                                   \
-        wdst[r__] = make_uint4(                                                  \
+        *reinterpret_cast<uint4*>(ws + wrow_off[r__]) = make_uint4(              \
             dqv[4 * r__], dqv[4 * r__ + 1], dqv[4 * r__ + 2], dqv[4 * r__ + 3]); \
       }                                                                          \
     }                                                                            \
@@ -631,8 +651,6 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const int k2 = kclamp((tt) + 2);                                             \
     const int kx = k2;                                                           \
     T* ws = lds + kWBase + nxt * kWTile;                                         \
-    uint4* wdst = reinterpret_cast<uint4*>(&ws[wr * kLdsStride + wh * 32]);      \
-    T* wcol = &ws[(8 * ng) * kLdsStride + 4 * kg];                               \
     float sf[kSB], bf[kSB];                                                      \
     _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
       sf[j__] = WN ? wn_value(swn, j__) : raw_value<TS>(sreg);                   \
@@ -755,7 +773,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 template <int NT>
 constexpr size_t qmm_smem_bytes() {
   constexpr size_t stages =
-      (static_cast<size_t>(3) * kBM * kBK + static_cast<size_t>(2) * 32 * NT * kLdsStride) * 2;
+      (static_cast<size_t>(3) * kBM * kBK + static_cast<size_t>(2) * 32 * NT * kBK) * 2;
   // staged y tile: all 256 rows of a 16-bit tile or 128 rows of an fp32 tile
   constexpr size_t out = static_cast<size_t>(kBM) * (32 * NT + kOutPad) * 2;
   return stages > out ? stages : out;
