@@ -60,9 +60,17 @@ __device__ __forceinline__ uint32_t code32(const uint32_t (&w)[BITS], int i) {
 template <typename T, int BITS>
 struct PairDequant {
   uint32_t lo, hi; // 4-bit: codes 0,2,4,6 / 1,3,5,7 of the current dword as bytes
+  floatx2 flo, fhi; // 4-bit: two of those bytes each, converted
+
+  // 4-bit codes are converted two at a time with the fp8 convert: a byte 0..15
+  // read as an OCP e4m3 number is exactly code * 2^-9 (the format is linear
+  // through its subnormals and first binade), so fma(512 s, code / 512, b) is
+  // the same real product, and the same rounding, as fma(s, code, b).
+  static constexpr float kCodeScale = BITS == 4 ? 512.0f : 1.0f;
 
   // low_part: return v - T(v) instead of v (the second term of the split of an
-  // fp32 weight into two T values); wave-uniform.
+  // fp32 weight into two T values); wave-uniform.  `s` is kCodeScale times the
+  // group's scale.
   template <int Q>
   __device__ __forceinline__ uint32_t
   pair(const uint32_t (&w)[BITS], float s, float b, bool low_part = false) {
@@ -73,13 +81,13 @@ struct PairDequant {
       if constexpr (j == 0) {
         lo = w[d] & 0x0f0f0f0fu;
         hi = (w[d] >> 4) & 0x0f0f0f0fu;
-        // keep the byte form: otherwise the shifts are folded back into one
-        // bit-field extract per code
-        asm("" : "+v"(lo));
-        asm("" : "+v"(hi));
       }
-      c0 = static_cast<float>((lo >> (8 * j)) & 0xffu);
-      c1 = static_cast<float>((hi >> (8 * j)) & 0xffu);
+      if constexpr (j % 2 == 0) {
+        flo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(lo), j == 2);
+        fhi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(hi), j == 2);
+      }
+      c0 = flo[j % 2];
+      c1 = fhi[j % 2];
     } else if constexpr (BITS == 8) {
       constexpr int d = Q / 2;
       constexpr int j = Q % 2;
@@ -176,7 +184,8 @@ __device__ __forceinline__ void dequant32_impl(
     uint32_t (&out)[16],
     std::integer_sequence<int, Q...>) {
   PairDequant<T, BITS> dq;
-  ((out[Q] = dq.template pair<Q>(w, s, b)), ...);
+  const float sc = s * PairDequant<T, BITS>::kCodeScale;
+  ((out[Q] = dq.template pair<Q>(w, sc, b)), ...);
 }
 
 // 32 codes -> 32 elements of T in one go (prologue).

@@ -653,7 +653,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     T* ws = lds + kWBase + nxt * kWTile;                                         \
     float sf[kSB], bf[kSB];                                                      \
     _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
-      sf[j__] = WN ? wn_value(swn, j__) : raw_value<TS>(sreg);                   \
+      sf[j__] = WN ? wn_value(swn, j__)                                          \
+                   : raw_value<TS>(sreg) * PairDequant<T, BITS>::kCodeScale;     \
       bf[j__] = WN ? wn_value(bwn, j__) : raw_value<TS>(breg);                   \
     }                                                                            \
     /* the tile prepared in step tt is tile tt + 1: block (tt + 1) % 3 of its   \
