@@ -43,7 +43,20 @@ typedef enum {
 typedef enum {
   MLXROCM_FLOAT32 = 0,
   MLXROCM_FLOAT16 = 1,
-  MLXROCM_BFLOAT16 = 2
+  MLXROCM_BFLOAT16 = 2,
+  /* The quantization entry points take the three types above; the element
+   * copies also take the rest of mlx::core::Dtype (mlx/dtype.h:15-30). */
+  MLXROCM_BOOL = 3,
+  MLXROCM_UINT8 = 4,
+  MLXROCM_UINT16 = 5,
+  MLXROCM_UINT32 = 6,
+  MLXROCM_UINT64 = 7,
+  MLXROCM_INT8 = 8,
+  MLXROCM_INT16 = 9,
+  MLXROCM_INT32 = 10,
+  MLXROCM_INT64 = 11,
+  MLXROCM_FLOAT64 = 12,
+  MLXROCM_COMPLEX64 = 13
 } mlxrocm_dtype;
 
 typedef void* mlxrocm_stream_t; /* hipStream_t */
@@ -320,6 +333,51 @@ const char* mlxrocm_qmm_kernel_name(
     int transpose);
 
 /* ------------------------------------------------------------------------ */
+/* Element copies with dtype conversion                                      */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * The data movement eval_gpu bodies do around the matmul kernels: making an
+ * operand row-contiguous, converting scales/biases to the activation type,
+ * astype of a result, filling with a scalar.  Replaces copy_gpu_inplace and
+ * fill_gpu (mlx/backend/gpu/copy.h:14-51; CUDA kernels
+ * mlx/backend/cuda/copy/copy_contiguous.cu, copy_general.cu,
+ * copy_general_input.cu).  All pointers are device memory; offsets are applied
+ * by the caller (pointer + offset * item size).  Conversions follow static_cast:
+ * round-to-nearest-even into float types (16-bit floats through fp32),
+ * truncation toward zero into integers, != 0 into bool; complex64 -> real drops
+ * the imaginary part, real -> complex64 sets it to zero.
+ */
+size_t mlxrocm_dtype_size(int dtype); /* bytes per element, 0 if unknown */
+
+/* dst[i] = (dst_dtype) src[i] for i < n, or src[0] for every i when
+ * broadcast_scalar is non-zero (CopyType::Vector / CopyType::Scalar). */
+int mlxrocm_copy_contiguous(
+    const void* src,
+    int src_dtype,
+    void* dst,
+    int dst_dtype,
+    size_t n,
+    int broadcast_scalar,
+    mlxrocm_stream_t stream);
+
+/* dst[sum_d i_d * dst_strides[d]] = (dst_dtype) src[sum_d i_d * src_strides[d]]
+ * over the index space `shape` (CopyType::General / GeneralGeneral).  Strides
+ * are in elements and may be zero or negative; dst_strides == NULL means a
+ * row-contiguous destination.  Extent-1 and jointly contiguous dimensions are
+ * merged first; more than 8 remaining dimensions are MLXROCM_UNSUPPORTED. */
+int mlxrocm_copy_strided(
+    const void* src,
+    int src_dtype,
+    const int64_t* src_strides,
+    void* dst,
+    int dst_dtype,
+    const int64_t* dst_strides,
+    int ndim,
+    const int64_t* shape,
+    mlxrocm_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
 /* Device memory with explicit residency, streams, events                    */
 /* ------------------------------------------------------------------------ */
 
@@ -359,6 +417,9 @@ int mlxrocm_stream_synchronize(mlxrocm_stream_t stream);
 /* Event plumbing behind mlx::core::Event (mlx/event.h; model
  * mlx/backend/cuda/event.cu:330-420). */
 int mlxrocm_event_create(mlxrocm_event_t* event);
+/* An event without timing whose synchronize sleeps instead of spinning: for a
+ * host thread that waits on GPU completion (mlx/backend/cuda/worker.cpp:8-10). */
+int mlxrocm_event_create_blocking(mlxrocm_event_t* event);
 int mlxrocm_event_destroy(mlxrocm_event_t event);
 int mlxrocm_event_record(mlxrocm_event_t event, mlxrocm_stream_t stream);
 int mlxrocm_event_wait(mlxrocm_event_t event, mlxrocm_stream_t stream);

@@ -66,7 +66,13 @@ SIGNATURES = {
     "mlxrocm_stream_destroy": (_i, [_p]),
     "mlxrocm_stream_synchronize": (_i, [_p]),
     "mlxrocm_event_create": (_i, [ctypes.POINTER(_p)]),
+    "mlxrocm_event_create_blocking": (_i, [ctypes.POINTER(_p)]),
     "mlxrocm_event_destroy": (_i, [_p]),
+    "mlxrocm_dtype_size": (ctypes.c_size_t, [_i]),
+    "mlxrocm_copy_contiguous": (_i, [_p, _i, _p, _i, ctypes.c_size_t, _i, _p]),
+    "mlxrocm_copy_strided": (_i, [_p, _i, ctypes.POINTER(ctypes.c_int64), _p, _i,
+                                  ctypes.POINTER(ctypes.c_int64), _i,
+                                  ctypes.POINTER(ctypes.c_int64), _p]),
     "mlxrocm_event_record": (_i, [_p, _p]),
     "mlxrocm_event_wait": (_i, [_p, _p]),
     "mlxrocm_event_synchronize": (_i, [_p]),

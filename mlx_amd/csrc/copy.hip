@@ -1,0 +1,395 @@
+// copy.hip -- element copies with dtype conversion and scalar fill: the data
+// movement every eval_gpu body needs around the matmul kernels (making an input
+// row-contiguous, converting scales/biases to the activation type, astype of
+// the result).  Counterpart of copy_gpu_inplace / fill_gpu
+// (mlx/backend/gpu/copy.h:14-51; the CUDA kernels are
+// mlx/backend/cuda/copy/copy_contiguous.cu and copy_general*.cu).
+//
+// Both kernels are plain HBM streams: one 16-byte vector per lane on the
+// narrower side when source and destination are contiguous and aligned, one
+// element per lane with a div/mod walk over at most kMaxDims collapsed
+// dimensions otherwise.  Conversions follow static_cast (round-to-nearest-even
+// into the float types, truncation toward zero into the integer types, != 0
+// into bool); complex64 converts to a real type by dropping the imaginary part
+// and from one with a zero imaginary part.
+#include <algorithm>
+#include <type_traits>
+
+#include "common.h"
+
+namespace mlxrocm {
+namespace {
+
+struct complex64 {
+  float re;
+  float im;
+};
+
+template <int DT> struct TypeOf;
+template <> struct TypeOf<MLXROCM_FLOAT32> { using type = float; };
+template <> struct TypeOf<MLXROCM_FLOAT16> { using type = f16_t; };
+template <> struct TypeOf<MLXROCM_BFLOAT16> { using type = bf16_t; };
+template <> struct TypeOf<MLXROCM_BOOL> { using type = bool; };
+template <> struct TypeOf<MLXROCM_UINT8> { using type = uint8_t; };
+template <> struct TypeOf<MLXROCM_UINT16> { using type = uint16_t; };
+template <> struct TypeOf<MLXROCM_UINT32> { using type = uint32_t; };
+template <> struct TypeOf<MLXROCM_UINT64> { using type = uint64_t; };
+template <> struct TypeOf<MLXROCM_INT8> { using type = int8_t; };
+template <> struct TypeOf<MLXROCM_INT16> { using type = int16_t; };
+template <> struct TypeOf<MLXROCM_INT32> { using type = int32_t; };
+template <> struct TypeOf<MLXROCM_INT64> { using type = int64_t; };
+template <> struct TypeOf<MLXROCM_FLOAT64> { using type = double; };
+template <> struct TypeOf<MLXROCM_COMPLEX64> { using type = complex64; };
+
+constexpr int kNumDtypes = 14;
+constexpr size_t kItemSize[kNumDtypes] = {4, 2, 2, 1, 1, 2, 4, 8, 1, 2, 4, 8, 8, 8};
+
+template <typename T>
+constexpr bool is_half_v = std::is_same_v<T, f16_t> || std::is_same_v<T, bf16_t>;
+
+template <typename S, typename D>
+__device__ __forceinline__ D convert(S v) {
+  if constexpr (std::is_same_v<S, D>) {
+    return v;
+  } else if constexpr (std::is_same_v<S, complex64>) {
+    if constexpr (std::is_same_v<D, bool>) {
+      return v.re != 0.0f || v.im != 0.0f;
+    } else {
+      return convert<float, D>(v.re);
+    }
+  } else if constexpr (std::is_same_v<D, complex64>) {
+    return complex64{convert<S, float>(v), 0.0f};
+  } else if constexpr (std::is_same_v<D, bool>) {
+    if constexpr (is_half_v<S>) {
+      return static_cast<float>(v) != 0.0f;
+    } else {
+      return v != S(0);
+    }
+  } else if constexpr (is_half_v<S> && !std::is_floating_point_v<D>) {
+    // 16-bit floats reach the integer types (and each other) through fp32,
+    // which holds every one of their values.
+    return convert<float, D>(static_cast<float>(v));
+  } else if constexpr (is_half_v<D>) {
+    // Every source reaches a 16-bit float through fp32.
+    return static_cast<D>(static_cast<float>(v));
+  } else {
+    return static_cast<D>(v);
+  }
+}
+
+template <typename T, int E>
+struct alignas(sizeof(T) * E) Vec {
+  T v[E];
+};
+
+template <typename S, typename D>
+constexpr int vec_elems() {
+  constexpr size_t narrow = sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D);
+  constexpr int e = static_cast<int>(16 / narrow);
+  return e > 8 ? 8 : e;
+}
+
+constexpr int kCopyThreads = 256;
+
+// dst[i] = convert(src[i]) (or src[0] when SCALAR) for i < n; E elements per lane.
+template <typename S, typename D, int E, bool SCALAR>
+__global__ __launch_bounds__(kCopyThreads) void copy_contiguous_kernel(
+    const S* __restrict__ src,
+    D* __restrict__ dst,
+    size_t n) {
+  const size_t i = (static_cast<size_t>(blockIdx.x) * kCopyThreads + threadIdx.x) * E;
+  if (i >= n) {
+    return;
+  }
+  if constexpr (SCALAR) {
+    const D value = convert<S, D>(src[0]);
+    if (E > 1 && i + E <= n) {
+      Vec<D, E> out;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        out.v[e] = value;
+      }
+      *reinterpret_cast<Vec<D, E>*>(dst + i) = out;
+    } else {
+      for (size_t e = i; e < n && e < i + E; ++e) {
+        dst[e] = value;
+      }
+    }
+  } else {
+    if (E > 1 && i + E <= n) {
+      const Vec<S, E> in = *reinterpret_cast<const Vec<S, E>*>(src + i);
+      Vec<D, E> out;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        out.v[e] = convert<S, D>(in.v[e]);
+      }
+      *reinterpret_cast<Vec<D, E>*>(dst + i) = out;
+    } else {
+      for (size_t e = i; e < n && e < i + E; ++e) {
+        dst[e] = convert<S, D>(src[e]);
+      }
+    }
+  }
+}
+
+constexpr int kMaxDims = 8;
+
+struct StridedShape {
+  int ndim;
+  int64_t shape[kMaxDims];
+  int64_t src_stride[kMaxDims];
+  int64_t dst_stride[kMaxDims];
+};
+
+// One element per lane; IDX is uint32_t when every index fits.
+template <typename S, typename D, typename IDX>
+__global__ __launch_bounds__(kCopyThreads) void copy_strided_kernel(
+    const S* __restrict__ src,
+    D* __restrict__ dst,
+    StridedShape a,
+    size_t n) {
+  const size_t linear = static_cast<size_t>(blockIdx.x) * kCopyThreads + threadIdx.x;
+  if (linear >= n) {
+    return;
+  }
+  IDX rest = static_cast<IDX>(linear);
+  int64_t so = 0;
+  int64_t dof = 0;
+  for (int d = a.ndim - 1; d > 0; --d) {
+    const IDX extent = static_cast<IDX>(a.shape[d]);
+    const IDX q = rest / extent;
+    const IDX c = rest - q * extent;
+    so += static_cast<int64_t>(c) * a.src_stride[d];
+    dof += static_cast<int64_t>(c) * a.dst_stride[d];
+    rest = q;
+  }
+  so += static_cast<int64_t>(rest) * a.src_stride[0];
+  dof += static_cast<int64_t>(rest) * a.dst_stride[0];
+  dst[dof] = convert<S, D>(src[so]);
+}
+
+bool valid_copy_dtype(int dt) {
+  return dt >= 0 && dt < kNumDtypes;
+}
+
+// Calls f(TypeOf<dt>::type{}) for a runtime dtype code.
+template <typename F>
+int with_type(int dt, F&& f) {
+  switch (dt) {
+#define MLXROCM_CASE(code) \
+  case code:               \
+    return f(typename TypeOf<code>::type{});
+    MLXROCM_CASE(MLXROCM_FLOAT32)
+    MLXROCM_CASE(MLXROCM_FLOAT16)
+    MLXROCM_CASE(MLXROCM_BFLOAT16)
+    MLXROCM_CASE(MLXROCM_BOOL)
+    MLXROCM_CASE(MLXROCM_UINT8)
+    MLXROCM_CASE(MLXROCM_UINT16)
+    MLXROCM_CASE(MLXROCM_UINT32)
+    MLXROCM_CASE(MLXROCM_UINT64)
+    MLXROCM_CASE(MLXROCM_INT8)
+    MLXROCM_CASE(MLXROCM_INT16)
+    MLXROCM_CASE(MLXROCM_INT32)
+    MLXROCM_CASE(MLXROCM_INT64)
+    MLXROCM_CASE(MLXROCM_FLOAT64)
+    MLXROCM_CASE(MLXROCM_COMPLEX64)
+#undef MLXROCM_CASE
+    default:
+      return fail(MLXROCM_INVALID_ARGUMENT, "[copy] unknown dtype %d", dt);
+  }
+}
+
+constexpr size_t kMaxBlocks = 0x7fffffffull;
+
+template <typename S, typename D>
+int launch_contiguous(
+    const void* src, void* dst, size_t n, bool scalar, hipStream_t stream) {
+  constexpr int E = vec_elems<S, D>();
+  const bool aligned =
+      (scalar || reinterpret_cast<uintptr_t>(src) % (sizeof(S) * E) == 0) &&
+      reinterpret_cast<uintptr_t>(dst) % (sizeof(D) * E) == 0;
+  const S* s = static_cast<const S*>(src);
+  D* d = static_cast<D*>(dst);
+  const size_t per_block = static_cast<size_t>(kCopyThreads) * (aligned ? E : 1);
+  const size_t blocks = (n + per_block - 1) / per_block;
+  if (blocks > kMaxBlocks) {
+    return fail(MLXROCM_UNSUPPORTED, "[copy] %zu elements exceed one launch", n);
+  }
+  const dim3 grid(static_cast<unsigned>(blocks));
+  if (aligned && scalar) {
+    copy_contiguous_kernel<S, D, E, true><<<grid, kCopyThreads, 0, stream>>>(s, d, n);
+  } else if (aligned) {
+    copy_contiguous_kernel<S, D, E, false><<<grid, kCopyThreads, 0, stream>>>(s, d, n);
+  } else if (scalar) {
+    copy_contiguous_kernel<S, D, 1, true><<<grid, kCopyThreads, 0, stream>>>(s, d, n);
+  } else {
+    copy_contiguous_kernel<S, D, 1, false><<<grid, kCopyThreads, 0, stream>>>(s, d, n);
+  }
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return MLXROCM_OK;
+}
+
+template <typename S, typename D>
+int launch_strided(
+    const void* src, void* dst, const StridedShape& a, size_t n, bool wide, hipStream_t stream) {
+  const size_t blocks = (n + kCopyThreads - 1) / kCopyThreads;
+  if (blocks > kMaxBlocks) {
+    return fail(MLXROCM_UNSUPPORTED, "[copy] %zu elements exceed one launch", n);
+  }
+  const dim3 grid(static_cast<unsigned>(blocks));
+  const S* s = static_cast<const S*>(src);
+  D* d = static_cast<D*>(dst);
+  if (wide) {
+    copy_strided_kernel<S, D, uint64_t><<<grid, kCopyThreads, 0, stream>>>(s, d, a, n);
+  } else {
+    copy_strided_kernel<S, D, uint32_t><<<grid, kCopyThreads, 0, stream>>>(s, d, a, n);
+  }
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return MLXROCM_OK;
+}
+
+} // namespace
+} // namespace mlxrocm
+
+using namespace mlxrocm;
+
+extern "C" size_t mlxrocm_dtype_size(int dtype) {
+  return valid_copy_dtype(dtype) ? kItemSize[dtype] : 0;
+}
+
+extern "C" int mlxrocm_copy_contiguous(
+    const void* src,
+    int src_dtype,
+    void* dst,
+    int dst_dtype,
+    size_t n,
+    int broadcast_scalar,
+    mlxrocm_stream_t stream) {
+  if (!valid_copy_dtype(src_dtype) || !valid_copy_dtype(dst_dtype)) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT, "[copy] unknown dtype %d -> %d", src_dtype, dst_dtype);
+  }
+  if (n == 0) {
+    return MLXROCM_OK;
+  }
+  if (src == nullptr || dst == nullptr) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[copy] null pointer");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (src_dtype == dst_dtype && !broadcast_scalar) {
+    // Same type, same layout: the copy engine's path.
+    MLXROCM_HIP_TRY(hipMemcpyAsync(
+        dst, src, n * kItemSize[src_dtype], hipMemcpyDeviceToDevice, s));
+    return MLXROCM_OK;
+  }
+  return with_type(src_dtype, [&](auto st) {
+    using S = decltype(st);
+    return with_type(dst_dtype, [&](auto dt) {
+      using D = decltype(dt);
+      return launch_contiguous<S, D>(src, dst, n, broadcast_scalar != 0, s);
+    });
+  });
+}
+
+extern "C" int mlxrocm_copy_strided(
+    const void* src,
+    int src_dtype,
+    const int64_t* src_strides,
+    void* dst,
+    int dst_dtype,
+    const int64_t* dst_strides,
+    int ndim,
+    const int64_t* shape,
+    mlxrocm_stream_t stream) {
+  if (!valid_copy_dtype(src_dtype) || !valid_copy_dtype(dst_dtype)) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT, "[copy] unknown dtype %d -> %d", src_dtype, dst_dtype);
+  }
+  if (ndim < 0 || (ndim > 0 && (shape == nullptr || src_strides == nullptr))) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[copy] shape and source strides are required");
+  }
+  size_t n = 1;
+  for (int d = 0; d < ndim; ++d) {
+    if (shape[d] < 0) {
+      return fail(MLXROCM_INVALID_ARGUMENT, "[copy] negative extent");
+    }
+    n *= static_cast<size_t>(shape[d]);
+  }
+  if (n == 0) {
+    return MLXROCM_OK;
+  }
+  if (src == nullptr || dst == nullptr) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[copy] null pointer");
+  }
+
+  // Row-contiguous destination strides when none are given.
+  int64_t dense[64];
+  if (ndim > 64) {
+    return fail(MLXROCM_UNSUPPORTED, "[copy] %d dimensions", ndim);
+  }
+  if (dst_strides == nullptr) {
+    int64_t run = 1;
+    for (int d = ndim - 1; d >= 0; --d) {
+      dense[d] = run;
+      run *= shape[d];
+    }
+    dst_strides = dense;
+  }
+
+  // Drop extent-1 dimensions and merge neighbours that both sides walk as one
+  // run (outer stride == inner stride * inner extent).
+  StridedShape a;
+  a.ndim = 0;
+  int64_t cs[64], css[64], cds[64];
+  int nd = 0;
+  for (int d = 0; d < ndim; ++d) {
+    if (shape[d] == 1) {
+      continue;
+    }
+    if (nd > 0 && css[nd - 1] == src_strides[d] * shape[d] &&
+        cds[nd - 1] == dst_strides[d] * shape[d]) {
+      cs[nd - 1] *= shape[d];
+      css[nd - 1] = src_strides[d];
+      cds[nd - 1] = dst_strides[d];
+    } else {
+      cs[nd] = shape[d];
+      css[nd] = src_strides[d];
+      cds[nd] = dst_strides[d];
+      ++nd;
+    }
+  }
+  if (nd == 0) { // a single element
+    cs[0] = 1;
+    css[0] = 0;
+    cds[0] = 0;
+    nd = 1;
+  }
+  if (nd > kMaxDims) {
+    return fail(
+        MLXROCM_UNSUPPORTED,
+        "[copy] %d dimensions remain after merging; at most %d are supported",
+        nd,
+        kMaxDims);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (nd == 1 && css[0] == 1 && cds[0] == 1) {
+    return mlxrocm_copy_contiguous(src, src_dtype, dst, dst_dtype, n, 0, stream);
+  }
+  if (nd == 1 && css[0] == 0 && cds[0] == 1) {
+    return mlxrocm_copy_contiguous(src, src_dtype, dst, dst_dtype, n, 1, stream);
+  }
+  a.ndim = nd;
+  for (int d = 0; d < kMaxDims; ++d) {
+    a.shape[d] = d < nd ? cs[d] : 1;
+    a.src_stride[d] = d < nd ? css[d] : 0;
+    a.dst_stride[d] = d < nd ? cds[d] : 0;
+  }
+  const bool wide = n > 0xffffffffull;
+  return with_type(src_dtype, [&](auto st) {
+    using S = decltype(st);
+    return with_type(dst_dtype, [&](auto dt) {
+      using D = decltype(dt);
+      return launch_strided<S, D>(src, dst, a, n, wide, s);
+    });
+  });
+}

@@ -352,6 +352,15 @@ extern "C" int mlxrocm_event_create(mlxrocm_event_t* event) {
   *event = e;
   return MLXROCM_OK;
 }
+extern "C" int mlxrocm_event_create_blocking(mlxrocm_event_t* event) {
+  if (event == nullptr) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[event_create] null result pointer");
+  }
+  hipEvent_t e = nullptr;
+  MLXROCM_HIP_TRY(hipEventCreateWithFlags(&e, hipEventBlockingSync | hipEventDisableTiming));
+  *event = e;
+  return MLXROCM_OK;
+}
 extern "C" int mlxrocm_event_destroy(mlxrocm_event_t event) {
   if (event != nullptr) {
     MLXROCM_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));

@@ -17,6 +17,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
+from ._copy import astype as _astype, contiguous as _contiguous
 
 _DTYPE_CODE = {
     torch.float32: _lib.FLOAT32,
@@ -179,7 +180,7 @@ def quantize(
     _check_affine_params("quantize", group_size, bits)
     _require_gpu("quantize", w)
     lib = _lib.load()
-    w = w.contiguous()  # ensure_row_contiguous, cpu/quantized.cpp:1233
+    w = _contiguous(w)  # ensure_row_contiguous, cpu/quantized.cpp:1233
     lead = tuple(w.shape[:-1])
     K = w.shape[-1]
     wq = torch.empty(lead + (K * bits // 32,), dtype=torch.uint32, device=w.device)
@@ -240,9 +241,9 @@ def dequantize(
     # The affine step runs in scales' dtype (mlx/ops.cpp:5322-5323); biases are
     # promoted to it the way the Add primitive would.
     sdt = torch.promote_types(scales.dtype, biases.dtype)
-    w = w.contiguous()
-    scales = scales.to(sdt).contiguous()
-    biases = biases.to(sdt).contiguous()
+    w = _contiguous(w)
+    scales = _contiguous(_astype(scales, sdt))
+    biases = _contiguous(_astype(biases, sdt))
     out = torch.empty(tuple(w.shape[:-1]) + (out_size,), dtype=sdt, device=w.device)
     _lib.check(
         lib.mlxrocm_affine_dequantize(
@@ -250,17 +251,16 @@ def dequantize(
             out.numel(), group_size, bits, _DTYPE_CODE[sdt], _stream_ptr(w),
         )
     )
-    return out if out_type == sdt else out.to(out_type)  # astype, :5502-5505
+    return _astype(out, out_type)  # astype, :5502-5505
 
 
 def _dense_batches(t: torch.Tensor, batch_shape: Tuple[int, ...]):
     """Expand the leading dims of ``t`` to ``batch_shape``; returns the tensor
     and its batch stride in elements (0 when one matrix serves every batch)."""
     if t.dim() == 2:
-        return (t if _last_two_dense(t) else t.contiguous()), 0
+        return (t if _last_two_dense(t) else _contiguous(t)), 0
     t = t.expand(*batch_shape, *t.shape[-2:])
-    if not t.is_contiguous():
-        t = t.contiguous()
+    t = _contiguous(t)
     return t, t.shape[-1] * t.shape[-2]
 
 
@@ -300,9 +300,9 @@ def quantized_swiglu(
     M = 1
     for d in x.shape[:-1]:
         M *= d
-    xb = x.to(dtype).reshape(M, K).contiguous()
-    sg, bg, su, bu = (t.to(dtype).contiguous() for t in (sg, bg, su, bu))
-    wg, wu = wg.contiguous(), wu.contiguous()
+    xb = _contiguous(_astype(x, dtype)).reshape(M, K)
+    sg, bg, su, bu = (_contiguous(_astype(t, dtype)) for t in (sg, bg, su, bu))
+    wg, wu = _contiguous(wg), _contiguous(wu)
     code = _DTYPE_CODE[dtype]
     ws_bytes = lib.mlxrocm_qmm_swiglu_workspace_size(M, n_gate, code)
     workspace = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=x.device)
@@ -343,9 +343,9 @@ def quantized_matmul(
     _require_gpu("quantized_matmul", x, w, scales, biases)
     lib = _lib.load()
 
-    x = x.to(dtype)
-    scales = scales.to(dtype)
-    biases = biases.to(dtype)
+    x = _astype(x, dtype)
+    scales = _astype(scales, dtype)
+    biases = _astype(biases, dtype)
     K = x.shape[-1]
     M = x.shape[-2] if x.dim() > 1 else 1
     x_batch = tuple(x.shape[:-2]) if x.dim() > 2 else ()
@@ -363,7 +363,7 @@ def quantized_matmul(
     for d in batch_shape:
         L *= d
     xb = x.reshape(1, M, K) if x.dim() <= 2 else x.expand(*batch_shape, M, K)
-    xb = xb.contiguous()
+    xb = _contiguous(xb)
     if w.dim() == 2 and L > 1:
         # one weight matrix for every batch entry: the batch folds into the rows
         # of x, so W is read once for all of them (the GPU backends do the same,
@@ -402,7 +402,7 @@ def _indices_or_default(tag, indices, t):
             raise ValueError(
                 f"{tag} Got indices with invalid dtype. Indices must be integral."
             )
-        return indices.to(torch.int64)
+        return _astype(indices, torch.int64)
     shape = tuple(t.shape[:-2])
     total = 1
     for d in shape:
@@ -444,28 +444,28 @@ def gather_qmm(
     lhs, rhs = torch.broadcast_tensors(lhs, rhs)
     right_sorted = bool(sorted_indices) and lhs_indices is None
 
-    x = x.to(out_type)
-    scales = scales.to(out_type)
-    biases = biases.to(out_type)
+    x = _astype(x, out_type)
+    scales = _astype(scales, out_type)
+    biases = _astype(biases, out_type)
     M, K = x.shape[-2], x.shape[-1]
-    xb = x.contiguous().reshape(-1, M, K)
+    xb = _contiguous(x).reshape(-1, M, K)
     # Only the trailing matrices must be dense; a sliced expert stack keeps its
     # stride (python/tests/test_quantized.py:1567-1593).
     def experts(t):
         if t.dim() == 3 and _last_two_dense(t):
             return t, t.stride(0)
-        t = t.contiguous().reshape(-1, *t.shape[-2:])
+        t = _contiguous(t).reshape(-1, *t.shape[-2:])
         return t, t.shape[-1] * t.shape[-2]
     wb, w_stride = experts(w)
     sb, sb_stride = experts(scales)
     bb, bb_stride = experts(biases)
     if bb_stride != sb_stride:
-        bb = bb.contiguous()
-        sb = sb.contiguous()
+        bb = _contiguous(bb)
+        sb = _contiguous(sb)
         sb_stride = sb.shape[-1] * sb.shape[-2]
     n_idx = lhs.numel()
-    lhs_u = lhs.reshape(-1).to(torch.uint32).contiguous() if n_idx else lhs.reshape(-1)
-    rhs_u = rhs.reshape(-1).to(torch.uint32).contiguous() if n_idx else rhs.reshape(-1)
+    lhs_u = _astype(_contiguous(lhs).reshape(-1), torch.uint32) if n_idx else lhs.reshape(-1)
+    rhs_u = _astype(_contiguous(rhs).reshape(-1), torch.uint32) if n_idx else rhs.reshape(-1)
     out = torch.empty(tuple(lhs.shape) + (M, w_outer), dtype=out_type, device=x.device)
     code = _DTYPE_CODE[out_type]
     ws_bytes = lib.mlxrocm_gather_qmm_workspace_size(
