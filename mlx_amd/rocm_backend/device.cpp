@@ -1,74 +1,12 @@
 // device.cpp -- see device.h.
 #include "device.h"
 
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
 
 namespace mlx::core::rocm {
-
-void check(int status) {
-  if (status == MLXROCM_OK) {
-    return;
-  }
-  std::string msg = mlxrocm_last_error();
-  if (status == MLXROCM_INVALID_ARGUMENT) {
-    throw std::invalid_argument(msg);
-  }
-  throw std::runtime_error(msg);
-}
-
-CommandEncoder::CommandEncoder(Stream s) : mlx_stream_(s) {
-  check(mlxrocm_stream_create(&stream_));
-}
-
-CommandEncoder::~CommandEncoder() {
-  // Devices are torn down at process exit in an unspecified order: drop the
-  // bookkeeping, do not call into the runtime.
-}
-
-void CommandEncoder::commit() {
-  reap(/* wait */ false);
-  if (!needs_commit()) {
-    return;
-  }
-  Batch b;
-  check(mlxrocm_event_create(&b.event));
-  check(mlxrocm_event_record(b.event, stream_));
-  b.arrays = std::move(pending_);
-  b.handlers = std::move(handlers_);
-  pending_.clear();
-  handlers_.clear();
-  in_flight_.push_back(std::move(b));
-}
-
-void CommandEncoder::reap(bool wait) {
-  while (!in_flight_.empty()) {
-    Batch& b = in_flight_.front();
-    if (wait) {
-      check(mlxrocm_event_synchronize(b.event));
-    } else {
-      int done = mlxrocm_event_query(b.event);
-      if (done < 0) {
-        check(done);
-      }
-      if (done == 0) {
-        return; // batches complete in order
-      }
-    }
-    for (auto& fn : b.handlers) {
-      fn();
-    }
-    check(mlxrocm_event_destroy(b.event));
-    in_flight_.pop_front(); // releases the retained arrays
-  }
-}
-
-void CommandEncoder::synchronize() {
-  commit();
-  check(mlxrocm_stream_synchronize(stream_));
-  reap(/* wait */ true);
-}
 
 namespace {
 
@@ -117,7 +55,11 @@ CommandEncoder& get_command_encoder(Stream s) {
 }
 
 void clear_encoders() {
-  thread_encoders().clear();
+  auto& local = thread_encoders();
+  for (auto& [index, encoder] : local) {
+    encoder->synchronize(); // so that each completion thread can be joined
+  }
+  local.clear();
 }
 
 } // namespace mlx::core::rocm

@@ -1,32 +1,26 @@
-// event.cpp -- mlx::core::Event over HIP events of the C ABI
+// event.cpp -- mlx::core::Event for the ROCm backend
 // (interface: mlx/event.h:12-90; CUDA counterpart: mlx/backend/cuda/event.cu:330-409).
 //
-// A GPU-stream event is a HIP event recorded behind the stream's work; a
-// CPU-stream signal/wait runs as a task of that stream's scheduler thread, as
-// the other backends do.
+// The state is a rocm::Signal (signal.h): a host counter that says a signal has
+// been issued, plus a HIP event when it was issued on a GPU stream.  A waiter
+// that comes first blocks until the signal exists; a CPU-stream producer or
+// consumer runs as a task of that stream's scheduler thread, as in the other
+// backends.
 #include <atomic>
-#include <stdexcept>
 
 #include "mlx/event.h"
 #include "mlx/scheduler.h"
 
 #include "device.h"
+#include "signal.h"
 
 namespace mlx::core {
 
 namespace rocm {
 
 struct EventImpl {
-  mlxrocm_event_t event{nullptr};
-  std::atomic<bool> recorded{false};
+  Signal signal;
   std::atomic<Error*> error{nullptr};
-
-  EventImpl() {
-    check(mlxrocm_event_create(&event));
-  }
-  ~EventImpl() {
-    (void)mlxrocm_event_destroy(event);
-  }
 };
 
 } // namespace rocm
@@ -37,51 +31,34 @@ Event::Event(Stream s) : stream_(s) {
 
 void Event::wait() {
   check_error();
-  auto& ev = cast<rocm::EventImpl>();
-  if (ev.recorded.load()) {
-    rocm::check(mlxrocm_event_synchronize(ev.event));
-  }
+  cast<rocm::EventImpl>().signal.wait(value());
 }
 
 void Event::wait(Stream s) {
   if (s.device == Device::cpu) {
+    // The CPU stream's thread blocks, not the caller.
     scheduler::enqueue(s, [*this]() mutable { wait(); });
     return;
   }
-  auto& ev = cast<rocm::EventImpl>();
-  if (ev.recorded.load()) {
-    auto& enc = rocm::get_command_encoder(s);
-    rocm::check(mlxrocm_event_wait(ev.event, enc.stream()));
-  }
+  cast<rocm::EventImpl>().signal.wait_on_stream(
+      rocm::get_command_encoder(s).stream(), value());
 }
 
 void Event::signal(Stream s) {
-  auto& ev = cast<rocm::EventImpl>();
   if (s.device == Device::cpu) {
-    // Recorded on the null stream from the CPU stream's thread: everything the
-    // CPU task produced is already in host memory at that point.
+    // Runs after the CPU tasks queued so far: what they produced is in host
+    // memory by then.
     scheduler::enqueue(s, [*this]() mutable {
-      auto& e = cast<rocm::EventImpl>();
-      rocm::check(mlxrocm_event_record(e.event, nullptr));
-      e.recorded.store(true);
+      cast<rocm::EventImpl>().signal.signal_from_host(value());
     });
     return;
   }
-  auto& enc = rocm::get_command_encoder(s);
-  rocm::check(mlxrocm_event_record(ev.event, enc.stream()));
-  ev.recorded.store(true);
+  cast<rocm::EventImpl>().signal.signal_on_stream(
+      rocm::get_command_encoder(s).stream(), value());
 }
 
 bool Event::is_signaled() const {
-  auto& ev = cast<rocm::EventImpl>();
-  if (!ev.recorded.load()) {
-    return false;
-  }
-  int done = mlxrocm_event_query(ev.event);
-  if (done < 0) {
-    rocm::check(done);
-  }
-  return done == 1;
+  return cast<rocm::EventImpl>().signal.is_signaled(value());
 }
 
 std::atomic<Error*>& Event::error() {

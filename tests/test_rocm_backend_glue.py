@@ -47,6 +47,38 @@ def test_glue_defines_the_three_eval_gpu_bodies():
         assert sig in text
 
 
+@pytest.mark.skipif(not (MLX_TREE / "mlx" / "primitives.h").exists(),
+                    reason="MLX source tree not present")
+def test_every_primitive_has_exactly_one_eval_gpu():
+    """Each primitive class MLX declares gets its eval_gpu from exactly one of:
+    the glue's kernels (quantized.cpp), the glue's throwing stubs
+    (primitives.cpp), MLX's shared data-movement file, or an inline definition
+    in MLX's headers -- so that libmlx would link with neither a missing nor a
+    duplicate symbol."""
+    import re
+    declared = {}
+    for header in ("primitives.h", "fast_primitives.h", "distributed/primitives.h"):
+        text = (MLX_TREE / "mlx" / header).read_text()
+        for m in re.finditer(r"class\s+(?:MLX_API\s+)?(\w+)\s*(?:final\s*)?:\s*public\s+\w+[^{]*\{", text):
+            start = m.end()
+            nxt = re.search(r"\nclass\s", text[start:])
+            body = text[start:start + nxt.start()] if nxt else text[start:]
+            decl = re.search(r"void\s+eval_gpu\s*\([^)]*\)\s*(?:override)?\s*(;|\{)", body)
+            if decl and decl.group(1) == ";":
+                declared[m.group(1)] = header
+    stubs = (GLUE / "primitives.cpp").read_text()
+    stubbed = set(re.findall(r"ROCM_NO_(?:UNARY|MULTI)\((\w+)\)", stubs)) - {"cls"}
+    ours = set(re.findall(r"void (?:fast::)?(\w+)::eval_gpu\(", (GLUE / "quantized.cpp").read_text()))
+    shared = set(re.findall(r"void (\w+)::eval_gpu\(",
+                            (MLX_TREE / "mlx" / "backend" / "gpu" / "primitives.cpp").read_text()))
+    assert not (stubbed & ours) and not (stubbed & shared) and not (ours & shared)
+    provided = stubbed | ours | shared
+    missing = sorted(set(declared) - provided)
+    extra = sorted(provided - set(declared))
+    assert not missing, f"no eval_gpu for: {missing}"
+    assert not extra, f"eval_gpu for unknown classes: {extra}"
+
+
 def test_glue_calls_only_declared_abi_symbols():
     import re
     header = (ROOT / "include" / "mlx_rocm_qmm.h").read_text()
