@@ -55,6 +55,34 @@ def build(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+GLUE = os.path.join(HERE, "rocm_backend")
+GLUE_TEST_DIR = os.path.join(os.path.dirname(HERE), "tests", "rocm_backend")
+GLUE_GPU_TEST = os.path.join(GLUE_TEST_DIR, "_build", "gpu_core_test")
+
+
+def build_glue_gpu_test(verbose: bool = False) -> str:
+    """Link the backend's host cores (no MLX headers needed) with the HIP
+    library into the executable that the GPU test of the glue runs."""
+    os.makedirs(os.path.dirname(GLUE_GPU_TEST), exist_ok=True)
+    rocm_lib = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
+    cmd = [
+        "g++", "-std=c++20", "-O1", "-g", "-Wall",
+        "-I", INCLUDE, "-I", GLUE,
+        os.path.join(GLUE_TEST_DIR, "gpu_core_test.cpp"),
+        *[os.path.join(GLUE, f) for f in ("completion.cpp", "signal.cpp", "residency.cpp")],
+        "-o", GLUE_GPU_TEST, "-pthread",
+        "-L", LIB_DIR, "-lmlx_rocm_qmm",
+        "-Wl,-rpath,$ORIGIN/../../../mlx_amd/lib", f"-Wl,-rpath-link,{rocm_lib}",
+    ]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building the glue's GPU test failed:\n{proc.stdout}\n{proc.stderr}")
+    if verbose:
+        print("built", GLUE_GPU_TEST)
+    return GLUE_GPU_TEST
+
+
 if __name__ == "__main__":
     build(verbose=True)
+    build_glue_gpu_test(verbose=True)
     sys.exit(0)
