@@ -82,7 +82,26 @@ def build_glue_gpu_test(verbose: bool = False) -> str:
     return GLUE_GPU_TEST
 
 
+PROBE_DIR = os.path.join(os.path.dirname(HERE), "tests", "probe")
+READ_PROBE = os.path.join(PROBE_DIR, "_build", "read_probe")
+
+
+def build_read_probe(verbose: bool = False) -> str:
+    """The read-only HBM probe that the decode kernel's duration is judged against."""
+    os.makedirs(os.path.dirname(READ_PROBE), exist_ok=True)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           os.path.join(PROBE_DIR, "read_probe.hip"), "-o", READ_PROBE]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building the read probe failed:\n{proc.stdout}\n{proc.stderr}")
+    if verbose:
+        print("built", READ_PROBE)
+    return READ_PROBE
+
+
 if __name__ == "__main__":
     build(verbose=True)
     build_glue_gpu_test(verbose=True)
+    build_read_probe(verbose=True)
     sys.exit(0)

@@ -7,7 +7,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libmlx_rocm_qmm.so")
+# MLX_ROCM_QMM_LIBRARY names another build of the library (e.g. one under test).
+LIB_PATH = os.environ.get("MLX_ROCM_QMM_LIBRARY") or os.path.join(HERE, "lib", "libmlx_rocm_qmm.so")
 
 OK = 0
 INVALID_ARGUMENT = -1

@@ -50,10 +50,14 @@ namespace {
 // which LDS bytes they write), and any wait it inserted for the W words would
 // also wait for the younger x loads (vmcnt completes in order).  So all loads
 // of the loop are inline assembly, whose results the compiler believes ready at
-// once, and the loop waits for them itself, once per step, right before the
-// barrier: `s_waitcnt vmcnt(4)` leaves exactly that step's four x loads in
-// flight.  Nothing may read a RawWords / raw value between its load and that
-// wait; every slot of the loop ends in a scheduling barrier, so no use moves up.
+// once, and the loop waits for them itself, twice per step.  Right before the
+// barrier, a wait that leaves only the step's own loads in flight (the W words
+// fetched in slot 0 and the four x loads): the x loads of the step before have
+// then landed.  At the end of the step `s_waitcnt vmcnt(4)`: the W words are
+// older than the four x loads, so they have arrived -- a whole step after they
+// were asked for -- and the x loads stay in flight.  Nothing may read a
+// RawWords / raw value between its load and that second wait; every slot of
+// the loop ends in a scheduling barrier, so no use moves up.
 typedef uint32_t raw_u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t raw_u32x3 __attribute__((ext_vector_type(3)));
 typedef uint32_t raw_u32x4 __attribute__((ext_vector_type(4)));
@@ -162,10 +166,17 @@ constexpr int kOutPad = 8; // elements of padding per row of the staged y tile
 // NS = 8 NT slots.  Everything that writes LDS has to be issued before the
 // barrier in slot NS - 14, so the 16 dequantization pairs are spread over the
 // first NS - 16 slots: pair q goes to slot q (NS - 16) / 16, the 16-byte store
-// of pairs 4r..4r+3 to the slot after pair 4r+3, the x store + refetch of row
-// block i to slot 4i + 1 and the packed-W fetch to slot 0.
+// of pairs 4r..4r+3 to the slot after pair 4r+3, the direct-to-LDS load of x
+// row block i to slot xdma_slot(i) and the packed-W fetch to slot 0.
 constexpr int pair_slot(int q, int ns) {
   return q * (ns - 16) / 16;
+}
+// The four direct-to-LDS loads of an x tile are spread evenly over the slots
+// before the barrier: bunched together they compete with the fragment reads for
+// the LDS, and every one of them has to be issued before the barrier's wait
+// counts it.
+constexpr int xdma_slot(int i, int ns) {
+  return 1 + i * (ns - 17) / 3;
 }
 constexpr int pair_at(int m, int ns) {
   for (int q = 0; q < 16; ++q) {
@@ -364,6 +375,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   uint32_t sreg, breg, snext, bnext;             // one scale / bias as loaded
   uint2 swn, bwn;                                // WN: four 16-bit values each
   RawTuple<2> swn_next, bwn_next;
+  // load instructions one QMM_LOAD_W issues (vmcnt counts instructions)
+  constexpr int kWLoads = WN ? 6 : (BITS > 4 ? 2 : 1) + 2;
   auto wn_value = [](const uint2& v, int j) {
     const uint32_t word = j < 2 ? v.x : v.y;
     return to_f32(__builtin_bit_cast(TS, static_cast<
@@ -618,22 +631,22 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     }                                                                            \
     /* x tile tt + 2 into the stage that the barrier of the previous step freed; \
        these are the last loads issued before this step's barrier */            \
-    if constexpr ((m) == 1) {                                                    \
+    if constexpr ((m) == xdma_slot(0, kNS)) {                                    \
       QMM_DMA_X1(xs_new, kx, 0, xoff0);                                          \
     }                                                                            \
-    if constexpr ((m) == 5) {                                                    \
+    if constexpr ((m) == xdma_slot(1, kNS)) {                                    \
       QMM_DMA_X1(xs_new, kx, 1, xoff1);                                          \
     }                                                                            \
-    if constexpr ((m) == 9) {                                                    \
+    if constexpr ((m) == xdma_slot(2, kNS)) {                                    \
       QMM_DMA_X1(xs_new, kx, 2, xoff2);                                          \
     }                                                                            \
-    if constexpr ((m) == 13) {                                                   \
+    if constexpr ((m) == xdma_slot(3, kNS)) {                                    \
       QMM_DMA_X1(xs_new, kx, 3, xoff3);                                          \
     }                                                                            \
     if constexpr ((m) == kNS - 14) {                                             \
-      /* all but this step's four x loads have completed: x tile tt + 1 is in */ \
-      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");                           \
-      QMM_PIN_W();                                                               \
+      /* everything but this step's own loads has completed: x tile tt + 1 is   \
+         in LDS */                                                               \
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWLoads + 4) : "memory");         \
       __syncthreads();                                                           \
     }                                                                            \
     __builtin_amdgcn_sched_barrier(0);                                           \
@@ -666,6 +679,11 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     __builtin_amdgcn_sched_barrier(0);                                           \
     QMM_SLOTS8(0, P) QMM_SLOTS8(8, P) QMM_SLOTS8(16, P) QMM_SLOTS8(24, P)        \
     QMM_SLOTS8(32, P) QMM_SLOTS8(40, P) QMM_SLOTS8(48, P) QMM_SLOTS8(56, P)      \
+    /* the packed W fetched in slot 0 is older than the four x loads: it has    \
+       had the whole step to arrive */                                          \
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");                             \
+    QMM_PIN_W();                                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                           \
     QMM_ROTATE_W();                                                              \
     {                                                                            \
       const int freed = xs_cur;                                                  \
