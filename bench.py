@@ -28,9 +28,9 @@ BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes, scaled by
 # a copy of known size (profiles/qmv_stream_4bit_g64_bf16_14336x4096.md and
 # profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md).
-QMV_TRAFFIC_BYTES = 33224063
+QMV_TRAFFIC_BYTES = 33220710
 QMV_TRAFFIC_SOURCE = "profiles/qmv_stream_4bit_g64_bf16_14336x4096.md"
-QMM_T_TRAFFIC_BYTES = 260219533
+QMM_T_TRAFFIC_BYTES = 260195251
 QMM_T_TRAFFIC_SOURCE = "profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md"
 
 N, K = 14336, 4096
@@ -431,11 +431,29 @@ def main() -> int:
     g = torch.Generator().manual_seed(0)
     x_cpu = torch.randn((1, K), generator=g, dtype=torch.float32).to(dt)
     x = x_cpu.to(dev)
+    # The ring lives in one allocation made before anything else, each weight at
+    # a 2 MiB boundary: how the driver backs many separate allocations (page
+    # sizes, placement) differs from box to box and showed up as a spread in the
+    # streaming rate.
+    w_words, sb_elems = N * K * BITS // 32, N * K // GS
+    slot = -(-(w_words * 4 + 2 * sb_elems * 2) // (2 << 20)) * (2 << 20)
+    pool = torch.empty(RING * slot + (2 << 20), dtype=torch.uint8, device=dev)
+    pool = pool[(-pool.data_ptr()) % (2 << 20):]
     ring = []
     for i in range(RING):
         w = (torch.randn((N, K), generator=g, dtype=torch.float32) * 0.02).to(dt).to(dev)
-        ring.append(mlx_amd.quantize(w, GS, BITS))
-        del w
+        wq, s, b = mlx_amd.quantize(w, GS, BITS)
+        base = pool[i * slot:(i + 1) * slot]
+        wq_v = base[:w_words * 4].view(torch.uint32).view(N, -1)
+        s_v = base[w_words * 4:w_words * 4 + sb_elems * 2].view(dt).view(N, -1)
+        b_v = base[w_words * 4 + sb_elems * 2:w_words * 4 + sb_elems * 4].view(dt).view(N, -1)
+        wq_v.copy_(wq)
+        s_v.copy_(s)
+        b_v.copy_(b)
+        ring.append((wq_v, s_v, b_v))
+        del w, wq, s, b
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
     out = torch.empty((1, N), dtype=dt, device=dev)
     code = _lib.BFLOAT16
     result = {}
