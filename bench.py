@@ -377,6 +377,38 @@ def sweep(torch, mlx_amd, dev) -> list:
         blocks = torch.randint(0, 256, (n_blocks * block_bytes,), generator=g, dtype=torch.uint8).to(dev)
         ms = timed(lambda i: gguf.repack(blocks, type_id, (14336, 4096)))
         add("gguf", f"repack {name} [14336,4096] -> affine g32", ms, nbytes=n_blocks * (block_bytes + out_bytes))
+
+    # element copies around the matmuls (C-ABI launches into a preallocated output)
+    from mlx_amd import _copy, _lib
+    import ctypes
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    n = 64 << 20
+    src = torch.randn(n, generator=torch.Generator(device=dev).manual_seed(1), device=dev,
+                      dtype=torch.float32).to(torch.bfloat16)
+    dst = torch.empty(n, dtype=torch.float32, device=dev)
+    code = _copy.DTYPE_CODE
+    ms = timed(lambda i: _lib.check(lib.mlxrocm_copy_contiguous(
+        src.data_ptr(), code[torch.bfloat16], dst.data_ptr(), code[torch.float32], n, 0, stream)))
+    add("copy", "contiguous bfloat16 -> float32, 64 Mi elements", ms, nbytes=n * 6)
+    back = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    ms = timed(lambda i: _lib.check(lib.mlxrocm_copy_contiguous(
+        dst.data_ptr(), code[torch.float32], back.data_ptr(), code[torch.bfloat16], n, 0, stream)))
+    add("copy", "contiguous float32 -> bfloat16, 64 Mi elements", ms, nbytes=n * 6)
+    arr = lambda v: (ctypes.c_int64 * len(v))(*v)
+    ms = timed(lambda i: _lib.check(lib.mlxrocm_copy_strided(
+        src.data_ptr(), code[torch.bfloat16], arr((1, 8192)), back.data_ptr(), code[torch.bfloat16],
+        None, 2, arr((8192, 8192)), stream)))
+    add("copy", "transpose of bfloat16 [8192,8192] into rows (strided source)", ms, nbytes=n * 4)
+    ms = timed(lambda i: _lib.check(lib.mlxrocm_copy_strided(
+        src.data_ptr(), code[torch.bfloat16], arr((2 * 4096, 1)), back.data_ptr(), code[torch.bfloat16],
+        None, 2, arr((8192, 4096)), stream)))
+    add("copy", "left half of bfloat16 [8192,8192] rows into [8192,4096] (row-strided source)", ms,
+        nbytes=8192 * 4096 * 4)
+    one = torch.ones(1, dtype=torch.float32, device=dev)
+    ms = timed(lambda i: _lib.check(lib.mlxrocm_copy_contiguous(
+        one.data_ptr(), code[torch.float32], back.data_ptr(), code[torch.bfloat16], n, 1, stream)))
+    add("copy", "fill bfloat16, 64 Mi elements", ms, nbytes=n * 2)
     return rows
 
 

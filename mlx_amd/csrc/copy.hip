@@ -24,6 +24,11 @@ struct complex64 {
   float re;
   float im;
 };
+// Sixteen opaque bytes: the element of a same-type copy whose innermost runs
+// are contiguous and aligned on both sides.
+struct alignas(16) bytes16 {
+  uint32_t w[4];
+};
 
 template <int DT> struct TypeOf;
 template <> struct TypeOf<MLXROCM_FLOAT32> { using type = float; };
@@ -378,6 +383,34 @@ extern "C" int mlxrocm_copy_strided(
   if (nd == 1 && css[0] == 0 && cds[0] == 1) {
     return mlxrocm_copy_contiguous(src, src_dtype, dst, dst_dtype, n, 1, stream);
   }
+  // A same-type copy moves bytes: when both sides walk the innermost dimension
+  // contiguously, widen the element to 16, 8 or 4 bytes (fewer, wider accesses)
+  // as far as extents, strides and base addresses allow.
+  size_t item = kItemSize[src_dtype];
+  int wide_code = -1; // 16 bytes when -2
+  if (src_dtype == dst_dtype && css[nd - 1] == 1 && cds[nd - 1] == 1) {
+    for (size_t bytes : {size_t(16), size_t(8), size_t(4)}) {
+      if (bytes <= item) {
+        break;
+      }
+      const int64_t v = static_cast<int64_t>(bytes / item);
+      bool ok = cs[nd - 1] % v == 0 && reinterpret_cast<uintptr_t>(src) % bytes == 0 &&
+          reinterpret_cast<uintptr_t>(dst) % bytes == 0;
+      for (int d = 0; ok && d < nd - 1; ++d) {
+        ok = css[d] % v == 0 && cds[d] % v == 0;
+      }
+      if (ok) {
+        cs[nd - 1] /= v;
+        for (int d = 0; d < nd - 1; ++d) {
+          css[d] /= v;
+          cds[d] /= v;
+        }
+        n /= static_cast<size_t>(v);
+        wide_code = bytes == 16 ? -2 : (bytes == 8 ? MLXROCM_UINT64 : MLXROCM_UINT32);
+        break;
+      }
+    }
+  }
   a.ndim = nd;
   for (int d = 0; d < kMaxDims; ++d) {
     a.shape[d] = d < nd ? cs[d] : 1;
@@ -385,6 +418,12 @@ extern "C" int mlxrocm_copy_strided(
     a.dst_stride[d] = d < nd ? cds[d] : 0;
   }
   const bool wide = n > 0xffffffffull;
+  if (wide_code == -2) {
+    return launch_strided<bytes16, bytes16>(src, dst, a, n, wide, s);
+  }
+  if (wide_code >= 0) {
+    src_dtype = dst_dtype = wide_code;
+  }
   return with_type(src_dtype, [&](auto st) {
     using S = decltype(st);
     return with_type(dst_dtype, [&](auto dt) {

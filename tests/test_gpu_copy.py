@@ -187,6 +187,21 @@ def test_many_dimensions_merge_or_are_refused():
     assert torch.equal(got.cpu(), perm.contiguous())
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.int64],
+                         ids=lambda d: str(d).split(".")[-1])
+def test_row_slices_take_the_widened_path_and_its_fallbacks(dtype):
+    """Same-type copies whose rows are contiguous move 16, 8 or 4 bytes per lane
+    when extents, strides and addresses allow, and single elements otherwise: every
+    alignment of the column window must give the same bytes."""
+    src = _source(dtype, 64 * 96, seed=21).reshape(64, 96)
+    dev = src.to(DEV)
+    for lo, hi in ((0, 64), (16, 80), (8, 72), (4, 36), (2, 50), (1, 33), (3, 96)):
+        got = _copy.contiguous(dev[:, lo:hi])
+        assert _bytes(got) == _bytes(src[:, lo:hi].contiguous()), (lo, hi)
+        got = _copy.contiguous(dev[5:61:3, lo:hi])
+        assert _bytes(got) == _bytes(src[5:61:3, lo:hi].contiguous()), (lo, hi)
+
+
 def test_fill_broadcasts_one_device_scalar():
     like = torch.empty((33, 77), dtype=torch.bfloat16, device=DEV)
     value = torch.tensor([1.2345], dtype=torch.float32, device=DEV)
