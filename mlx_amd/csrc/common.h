@@ -17,6 +17,20 @@ constexpr int kWaveSize = 64;
 int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t err, const char* what);
 
+// A roctx range around one entry point of the C ABI, so that a profiler's
+// marker trace shows which operator call a kernel belongs to.  The marker
+// library is looked up at the first call; without it the range is a no-op.
+class ApiRange {
+ public:
+  explicit ApiRange(const char* name);
+  ~ApiRange();
+  ApiRange(const ApiRange&) = delete;
+  ApiRange& operator=(const ApiRange&) = delete;
+
+ private:
+  bool open_;
+};
+
 #define MLXROCM_HIP_TRY(expr)                    \
   do {                                           \
     hipError_t err__ = (expr);                   \

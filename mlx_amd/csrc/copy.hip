@@ -270,6 +270,7 @@ extern "C" int mlxrocm_copy_contiguous(
     size_t n,
     int broadcast_scalar,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_copy_contiguous");
   if (!valid_copy_dtype(src_dtype) || !valid_copy_dtype(dst_dtype)) {
     return fail(
         MLXROCM_INVALID_ARGUMENT, "[copy] unknown dtype %d -> %d", src_dtype, dst_dtype);
@@ -306,6 +307,7 @@ extern "C" int mlxrocm_copy_strided(
     int ndim,
     const int64_t* shape,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_copy_strided");
   if (!valid_copy_dtype(src_dtype) || !valid_copy_dtype(dst_dtype)) {
     return fail(
         MLXROCM_INVALID_ARGUMENT, "[copy] unknown dtype %d -> %d", src_dtype, dst_dtype);

@@ -146,6 +146,7 @@ extern "C" int mlxrocm_gguf_repack(
     size_t n_blocks,
     int ggml_type,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_gguf_repack");
   using namespace mlxrocm;
   if (ggml_type != MLXROCM_GGML_Q4_0 && ggml_type != MLXROCM_GGML_Q4_1 &&
       ggml_type != MLXROCM_GGML_Q8_0) {

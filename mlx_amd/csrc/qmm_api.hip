@@ -562,6 +562,7 @@ extern "C" int mlxrocm_qmm_swiglu(
     int bits,
     int dtype,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_qmm_swiglu");
   int rc = check_shape("quantized_swiglu", M, N, K, 1, group_size, bits, dtype, 1);
   if (rc != MLXROCM_OK) {
     return rc;
@@ -751,6 +752,7 @@ extern "C" int mlxrocm_qmm(
     void* workspace,
     size_t workspace_bytes,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_qmm");
   Scratch sc;
   sc.base = static_cast<char*>(workspace);
   sc.bytes = workspace != nullptr ? workspace_bytes : 0;
@@ -818,6 +820,7 @@ extern "C" int mlxrocm_qmm_static(
     int dtype,
     int transpose,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_qmm_static");
   void* region = nullptr;
   int rc = static_scratch(&region);
   if (rc != MLXROCM_OK) {
@@ -916,6 +919,7 @@ extern "C" int mlxrocm_gather_qmm(
     void* workspace,
     size_t workspace_bytes,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_gather_qmm");
   int rc = check_shape(
       "gather_qmm", M, N, K, n_indices, group_size, bits, dtype, transpose);
   if (rc != MLXROCM_OK) {

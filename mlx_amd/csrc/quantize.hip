@@ -231,6 +231,7 @@ extern "C" int mlxrocm_affine_quantize(
     int bits,
     int dtype,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_affine_quantize");
   int rc = check_common(
       w, wq, scales, biases, n_elems, group_size, bits, dtype, "quantize");
   if (rc != MLXROCM_OK || n_elems == 0) {
@@ -269,6 +270,7 @@ extern "C" int mlxrocm_affine_dequantize(
     int bits,
     int dtype,
     mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_affine_dequantize");
   int rc = check_common(
       wq, scales, biases, out, n_elems, group_size, bits, dtype, "dequantize");
   if (rc != MLXROCM_OK || n_elems == 0) {
