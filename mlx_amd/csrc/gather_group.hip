@@ -4,7 +4,8 @@
 // mlx/backend/cpu/quantized.cpp:700-747; the Metal backend groups sorted runs,
 // mlx/backend/metal/quantized.cpp:1905-1923).
 //
-// Three small kernels fill a caller-provided workspace:
+// Three small kernels fill a caller-provided workspace (one workgroup does all
+// three steps in a single launch when there are at most 16384 pairs):
 //   count    a histogram per workgroup in LDS, then one global atomic per
 //            workgroup and expert into counts[expert] (one global atomic per
 //            pair serializes on the few counters, worst for sorted indices);
@@ -140,6 +141,83 @@ __global__ __launch_bounds__(256) void group_scatter_kernel(
   }
 }
 
+// All three steps in one workgroup, for calls with so few pairs that four
+// launches cost more than the work: counts, scan and cursors stay in LDS, no
+// global atomics, nothing to clear beforehand.
+constexpr int kFusedThreads = 1024;
+constexpr int kFusedMaxPairs = 16384;
+
+template <typename T>
+__global__ __launch_bounds__(kFusedThreads) void group_fused_kernel(
+    const uint32_t* lhs,
+    const uint32_t* rhs,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int tile_rows,
+    int32_t* offsets,
+    int32_t* tiles,
+    int32_t* n_tiles,
+    int32_t* perm,
+    T* out,
+    int N) {
+  __shared__ int32_t cnt[kMaxExperts];
+  __shared__ int32_t first_pos[kMaxExperts];
+  __shared__ int32_t first_tile[kMaxExperts]; // later: the scatter cursor
+  for (int e = threadIdx.x; e < n_experts; e += kFusedThreads) {
+    cnt[e] = 0;
+  }
+  __syncthreads();
+  for (int l = threadIdx.x; l < n_indices; l += kFusedThreads) {
+    const uint32_t xi = lhs[l];
+    const uint32_t wi = rhs[l];
+    if (xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts)) {
+      atomicAdd(&cnt[wi], 1);
+    } else {
+      T* row = out + static_cast<size_t>(l) * N;
+      for (int n = 0; n < N; ++n) {
+        row[n] = static_cast<T>(0.0f);
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int pos = 0;
+    int tile = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      first_pos[e] = pos;
+      first_tile[e] = tile;
+      pos += cnt[e];
+      tile += (cnt[e] + tile_rows - 1) / tile_rows;
+    }
+    *n_tiles = tile;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_experts; e += kFusedThreads) {
+    offsets[e] = first_pos[e];
+    const int c = cnt[e];
+    int t = first_tile[e];
+    for (int r = 0; r < c; r += tile_rows, ++t) {
+      tiles[3 * t + 0] = e;
+      tiles[3 * t + 1] = first_pos[e] + r;
+      tiles[3 * t + 2] = (c - r < tile_rows) ? c - r : tile_rows;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_experts; e += kFusedThreads) {
+    first_tile[e] = 0;
+  }
+  __syncthreads();
+  for (int l = threadIdx.x; l < n_indices; l += kFusedThreads) {
+    const uint32_t xi = lhs[l];
+    const uint32_t wi = rhs[l];
+    if (xi < static_cast<uint32_t>(x_batches) && wi < static_cast<uint32_t>(n_experts)) {
+      const int rank = atomicAdd(&first_tile[wi], 1);
+      perm[first_pos[wi] + rank] = l;
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* p, int n, int32_t v) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) {
@@ -180,6 +258,24 @@ int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, h
   int32_t* tiles = n_tiles + 4;
   int32_t* perm = tiles + 3 * gather_group_max_tiles(n, E, tile_rows);
 
+  a.group_tiles = tiles;
+  a.group_perm = perm;
+  a.group_ntiles = n_tiles;
+  a.group_tile_rows = tile_rows;
+  if (n <= kFusedMaxPairs) {
+    if (dtype == MLXROCM_BFLOAT16) {
+      group_fused_kernel<bf16_t><<<1, kFusedThreads, 0, s>>>(
+          a.lhs_indices, a.rhs_indices, n, a.x_batches, E, tile_rows, offsets, tiles, n_tiles,
+          perm, static_cast<bf16_t*>(a.out), a.N);
+    } else {
+      group_fused_kernel<f16_t><<<1, kFusedThreads, 0, s>>>(
+          a.lhs_indices, a.rhs_indices, n, a.x_batches, E, tile_rows, offsets, tiles, n_tiles,
+          perm, static_cast<f16_t*>(a.out), a.N);
+    }
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return MLXROCM_OK;
+  }
+
   // counts and cursors start at zero (a fill kernel, so that the sequence can be
   // captured into a graph)
   fill_i32_kernel<<<(2 * E + 255) / 256, 256, 0, s>>>(counts, 2 * E, 0);
@@ -200,11 +296,6 @@ int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, h
   group_scatter_kernel<<<blocks, 256, 0, s>>>(
       a.lhs_indices, a.rhs_indices, n, a.x_batches, E, offsets, cursor, perm);
   MLXROCM_HIP_TRY(hipGetLastError());
-
-  a.group_tiles = tiles;
-  a.group_perm = perm;
-  a.group_ntiles = n_tiles;
-  a.group_tile_rows = tile_rows;
   return MLXROCM_OK;
 }
 

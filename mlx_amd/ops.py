@@ -402,12 +402,24 @@ def _indices_or_default(tag, indices, t):
             raise ValueError(
                 f"{tag} Got indices with invalid dtype. Indices must be integral."
             )
-        return _astype(indices, torch.int64)
+        return indices
     shape = tuple(t.shape[:-2])
     total = 1
     for d in shape:
         total *= d
-    return torch.arange(total, dtype=torch.int64, device=t.device).reshape(shape)
+    return torch.arange(total, dtype=torch.int32, device=t.device).reshape(shape)
+
+
+def _as_uint32(indices: torch.Tensor) -> torch.Tensor:
+    """Flat uint32 view or copy of an index tensor: what ``astype(indices,
+    uint32)`` gives (mlx/ops.cpp:5600-5601) -- two's-complement truncation, so
+    32-bit indices are reinterpreted without a kernel."""
+    flat = _contiguous(indices).reshape(-1)
+    if flat.dtype == torch.uint32:
+        return flat
+    if flat.dtype == torch.int32:
+        return flat.view(torch.uint32)
+    return _astype(flat, torch.uint32)
 
 
 def gather_qmm(
@@ -441,7 +453,8 @@ def gather_qmm(
     _check_affine_params("gather_qmm", group_size, bits)
     _require_gpu("gather_qmm", x, w, scales, biases, lhs, rhs)
     lib = _lib.load()
-    lhs, rhs = torch.broadcast_tensors(lhs, rhs)
+    if lhs.shape != rhs.shape:
+        lhs, rhs = torch.broadcast_tensors(lhs, rhs)
     right_sorted = bool(sorted_indices) and lhs_indices is None
 
     x = _astype(x, out_type)
@@ -464,8 +477,8 @@ def gather_qmm(
         sb = _contiguous(sb)
         sb_stride = sb.shape[-1] * sb.shape[-2]
     n_idx = lhs.numel()
-    lhs_u = _astype(_contiguous(lhs).reshape(-1), torch.uint32) if n_idx else lhs.reshape(-1)
-    rhs_u = _astype(_contiguous(rhs).reshape(-1), torch.uint32) if n_idx else rhs.reshape(-1)
+    lhs_u = _as_uint32(lhs) if n_idx else lhs.reshape(-1)
+    rhs_u = _as_uint32(rhs) if n_idx else rhs.reshape(-1)
     out = torch.empty(tuple(lhs.shape) + (M, w_outer), dtype=out_type, device=x.device)
     code = _DTYPE_CODE[out_type]
     ws_bytes = lib.mlxrocm_gather_qmm_workspace_size(

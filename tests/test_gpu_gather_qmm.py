@@ -167,6 +167,31 @@ def test_gather_qmm_grouped_by_expert(oracle, gpu, dtype, bits, gs):
     assert float((got[sub].double() - ref.double()).abs().max()) <= tol
 
 
+@pytest.mark.parametrize("index_dtype", (torch.int64, torch.int32, torch.uint32, torch.int16))
+def test_gather_qmm_many_pairs_and_index_types(gpu, index_dtype):
+    """More than 16384 pairs take the three-kernel grouping (fewer take the
+    one-workgroup form); both must give what a plain matmul per expert gives.
+    Index tensors of every integer width are accepted: 32-bit ones are used as
+    they are, others are converted."""
+    E, N, K, X = 4, 96, 128, 50
+    dtype = torch.bfloat16
+    w = normal_weights((E, N, K), dtype, std=0.5).to(gpu)
+    wq, s, b = mlx_amd.quantize(w, 64, 4)
+    w_hat = mlx_amd.dequantize(wq, s, b, 64, 4).float()          # [E, N, K]
+    x = activations((X, 1, K), dtype).to(gpu)
+    for T in (3000, 20000):
+        g = torch.Generator().manual_seed(T)
+        rhs = torch.randint(0, E, (T,), generator=g)
+        lhs = torch.randint(0, X, (T,), generator=g)
+        got = mlx_amd.gather_qmm(x, wq, s, b, lhs.to(index_dtype).to(gpu),
+                                 rhs.to(index_dtype).to(gpu), True, 64, 4)
+        assert got.shape == (T, 1, N)
+        want = torch.einsum("tk,tnk->tn", x.reshape(X, K).float()[lhs.to(gpu)],
+                            w_hat[rhs.to(gpu)])
+        err = float((got.reshape(T, N).float() - want).abs().max())
+        assert err <= 2 ** -7 * float(want.abs().max()), (T, err)
+
+
 def test_gather_qmm_grouped_matches_ungrouped(gpu):
     """The grouped launch and the one-GEMV-per-pair launch agree row for row up
     to accumulation order (same fp32 accumulate, one rounding), also with a
