@@ -173,6 +173,87 @@ __global__ __launch_bounds__(kCopyThreads) void copy_strided_kernel(
   dst[dof] = convert<S, D>(src[so]);
 }
 
+// A same-type copy whose source runs along another dimension than the last
+// (a transpose): square tiles through LDS, read along the source's unit-stride
+// dimension `jd`, written along the destination's (the last one).  A tile row is
+// at least one 128-byte line (32 x 32 elements of four or eight bytes, 64 x 64 of
+// two, 128 x 128 of one); rows are padded by one dword against bank conflicts.
+// The other dimensions are a batch walked with div/mod per workgroup.
+template <typename E>
+constexpr int tile_width() {
+  return sizeof(E) >= 4 ? 32 : static_cast<int>(128 / sizeof(E));
+}
+
+struct TransposeShape {
+  int ndim;        // of the batch part
+  int64_t extent_i;
+  int64_t extent_j;
+  int64_t src_stride_i; // elements; the source's stride along j is 1
+  int64_t dst_stride_j; // elements; the destination's stride along i is 1
+  int64_t batch_shape[kMaxDims];
+  int64_t batch_src_stride[kMaxDims];
+  int64_t batch_dst_stride[kMaxDims];
+  int64_t tiles_i;
+  int64_t tiles_j;
+};
+
+template <typename E>
+__global__ __launch_bounds__(256) void transpose_tile_kernel(
+    const E* __restrict__ src,
+    E* __restrict__ dst,
+    TransposeShape t) {
+  constexpr int kTile = tile_width<E>();
+  constexpr int kPad = sizeof(E) >= 4 ? 1 : static_cast<int>(4 / sizeof(E));
+  constexpr int kRowsPerPass = 256 / kTile;
+  __shared__ E tile[kTile][kTile + kPad];
+  int64_t block = blockIdx.x;
+  const int64_t tj = block % t.tiles_j;
+  block /= t.tiles_j;
+  const int64_t ti = block % t.tiles_i;
+  int64_t rest = block / t.tiles_i;
+  int64_t so = 0;
+  int64_t dof = 0;
+  for (int d = t.ndim - 1; d >= 0; --d) {
+    const int64_t c = rest % t.batch_shape[d];
+    rest /= t.batch_shape[d];
+    so += c * t.batch_src_stride[d];
+    dof += c * t.batch_dst_stride[d];
+  }
+  const int tx = threadIdx.x % kTile;
+  const int ty = threadIdx.x / kTile;
+  const int64_t i0 = ti * kTile;
+  const int64_t j0 = tj * kTile;
+#pragma unroll
+  for (int r = 0; r < kTile; r += kRowsPerPass) {
+    const int64_t i = i0 + ty + r;
+    const int64_t j = j0 + tx;
+    if (i < t.extent_i && j < t.extent_j) {
+      tile[ty + r][tx] = src[so + i * t.src_stride_i + j];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kTile; r += kRowsPerPass) {
+    const int64_t j = j0 + ty + r;
+    const int64_t i = i0 + tx;
+    if (i < t.extent_i && j < t.extent_j) {
+      dst[dof + j * t.dst_stride_j + i] = tile[tx][ty + r];
+    }
+  }
+}
+
+template <typename E>
+int launch_transpose(const void* src, void* dst, const TransposeShape& t, size_t batch, hipStream_t stream) {
+  const size_t blocks = static_cast<size_t>(t.tiles_i) * t.tiles_j * batch;
+  if (blocks > 0x7fffffffull) {
+    return fail(MLXROCM_UNSUPPORTED, "[copy] too many tiles for one launch");
+  }
+  transpose_tile_kernel<E><<<dim3(static_cast<unsigned>(blocks)), 256, 0, stream>>>(
+      static_cast<const E*>(src), static_cast<E*>(dst), t);
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return MLXROCM_OK;
+}
+
 bool valid_copy_dtype(int dt) {
   return dt >= 0 && dt < kNumDtypes;
 }
@@ -384,6 +465,59 @@ extern "C" int mlxrocm_copy_strided(
   }
   if (nd == 1 && css[0] == 0 && cds[0] == 1) {
     return mlxrocm_copy_contiguous(src, src_dtype, dst, dst_dtype, n, 1, stream);
+  }
+  // A same-type copy that the destination walks along its last dimension while
+  // the source runs along another one: tiled transpose.
+  if (src_dtype == dst_dtype && nd >= 2 && cds[nd - 1] == 1 && css[nd - 1] != 1 &&
+      cs[nd - 1] >= 8) {
+    int jd = -1;
+    for (int d = nd - 2; d >= 0; --d) {
+      if (css[d] == 1 && cs[d] >= 8) {
+        jd = d;
+        break;
+      }
+    }
+    bool positive = true;
+    for (int d = 0; d < nd; ++d) {
+      positive = positive && css[d] >= 0 && cds[d] >= 0;
+    }
+    if (jd >= 0 && positive) {
+      TransposeShape t;
+      t.extent_i = cs[nd - 1];
+      t.extent_j = cs[jd];
+      t.src_stride_i = css[nd - 1];
+      t.dst_stride_j = cds[jd];
+      const int64_t tile = kItemSize[src_dtype] >= 4 ? 32 : 128 / static_cast<int64_t>(kItemSize[src_dtype]);
+      t.tiles_i = (t.extent_i + tile - 1) / tile;
+      t.tiles_j = (t.extent_j + tile - 1) / tile;
+      t.ndim = 0;
+      size_t batch = 1;
+      for (int d = 0; d < nd - 1; ++d) {
+        if (d == jd) {
+          continue;
+        }
+        t.batch_shape[t.ndim] = cs[d];
+        t.batch_src_stride[t.ndim] = css[d];
+        t.batch_dst_stride[t.ndim] = cds[d];
+        batch *= static_cast<size_t>(cs[d]);
+        ++t.ndim;
+      }
+      for (int d = t.ndim; d < kMaxDims; ++d) {
+        t.batch_shape[d] = 1;
+        t.batch_src_stride[d] = 0;
+        t.batch_dst_stride[d] = 0;
+      }
+      switch (kItemSize[src_dtype]) {
+        case 1:
+          return launch_transpose<uint8_t>(src, dst, t, batch, s);
+        case 2:
+          return launch_transpose<uint16_t>(src, dst, t, batch, s);
+        case 4:
+          return launch_transpose<uint32_t>(src, dst, t, batch, s);
+        default:
+          return launch_transpose<uint64_t>(src, dst, t, batch, s);
+      }
+    }
   }
   // A same-type copy moves bytes: when both sides walk the innermost dimension
   // contiguously, widen the element to 16, 8 or 4 bytes (fewer, wider accesses)

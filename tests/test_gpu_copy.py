@@ -202,6 +202,39 @@ def test_row_slices_take_the_widened_path_and_its_fallbacks(dtype):
         assert _bytes(got) == _bytes(src[5:61:3, lo:hi].contiguous()), (lo, hi)
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.complex64],
+                         ids=lambda d: str(d).split(".")[-1])
+def test_transposed_sources_take_the_tiled_path(dtype):
+    """A same-type copy whose source runs along another dimension than the last
+    goes through 32 x 32 LDS tiles: ragged extents, batch dimensions on either
+    side of the transposed pair, a batch dimension with its own stride."""
+    base = _source(dtype, 7 * 45 * 70, seed=31).reshape(7, 45, 70)
+    dev = base.to(DEV)
+    views = {
+        "2d": lambda t: t[0].t(),                       # [70, 45]
+        "batched": lambda t: t.transpose(1, 2),         # [7, 70, 45]
+        "batch_inside": lambda t: t.permute(2, 0, 1),   # [70, 7, 45]: last = dim 1, unit stride = dim 2
+        "outer_to_last": lambda t: t.permute(1, 2, 0),  # [45, 70, 7]: too short a last dim -> generic
+        "sliced": lambda t: t[1:6, 3:40, 5:69].transpose(1, 2),
+        "stepped_batch": lambda t: t[::2].transpose(1, 2),
+    }
+    for name, view in views.items():
+        got = _copy.contiguous(view(dev))
+        assert _bytes(got) == _bytes(view(base).contiguous()), name
+    # into a destination with its own row stride (general -> general)
+    lib = _lib.load()
+    arr = lambda v: (ctypes.c_int64 * len(v))(*v)
+    src2 = dev[0]                                           # [45, 70]
+    out = torch.zeros((70, 64), dtype=dtype, device=DEV)
+    code = _copy.DTYPE_CODE[dtype]
+    _lib.check(lib.mlxrocm_copy_strided(
+        src2.data_ptr(), code, arr((1, 70)), out.data_ptr(), code, arr((64, 1)),
+        2, arr((70, 45)), torch.cuda.current_stream().cuda_stream))
+    want = torch.zeros((70, 64), dtype=dtype)
+    want[:, :45] = base[0].t()
+    assert _bytes(out) == _bytes(want)
+
+
 def test_fill_broadcasts_one_device_scalar():
     like = torch.empty((33, 77), dtype=torch.bfloat16, device=DEV)
     value = torch.tensor([1.2345], dtype=torch.float32, device=DEV)
