@@ -28,9 +28,9 @@ BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes, scaled by
 # a copy of known size (profiles/qmv_stream_4bit_g64_bf16_14336x4096.md and
 # profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md).
-QMV_TRAFFIC_BYTES = 33220710
+QMV_TRAFFIC_BYTES = 33220712
 QMV_TRAFFIC_SOURCE = "profiles/qmv_stream_4bit_g64_bf16_14336x4096.md"
-QMM_T_TRAFFIC_BYTES = 260195251
+QMM_T_TRAFFIC_BYTES = 260196713
 QMM_T_TRAFFIC_SOURCE = "profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md"
 
 N, K = 14336, 4096
