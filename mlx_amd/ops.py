@@ -12,6 +12,7 @@ raise ``ValueError`` exactly where the reference throws
 """
 from __future__ import annotations
 
+import functools
 from typing import Optional, Tuple
 
 import torch
@@ -410,6 +411,41 @@ def _indices_or_default(tag, indices, t):
     return torch.arange(total, dtype=torch.int32, device=t.device).reshape(shape)
 
 
+def _broadcast_shape(a: tuple, b: tuple) -> tuple:
+    """Numpy broadcasting of two shapes in plain Python (the library routine
+    costs more than the rest of a decode-sized call)."""
+    if a == b:
+        return a
+    if len(a) < len(b):
+        a, b = b, a
+    out = list(a)
+    off = len(a) - len(b)
+    for i, d in enumerate(b):
+        e = out[off + i]
+        if e == d or d == 1:
+            continue
+        if e != 1:
+            raise ValueError(f"Shapes {a} and {b} cannot be broadcast.")
+        out[off + i] = d
+    return tuple(out)
+
+
+@functools.lru_cache(maxsize=64)
+def _default_lhs_uint32(batch_shape: tuple, like_shape: tuple, device: torch.device) -> torch.Tensor:
+    """The default ``lhs_indices`` (``arange`` over the batch dims of x,
+    mlx/ops.cpp:100-107) broadcast against ``like_shape`` and flattened to
+    uint32.  It depends on shapes only, so it is built once per shape and kept:
+    a decode step then issues no kernel for it.  Callers only read it."""
+    total = 1
+    for d in batch_shape:
+        total *= d
+    lhs = torch.arange(total, dtype=torch.int32, device=device).reshape(batch_shape)
+    shape = _broadcast_shape(batch_shape, like_shape)
+    flat = lhs.expand(shape).reshape(-1).contiguous().view(torch.uint32)
+    torch.cuda.current_stream(device).synchronize()  # later calls may run on other streams
+    return flat
+
+
 def _as_uint32(indices: torch.Tensor) -> torch.Tensor:
     """Flat uint32 view or copy of an index tensor: what ``astype(indices,
     uint32)`` gives (mlx/ops.cpp:5600-5601) -- two's-complement truncation, so
@@ -448,12 +484,24 @@ def gather_qmm(
         raise ValueError(
             f"[gather_qmm] Only real floating types are supported but x.dtype() == {x.dtype}."
         )
-    lhs = _indices_or_default("[gather_qmm]", lhs_indices, x)
+    lhs = None if lhs_indices is None and rhs_indices is not None else \
+        _indices_or_default("[gather_qmm]", lhs_indices, x)
     rhs = _indices_or_default("[gather_qmm]", rhs_indices, w)
+    if lhs is None:
+        # default lhs against given rhs: shapes decide everything
+        if x.dim() < 2:
+            raise ValueError(
+                "[gather_qmm] Input must have at least two dimensions but got input with "
+                f"shape {tuple(x.shape)}."
+            )
+        lhs_shape = _broadcast_shape(tuple(x.shape[:-2]), tuple(rhs.shape))
     _check_affine_params("gather_qmm", group_size, bits)
-    _require_gpu("gather_qmm", x, w, scales, biases, lhs, rhs)
+    _require_gpu("gather_qmm", x, w, scales, biases, rhs, *(() if lhs is None else (lhs,)))
     lib = _lib.load()
-    if lhs.shape != rhs.shape:
+    if lhs is None:
+        if tuple(rhs.shape) != lhs_shape:
+            rhs = rhs.expand(lhs_shape)
+    elif lhs.shape != rhs.shape:
         lhs, rhs = torch.broadcast_tensors(lhs, rhs)
     right_sorted = bool(sorted_indices) and lhs_indices is None
 
@@ -476,10 +524,13 @@ def gather_qmm(
         bb = _contiguous(bb)
         sb = _contiguous(sb)
         sb_stride = sb.shape[-1] * sb.shape[-2]
-    n_idx = lhs.numel()
-    lhs_u = _as_uint32(lhs) if n_idx else lhs.reshape(-1)
+    n_idx = rhs.numel()
+    if lhs is None:
+        lhs_u = _default_lhs_uint32(tuple(x.shape[:-2]), tuple(rhs.shape), x.device)
+    else:
+        lhs_u = _as_uint32(lhs) if n_idx else lhs.reshape(-1)
     rhs_u = _as_uint32(rhs) if n_idx else rhs.reshape(-1)
-    out = torch.empty(tuple(lhs.shape) + (M, w_outer), dtype=out_type, device=x.device)
+    out = torch.empty(tuple(rhs.shape) + (M, w_outer), dtype=out_type, device=x.device)
     code = _DTYPE_CODE[out_type]
     ws_bytes = lib.mlxrocm_gather_qmm_workspace_size(
         M, w_outer, K, n_idx, wb.shape[0], group_size, bits, code,

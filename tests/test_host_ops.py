@@ -79,3 +79,23 @@ def test_gather_qmm_errors_and_defaults():
     # without indices it is quantized_matmul (mlx/ops.cpp:5566-5569)
     with pytest.raises(RuntimeError, match="GPU"):
         mlx_amd.gather_qmm(x, wq, s, b)
+
+
+def test_broadcast_shape_matches_numpy():
+    """The plain-Python shape broadcast used for default gather indices agrees
+    with numpy on every pair, errors included."""
+    import itertools
+
+    import numpy as np
+
+    from mlx_amd.ops import _broadcast_shape
+
+    shapes = [(), (1,), (3,), (2, 3), (1, 3), (2, 1), (4, 2, 3), (4, 1, 1), (0,), (2, 0)]
+    for a, b in itertools.product(shapes, repeat=2):
+        try:
+            want = tuple(np.broadcast_shapes(a, b))
+        except ValueError:
+            with pytest.raises(ValueError):
+                _broadcast_shape(a, b)
+            continue
+        assert _broadcast_shape(a, b) == want, (a, b)
