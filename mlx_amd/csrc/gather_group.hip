@@ -87,7 +87,8 @@ __global__ __launch_bounds__(256) void group_plan_kernel(
       pos += cnt[e];
       tile += (cnt[e] + tile_rows - 1) / tile_rows;
     }
-    *n_tiles = tile;
+    n_tiles[0] = tile;
+    n_tiles[1] = pos; // pairs with both indices in range
   }
   __syncthreads();
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
@@ -190,7 +191,8 @@ __global__ __launch_bounds__(kFusedThreads) void group_fused_kernel(
       pos += cnt[e];
       tile += (cnt[e] + tile_rows - 1) / tile_rows;
     }
-    *n_tiles = tile;
+    n_tiles[0] = tile;
+    n_tiles[1] = pos; // pairs with both indices in range
   }
   __syncthreads();
   for (int e = threadIdx.x; e < n_experts; e += kFusedThreads) {

@@ -405,6 +405,28 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
       return MLXROCM_LAUNCH(sc, launch_qmv_quad(a, gs, bits, dtype, s));
     }
   }
+  // 5..32 rows of 4-bit codes: packed rows streamed through LDS, x resident per
+  // K range (measured against the kernels below on 4096..28672 x 4096 and
+  // 4096 x 14336: 15-34 us against 19-41 us from 9 rows on, level at 5..8 rows).
+  // Its units (K ranges x 256-row slabs) must fill at least half the compute
+  // units: 4096 x 4096 has 64 of them and stays on the kernels below (12 us
+  // against 8 us).
+  if (transpose && a.M >= 5 && a.M <= 32 && a.lhs_indices == nullptr &&
+      a.group_tiles == nullptr && a.w_alt == nullptr &&
+      qmm_slab_supported(a, gs, bits, dtype, transpose) &&
+      2 * qmm_slab_units(a) >= compute_units()) {
+    const size_t plane_bytes = qmm_slab_plane_bytes(a);
+    if (plane_bytes == 0 || (static_cast<int64_t>(a.L) * a.M * a.N) % 4 == 0) {
+      void* region = nullptr;
+      if (plane_bytes != 0) {
+        const int rc = claim(sc, plane_bytes, &region);
+        if (rc != MLXROCM_OK) {
+          return rc;
+        }
+      }
+      return MLXROCM_LAUNCH(sc, launch_qmm_slab(a, gs, bits, dtype, region, s));
+    }
+  }
   // (two rows of 8-bit codes over a long K: the streaming kernel's dot products
   // are issue-bound there, 28 us against 20 us for the wide kernel at K = 14336)
   const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype) ||
@@ -875,14 +897,23 @@ bool group_gather(
   return gather_group_workspace_bytes(n_indices, n_experts) > 0;
 }
 
+// Small expert groups of 4-bit weights run on the slab kernel, whose K ranges
+// meet in fp32 planes behind the grouping tables.
+bool group_gather_small(int K, int n_indices, int n_experts) {
+  return K % 128 == 0 && static_cast<int64_t>(n_indices) <= 64 * static_cast<int64_t>(n_experts);
+}
+bool group_gather_slab(int N, int K, int n_indices, int n_experts, int gs, int bits) {
+  return group_gather_small(K, n_indices, n_experts) && qmm_slab_shape_ok(32, N, K, gs, bits);
+}
+
 extern "C" size_t mlxrocm_gather_qmm_workspace_size(
     int M,
-    int /*N*/,
+    int N,
     int K,
     int n_indices,
     int n_experts,
-    int /*group_size*/,
-    int /*bits*/,
+    int group_size,
+    int bits,
     int dtype,
     int transpose,
     int /*rhs_sorted*/) {
@@ -891,7 +922,11 @@ extern "C" size_t mlxrocm_gather_qmm_workspace_size(
   if (!group_gather(M, K, n_indices, n_experts, 1, 0, dtype, transpose != 0)) {
     return 0;
   }
-  return gather_group_workspace_bytes(n_indices, n_experts);
+  size_t bytes = gather_group_workspace_bytes(n_indices, n_experts);
+  if (group_gather_slab(N, K, n_indices, n_experts, group_size, bits)) {
+    bytes += qmm_slab_grouped_plane_bytes(n_indices, N, K);
+  }
+  return bytes;
 }
 
 extern "C" int mlxrocm_gather_qmm(
@@ -972,11 +1007,16 @@ extern "C" int mlxrocm_gather_qmm(
     }
     // small groups (at most 64 pairs per expert on average) go to the few-row
     // kernel in 32-row tiles, larger ones to the 256-row tile GEMM
-    const bool small = K % 128 == 0 &&
-        static_cast<int64_t>(n_indices) <= 64 * static_cast<int64_t>(n_experts);
+    const bool small = group_gather_small(K, n_indices, n_experts);
     rc = launch_gather_group(a, dtype, small ? kGroupSmallTile : kGroupLargeTile, workspace, s);
     if (rc != MLXROCM_OK) {
       return rc;
+    }
+    const size_t tables = gather_group_workspace_bytes(n_indices, n_experts);
+    if (group_gather_slab(N, K, n_indices, n_experts, group_size, bits) &&
+        workspace_bytes >= tables + qmm_slab_grouped_plane_bytes(n_indices, N, K)) {
+      return launch_qmm_slab_grouped(
+          a, group_size, bits, dtype, static_cast<char*>(workspace) + tables, s);
     }
     return small ? launch_qmm_skinny_grouped(a, group_size, bits, dtype, s)
                  : launch_qmm_mfma_grouped(a, group_size, bits, dtype, s);

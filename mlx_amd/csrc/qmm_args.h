@@ -28,8 +28,8 @@ struct QmmArgs {
   // Grouped gather (M == 1): the index pairs sorted by expert and cut into tiles
   // of up to group_tile_rows rows.  group_tiles holds {expert, first sorted position, rows}
   // per tile, group_perm maps a sorted position to its index pair, group_ntiles
-  // points at the number of tiles (known on the device only).  All null
-  // otherwise.
+  // points at the number of tiles followed by the number of sorted positions
+  // (both known on the device only).  All null otherwise.
   const int32_t* group_tiles;
   const int32_t* group_perm;
   const int32_t* group_ntiles;
@@ -120,6 +120,17 @@ size_t gather_group_workspace_bytes(int n_indices, int n_experts);
 int gather_group_max_tiles(int n_indices, int n_experts, int tile_rows);
 int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, hipStream_t s);
 int launch_qmm_skinny_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+// Up to 32 rows of x per weight matrix, 4-bit codes, 16-bit types, K % 1024 == 0:
+// packed rows streamed through LDS, x resident per K range.  With more than one
+// K range the partial sums go through fp32 planes (`planes`, *_plane_bytes()).
+bool qmm_slab_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
+bool qmm_slab_shape_ok(int rows, int N, int K, int gs, int bits);
+long qmm_slab_units(const QmmArgs& a); // work items of a plain call
+size_t qmm_slab_plane_bytes(const QmmArgs& a);
+int launch_qmm_slab(const QmmArgs& a, int gs, int bits, int dtype, void* planes, hipStream_t s);
+size_t qmm_slab_grouped_plane_bytes(int n_indices, int N, int K);
+int launch_qmm_slab_grouped(
+    const QmmArgs& a, int gs, int bits, int dtype, void* planes, hipStream_t s);
 // fp32 operands on the bf16 matrix path: x is first split into bf16 high and
 // low parts (split_x_for_mfma into a buffer of split_x_bytes), then
 // launch_qmm_mfma_split runs with a.x pointing at that buffer.

@@ -1,0 +1,115 @@
+"""GPU parity of the few-row kernel that streams packed 4-bit rows through LDS
+with x resident per K range (5..32 rows of a plain call, small expert groups of
+a gather): against the CPU oracle and the fp64 product of the exact weights."""
+import pytest
+import torch
+
+import mlx_amd
+from mlx_amd import _lib
+from tests.test_gpu_qmm import _check_qmm
+from tests.util import (
+    activations, exact_affine_weights, exact_tolerance, matmul_tolerance, normal_weights,
+)
+
+pytestmark = pytest.mark.gpu
+
+CODE = {torch.float16: 1, torch.bfloat16: 2}
+
+
+def _planes_bytes(M, N, K, L=1):
+    return (K // 1024) * L * M * N * 4 if K > 1024 else 0
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("gs", (32, 64, 128))
+@pytest.mark.parametrize("M", (5, 9, 16, 17, 32))
+def test_slab_rows_and_groups(oracle, gpu, dtype, gs, M):
+    """[8192, 4096]: four K ranges x 32 slabs.  32-wide groups have no two-tile
+    form and stay on the older kernels from 17 rows on (still checked)."""
+    N, K = 8192, 4096
+    w = normal_weights((N, K), dtype, std=0.05)
+    x = activations((M, K), dtype)
+    _check_qmm(oracle, gpu, x, w, gs, 4, rows=torch.tensor([0, M - 1]))
+    if M >= 9 and (gs != 32 or M <= 16):  # (5..8 rows: only where the 4x4x4 kernel is not chosen)
+        ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, 4, CODE[dtype], 1)
+        assert ws == _planes_bytes(M, N, K), "the shape did not take the slab kernel"
+
+
+@pytest.mark.parametrize("N,K", ((8000, 4096), (32772, 1024), (4096, 14336)))
+def test_slab_ragged_and_single_range(oracle, gpu, N, K):
+    """N that is no multiple of the 256-row slab (the last slab's rows are
+    clamped and never written), a single K range (written directly, no planes)
+    and a long K (14 ranges)."""
+    dtype = torch.bfloat16
+    w = normal_weights((N, K), dtype, std=0.05)
+    for M in (9, 24):
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, w, 64, 4, rows=torch.tensor([M - 1]))
+        ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, 64, 4, 2, 1)
+        assert ws == _planes_bytes(M, N, K)
+
+
+def test_slab_batched_weights(oracle, gpu):
+    """Eight problems of [4096, 1024] with their own weights: the unit list runs
+    over problems, every workgroup restages x when it crosses into the next one."""
+    L, M, N, K = 8, 9, 4096, 1024
+    dtype = torch.float16
+    w = normal_weights((L, N, K), dtype, std=0.05)
+    wq, s, b = oracle.quantize(w, 64, 4)
+    x = activations((L, M, K), dtype)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq.to(gpu), s.to(gpu), b.to(gpu), True, 64, 4).cpu()
+    ref = oracle.qmm_batched(x, wq, s, b, True, 64, 4)
+    w_hat = exact_affine_weights(wq, s, b, 64, 4)
+    exact = torch.einsum("lmk,lnk->lmn", x.double(), w_hat)
+    assert float((got.double() - exact).abs().max()) <= exact_tolerance(dtype, K, x, w_hat, exact)
+    assert float((got.double() - ref.double()).abs().max()) <= matmul_tolerance(dtype, K, x, w_hat)
+
+
+@pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 64), (torch.float16, 64), (torch.bfloat16, 128)))
+def test_slab_grouped_gather(oracle, gpu, dtype, gs):
+    """64 tokens x top-2 of 8 experts of [520, 2048] (two K ranges, a ragged
+    slab): experts end up with fewer and with more than 16 rows, one pair names
+    an expert that does not exist (zero row), and the run on expert-sorted pairs
+    reproduces the unsorted one bit for bit."""
+    E, N, K, T = 8, 520, 2048, 64
+    w = normal_weights((E, N, K), dtype, std=0.5)
+    wq, s, b = oracle.quantize(w, gs, 4)
+    x = activations((T, 1, 1, K), dtype)
+    g = torch.Generator().manual_seed(3)
+    idx = torch.randint(0, E, (T, 2), generator=g)
+    idx[:12, 0] = 5  # one expert with well over 16 rows
+    counts = torch.bincount(idx.reshape(-1), minlength=E)
+    assert int(counts.max()) > 16 and int(counts.min()) <= 16
+    gx, gwq, gsc, gb, gidx = (t.to(gpu) for t in (x, wq, s, b, idx))
+    ws = _lib.load().mlxrocm_gather_qmm_workspace_size(1, N, K, 2 * T, E, gs, 4, CODE[dtype], 1, 0)
+    assert ws >= (K // 1024) * 2 * T * N * 4, "the call did not take the slab kernel"
+    got = mlx_amd.gather_qmm(gx, gwq, gsc, gb, rhs_indices=gidx, transpose=True,
+                             group_size=gs, bits=4)
+    assert got.shape == (T, 2, 1, N)
+    ref = oracle.gather_qmm(
+        x.reshape(T, 1, K), wq, s, b,
+        torch.arange(T).repeat_interleave(2), idx.reshape(-1), True, gs, 4,
+    ).reshape(T, 2, 1, N)
+    w_hat = exact_affine_weights(wq, s, b, gs, 4)
+    exact = torch.einsum("tk,tjnk->tjn", x.reshape(T, K).double(), w_hat[idx]).reshape(T, 2, 1, N)
+    assert float((got.cpu().double() - exact).abs().max()) <= exact_tolerance(
+        dtype, K, x, w_hat, exact)
+    assert float((got.cpu().double() - ref.double()).abs().max()) <= matmul_tolerance(
+        dtype, K, x, w_hat)
+    # sorted by expert: same rows, bit for bit
+    flat = gidx.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    xs = gx.reshape(T, 1, K)[order // 2]
+    ys = mlx_amd.gather_qmm(xs, gwq, gsc, gb, rhs_indices=flat[order].contiguous(),
+                            transpose=True, group_size=gs, bits=4, sorted_indices=True)
+    assert torch.equal(ys[torch.argsort(order)].reshape(T, 2, 1, N), got)
+    # an expert index out of range: that row is zero, the others unchanged
+    bad = gidx.clone()
+    bad[7, 1] = E + 3
+    got_bad = mlx_amd.gather_qmm(gx, gwq, gsc, gb, rhs_indices=bad, transpose=True,
+                                 group_size=gs, bits=4)
+    torch.cuda.synchronize()
+    assert bool((got_bad[7, 1] == 0).all())
+    keep = torch.ones((T, 2), dtype=torch.bool, device=gpu)
+    keep[7, 1] = False
+    assert torch.equal(got_bad[keep], got[keep])
