@@ -260,7 +260,7 @@ def sweep(torch, mlx_amd, dev) -> list:
     # Cfg2: decode, Llama-3-8B MLP shapes
     for (n, k) in ((14336, 4096), (4096, 14336)):
         for (bits, gs) in ((4, 64), (8, 128)):
-            for B in (1, 2, 4, 8):
+            for B in (1, 2, 4, 8) + ((16, 32) if bits == 4 else ()):
                 matmul_case("cfg2", B, n, k, bits, gs, bf16)
     # Cfg3: prefill
     for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336)):
