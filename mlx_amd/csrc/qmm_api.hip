@@ -1014,6 +1014,7 @@ extern "C" int mlxrocm_gather_qmm(
     }
     const size_t tables = gather_group_workspace_bytes(n_indices, n_experts);
     if (group_gather_slab(N, K, n_indices, n_experts, group_size, bits) &&
+        (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0 && // 16-byte stores into the planes
         workspace_bytes >= tables + qmm_slab_grouped_plane_bytes(n_indices, N, K)) {
       return launch_qmm_slab_grouped(
           a, group_size, bits, dtype, static_cast<char*>(workspace) + tables, s);
