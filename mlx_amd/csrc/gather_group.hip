@@ -248,6 +248,17 @@ size_t gather_group_workspace_bytes(int n_indices, int n_experts) {
   return align_up(ints * sizeof(int32_t), 256);
 }
 
+void bind_gather_group(QmmArgs& a, int tile_rows, void* workspace) {
+  const int E = a.n_experts;
+  int32_t* ws = static_cast<int32_t*>(workspace);
+  int32_t* n_tiles = ws + 3 * E;
+  int32_t* tiles = n_tiles + 4;
+  a.group_tiles = tiles;
+  a.group_perm = tiles + 3 * gather_group_max_tiles(a.L, E, tile_rows);
+  a.group_ntiles = n_tiles;
+  a.group_tile_rows = tile_rows;
+}
+
 // Fills the workspace and points the grouped-mode fields of `a` into it.
 int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, hipStream_t s) {
   const int E = a.n_experts;

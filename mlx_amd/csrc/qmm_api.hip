@@ -1008,16 +1008,23 @@ extern "C" int mlxrocm_gather_qmm(
     // small groups (at most 64 pairs per expert on average) go to the few-row
     // kernel in 32-row tiles, larger ones to the 256-row tile GEMM
     const bool small = group_gather_small(K, n_indices, n_experts);
+    const size_t tables = gather_group_workspace_bytes(n_indices, n_experts);
+    const bool slab = group_gather_slab(N, K, n_indices, n_experts, group_size, bits) &&
+        (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0 && // 16-byte stores into the planes
+        workspace_bytes >= tables + qmm_slab_grouped_plane_bytes(n_indices, N, K);
+    if (slab && qmm_slab_plans_in_kernel(n_indices, n_experts)) {
+      // few pairs: the kernel groups them itself, one launch less
+      bind_gather_group(a, kGroupSmallTile, workspace);
+      return launch_qmm_slab_grouped(
+          a, group_size, bits, dtype, static_cast<char*>(workspace) + tables, true, s);
+    }
     rc = launch_gather_group(a, dtype, small ? kGroupSmallTile : kGroupLargeTile, workspace, s);
     if (rc != MLXROCM_OK) {
       return rc;
     }
-    const size_t tables = gather_group_workspace_bytes(n_indices, n_experts);
-    if (group_gather_slab(N, K, n_indices, n_experts, group_size, bits) &&
-        (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0 && // 16-byte stores into the planes
-        workspace_bytes >= tables + qmm_slab_grouped_plane_bytes(n_indices, N, K)) {
+    if (slab) {
       return launch_qmm_slab_grouped(
-          a, group_size, bits, dtype, static_cast<char*>(workspace) + tables, s);
+          a, group_size, bits, dtype, static_cast<char*>(workspace) + tables, false, s);
     }
     return small ? launch_qmm_skinny_grouped(a, group_size, bits, dtype, s)
                  : launch_qmm_mfma_grouped(a, group_size, bits, dtype, s);

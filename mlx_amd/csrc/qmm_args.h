@@ -119,6 +119,8 @@ constexpr int kGroupSmallTile = 32;  // rows per tile of the few-row kernel
 size_t gather_group_workspace_bytes(int n_indices, int n_experts);
 int gather_group_max_tiles(int n_indices, int n_experts, int tile_rows);
 int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, hipStream_t s);
+// Only points the grouped-mode fields of `a` into the workspace (no launch).
+void bind_gather_group(QmmArgs& a, int tile_rows, void* workspace);
 int launch_qmm_skinny_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 // Up to 32 rows of x per weight matrix, 4-bit codes, 16-bit types, K % 1024 == 0:
 // packed rows streamed through LDS, x resident per K range.  With more than one
@@ -129,8 +131,13 @@ long qmm_slab_units(const QmmArgs& a); // work items of a plain call
 size_t qmm_slab_plane_bytes(const QmmArgs& a);
 int launch_qmm_slab(const QmmArgs& a, int gs, int bits, int dtype, void* planes, hipStream_t s);
 size_t qmm_slab_grouped_plane_bytes(int n_indices, int N, int K);
+// plan_in_kernel: the kernel groups the pairs itself (`a` carries the index
+// arrays and, from bind_gather_group, where the sorted order goes for the plane
+// reduction); otherwise launch_gather_group must have run.
+bool qmm_slab_plans_in_kernel(int n_indices, int n_experts);
 int launch_qmm_slab_grouped(
-    const QmmArgs& a, int gs, int bits, int dtype, void* planes, hipStream_t s);
+    const QmmArgs& a, int gs, int bits, int dtype, void* planes, bool plan_in_kernel,
+    hipStream_t s);
 // fp32 operands on the bf16 matrix path: x is first split into bf16 high and
 // low parts (split_x_for_mfma into a buffer of split_x_bytes), then
 // launch_qmm_mfma_split runs with a.x pointing at that buffer.

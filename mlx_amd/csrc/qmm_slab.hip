@@ -46,6 +46,19 @@ constexpr int kSlSteps = kSlKr / kSlStep;            // steps per unit
 constexpr int kSlSlotBytes = kSlWaveRows * kSlStep / 2; // packed codes of a step
 constexpr int kSlXStride = 2 * kSlKr + 16;           // bytes per staged row of x
 
+// Gathers of up to kSlPlanPairs index pairs over up to kSlPlanExperts experts
+// are grouped by expert inside the kernel: every workgroup builds the same
+// tile list and sorted order in LDS (a counting sort on ballots, positions
+// ascending by pair index inside an expert, so all workgroups agree), which
+// saves the planning launch in front of a kernel that lasts a few tens of
+// microseconds.
+constexpr int kSlPlanPairs = kSlThreads;  // one pair per thread
+constexpr int kSlPlanExperts = 64;
+constexpr int kSlPlanTiles = kSlPlanPairs / 32 + kSlPlanExperts;
+constexpr int kSlPlanInts = kSlPlanPairs + kSlWaves * (kSlPlanExperts + 1) +
+    3 * (kSlPlanExperts + 1) + 3 * kSlPlanTiles + 4;
+constexpr int kSlPlanBytes = (kSlPlanInts * 4 + 255) / 256 * 256;
+
 struct SlabPlan {
   int ranges;          // K / 1024
   int n_slabs;         // ceil(N / 256)
@@ -72,10 +85,10 @@ constexpr int slab_stages() {
   return (MT == 1 && GS >= 64) ? 3 : 2;
 }
 
-template <int GS, int MT>
+template <int GS, int MT, int MODE>
 constexpr size_t slab_smem_bytes() {
   constexpr size_t xr = 16 * MT;
-  return xr * kSlXStride + xr * (SlabShape<GS>::kGroupsPerRange + 1) * 4 + xr * 4 + xr * 8 +
+  return (MODE == 2 ? kSlPlanBytes : 0) + xr * kSlXStride + xr * (SlabShape<GS>::kGroupsPerRange + 1) * 4 + xr * 4 + xr * 8 +
       static_cast<size_t>(kSlWaves) *
       (slab_stages<GS, MT>() * kSlSlotBytes + SlabShape<GS>::kSbBytes);
 }
@@ -171,8 +184,12 @@ struct SlabUnit {
 
 // (two waves per SIMD as the register budget: the matrix instructions then keep
 // their results in ordinary registers, where the FMAs read them)
-template <typename T, int GS, int MT, bool GROUPED>
+// MODE 0: plain call; 1: gather, grouped by the planning kernel; 2: gather,
+// grouped here.
+template <typename T, int GS, int MT, int MODE>
 __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a, const SlabPlan pl) {
+  constexpr bool GROUPED = MODE != 0;
+  constexpr bool PLAN = MODE == 2;
   using Shape = SlabShape<GS>;
   constexpr int GPS = Shape::kGroupsPerStep;
   constexpr int DW = Shape::kDwords;
@@ -198,8 +215,16 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   const int groups = K / GS;   // groups per row of W
   const int row_bytes = K / 2;
 
-  uint8_t* xl = smem;
-  float* xsum = reinterpret_cast<float*>(smem + XR * kSlXStride);
+  // in-kernel planning tables (MODE 2), in front of everything else
+  int32_t* lperm = reinterpret_cast<int32_t*>(smem);         // sorted position -> pair
+  int32_t* lwave = lperm + kSlPlanPairs;                       // [wave][expert] counts, then bases
+  int32_t* lcnt = lwave + kSlWaves * (kSlPlanExperts + 1);     // pairs per expert
+  int32_t* lpos = lcnt + kSlPlanExperts + 1;                   // first sorted position
+  int32_t* lfirst = lpos + kSlPlanExperts + 1;                 // first tile
+  int32_t* ltiles = lfirst + kSlPlanExperts + 1;               // {expert, first position, rows}
+  int32_t* lnum = ltiles + 3 * kSlPlanTiles;                   // {tiles, sorted positions}
+  uint8_t* xl = smem + (PLAN ? kSlPlanBytes : 0);
+  float* xsum = reinterpret_cast<float*>(xl + XR * kSlXStride);
   int32_t* orow = reinterpret_cast<int32_t*>(xsum + XR * kXsStride);
   int64_t* xoff = reinterpret_cast<int64_t*>(orow + XR); // element offset of a staged row in x
   uint8_t* ring = reinterpret_cast<uint8_t*>(xoff + XR) +
@@ -208,9 +233,92 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   const uint32_t ring_lds = lds_address(ring);
 
   // ---- this workgroup's piece of the unit list ----
+  if constexpr (PLAN) {
+    const int n = a.L;
+    const int E = a.n_experts;
+    int e = E + 1; // no pair
+    if (tid < n) {
+      const uint32_t xi = a.lhs_indices[tid];
+      const uint32_t wi = a.rhs_indices[tid];
+      e = (xi < static_cast<uint32_t>(a.x_batches) && wi < static_cast<uint32_t>(E))
+          ? static_cast<int>(wi) : E; // E: a pair with an index out of range
+    }
+    int rank = 0;
+    for (int ee = 0; ee < E; ++ee) {
+      const uint64_t mask = __ballot(e == ee);
+      if (lane == 0) {
+        lwave[wave * (kSlPlanExperts + 1) + ee] = __popcll(mask);
+      }
+      if (e == ee) {
+        rank = __builtin_amdgcn_mbcnt_hi(
+            static_cast<uint32_t>(mask >> 32),
+            __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0));
+      }
+    }
+    __syncthreads();
+    if (tid < E) { // counts per expert; the wavefronts' counts become their bases
+      int sum = 0;
+      for (int w = 0; w < kSlWaves; ++w) {
+        const int c = lwave[w * (kSlPlanExperts + 1) + tid];
+        lwave[w * (kSlPlanExperts + 1) + tid] = sum;
+        sum += c;
+      }
+      lcnt[tid] = sum;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      int pos = 0;
+      int tile = 0;
+      for (int ee = 0; ee < E; ++ee) {
+        lpos[ee] = pos;
+        lfirst[ee] = tile;
+        pos += lcnt[ee];
+        tile += (lcnt[ee] + 31) / 32;
+      }
+      lnum[0] = tile;
+      lnum[1] = pos;
+    }
+    __syncthreads();
+    if (tid < E) {
+      const int c = lcnt[tid];
+      int t = lfirst[tid];
+      for (int r = 0; r < c; r += 32, ++t) {
+        ltiles[3 * t + 0] = tid;
+        ltiles[3 * t + 1] = lpos[tid] + r;
+        ltiles[3 * t + 2] = c - r < 32 ? c - r : 32;
+      }
+    }
+    if (e < E) {
+      lperm[lpos[e] + lwave[wave * (kSlPlanExperts + 1) + e] + rank] = tid;
+    }
+    __syncthreads();
+    if (blockIdx.x == 0) {
+      // for the kernel that adds up the planes; rows of pairs that name no
+      // expert or no x are zero
+      int32_t* gperm = const_cast<int32_t*>(a.group_perm);
+      int32_t* gnum = const_cast<int32_t*>(a.group_ntiles);
+      if (tid < lnum[1]) {
+        gperm[tid] = lperm[tid];
+      }
+      if (tid < 2) {
+        gnum[tid] = lnum[tid];
+      }
+      if (e == E) {
+        T* row = static_cast<T*>(a.out) + static_cast<size_t>(tid) * N;
+        for (int c = 0; c < N; ++c) {
+          row[c] = static_cast<T>(0.0f);
+        }
+      }
+    }
+  }
+  auto tile_field = [&](int t, int f) {
+    const int v = PLAN ? ltiles[3 * t + f] : a.group_tiles[3 * t + f];
+    return __builtin_amdgcn_readfirstlane(v);
+  };
+  auto perm_at = [&](int pos) { return PLAN ? lperm[pos] : a.group_perm[pos]; };
   int owners;
   if constexpr (GROUPED) {
-    owners = __builtin_amdgcn_readfirstlane(*a.group_ntiles);
+    owners = __builtin_amdgcn_readfirstlane(PLAN ? lnum[0] : *a.group_ntiles);
   } else {
     owners = a.L;
   }
@@ -226,7 +334,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   auto resolve = [&](SlabUnit<T>& u) {
     int64_t e = u.owner;
     if constexpr (GROUPED) {
-      e = __builtin_amdgcn_readfirstlane(a.group_tiles[3 * u.owner]);
+      e = tile_field(u.owner, 0);
     }
     u.w = reinterpret_cast<const uint8_t*>(a.w + e * a.w_batch_stride);
     u.scales = static_cast<const T*>(a.scales) + e * a.sb_batch_stride;
@@ -315,8 +423,8 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   int row0 = 0;    // grouped: first sorted position of the tile
   auto stage_x = [&](const SlabUnit<T>& u) {
     if constexpr (GROUPED) {
-      row0 = __builtin_amdgcn_readfirstlane(a.group_tiles[3 * u.owner + 1]);
-      M = __builtin_amdgcn_readfirstlane(a.group_tiles[3 * u.owner + 2]);
+      row0 = tile_field(u.owner, 1);
+      M = tile_field(u.owner, 2);
     }
     if (tid < XR) {
       int row = -1;
@@ -324,7 +432,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
       if (tid < M) {
         if constexpr (GROUPED) {
           // planes are indexed by sorted position, y by index pair
-          const int pair = a.group_perm[row0 + tid];
+          const int pair = perm_at(row0 + tid);
           row = R > 1 ? row0 + tid : pair;
           off = static_cast<int64_t>(a.lhs_indices[pair]) * a.x_batch_stride;
         } else {
@@ -743,11 +851,11 @@ __global__ __launch_bounds__(256) void slab_reduce_grouped_kernel(
   *reinterpret_cast<uint2*>(out + static_cast<int64_t>(perm[pos]) * N + n) = packed;
 }
 
-template <typename T, int GS, int MT, bool GROUPED>
+template <typename T, int GS, int MT, int MODE>
 int launch_one(const QmmArgs& a, const SlabPlan& pl, hipStream_t s) {
-  constexpr size_t smem = slab_smem_bytes<GS, MT>();
+  constexpr size_t smem = slab_smem_bytes<GS, MT, MODE>();
   static_assert(smem <= 160 * 1024, "LDS of a compute unit");
-  auto kern = qmm_slab_kernel<T, GS, MT, GROUPED>;
+  auto kern = qmm_slab_kernel<T, GS, MT, MODE>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -763,20 +871,20 @@ int launch_one(const QmmArgs& a, const SlabPlan& pl, hipStream_t s) {
 
 // (32-wide groups with two tiles of x would need more LDS than a compute unit
 // has: qmm_slab_supported() keeps them out)
-template <bool GROUPED>
+template <int MODE>
 int launch_any(const QmmArgs& a, const SlabPlan& pl, int gs, int dtype, int mt, hipStream_t s) {
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     if (mt == 1) {
-      return gs == 32 ? launch_one<T, 32, 1, GROUPED>(a, pl, s)
-                      : (gs == 64 ? launch_one<T, 64, 1, GROUPED>(a, pl, s)
-                                  : launch_one<T, 128, 1, GROUPED>(a, pl, s));
+      return gs == 32 ? launch_one<T, 32, 1, MODE>(a, pl, s)
+                      : (gs == 64 ? launch_one<T, 64, 1, MODE>(a, pl, s)
+                                  : launch_one<T, 128, 1, MODE>(a, pl, s));
     }
     if (gs == 32) {
       return fail(MLXROCM_UNSUPPORTED, "[qmm] slab kernel: 32-wide groups with more than 16 rows");
     }
-    return gs == 64 ? launch_one<T, 64, 2, GROUPED>(a, pl, s)
-                    : launch_one<T, 128, 2, GROUPED>(a, pl, s);
+    return gs == 64 ? launch_one<T, 64, 2, MODE>(a, pl, s)
+                    : launch_one<T, 128, 2, MODE>(a, pl, s);
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
 }
@@ -829,7 +937,7 @@ int launch_qmm_slab(const QmmArgs& a, int gs, int bits, int dtype, void* planes,
   SlabPlan pl = make_plan(a.N, a.K, a.L);
   pl.planes = static_cast<float*>(planes);
   pl.plane_elems = static_cast<int64_t>(a.L) * a.M * a.N;
-  int rc = launch_any<false>(a, pl, gs, dtype, mt, s);
+  int rc = launch_any<0>(a, pl, gs, dtype, mt, s);
   if (rc != MLXROCM_OK || pl.ranges <= 1) {
     return rc;
   }
@@ -844,14 +952,21 @@ size_t qmm_slab_grouped_plane_bytes(int n_indices, int N, int K) {
   return ranges <= 1 ? 0 : static_cast<size_t>(ranges) * n_indices * N * sizeof(float);
 }
 
+bool qmm_slab_plans_in_kernel(int n_indices, int n_experts) {
+  return n_indices <= kSlPlanPairs && n_experts <= kSlPlanExperts;
+}
+
 int launch_qmm_slab_grouped(
-    const QmmArgs& a, int gs, int bits, int dtype, void* planes, hipStream_t s) {
+    const QmmArgs& a, int gs, int bits, int dtype, void* planes, bool plan_in_kernel,
+    hipStream_t s) {
   (void)bits;
   SlabPlan pl = make_plan(
       a.N, a.K, gather_group_max_tiles(a.L, a.n_experts, kGroupSmallTile));
   pl.planes = static_cast<float*>(planes);
   pl.plane_elems = static_cast<int64_t>(a.L) * a.N;
-  int rc = launch_any<true>(a, pl, gs, dtype, 2, s);
+  // (mode 1 never runs with one tile of x: instantiating it would only cost build time)
+  int rc = plan_in_kernel ? launch_any<2>(a, pl, gs, dtype, 2, s)
+                          : launch_any<1>(a, pl, gs, dtype, 2, s);
   if (rc != MLXROCM_OK || pl.ranges <= 1) {
     return rc;
   }
