@@ -200,6 +200,58 @@ int mlxrocm_qmm(
     mlxrocm_stream_t stream);
 
 /*
+ * Prefill calls (16-bit types, transpose != 0, M >= 512) first transpose scales
+ * and biases to [K / group_size][N] so that consecutive rows of W read
+ * consecutive values (a few MB, about 5 us per call).  Weights do not change
+ * between calls: a caller that keeps that image beside a weight skips the
+ * pre-pass.  The reference has no such cache -- its GPU backends read scales in
+ * the caller's layout (mlx/backend/cuda/quantized/qmm/qmm.cu:143-146,
+ * mlx/backend/metal/quantized.cpp:1799-1801); an eval_gpu body would hang the
+ * image on the weight array's sibling list or key it by the scales' buffer.
+ *
+ * mlxrocm_qmm_sb_image_size: bytes of the image of `batches` weight matrices.
+ * mlxrocm_qmm_sb_image: builds it (scales / biases [batches][N][K / group_size],
+ * sb_batch_stride elements apart; image 16-byte aligned device memory).
+ * mlxrocm_qmm_prepacked: mlxrocm_qmm with the image as an extra argument (NULL:
+ * exactly mlxrocm_qmm).  Shapes that do not read an image ignore it; results
+ * are those of mlxrocm_qmm bit for bit.  The workspace may then be smaller than
+ * mlxrocm_qmm_workspace_size by mlxrocm_qmm_sb_image_size rounded up to 256.
+ */
+size_t mlxrocm_qmm_sb_image_size(int N, int K, int batches, int group_size, int dtype);
+int mlxrocm_qmm_sb_image(
+    const void* scales,
+    const void* biases,
+    void* image,
+    int N,
+    int K,
+    int batches,
+    int64_t sb_batch_stride,
+    int group_size,
+    int dtype,
+    mlxrocm_stream_t stream);
+int mlxrocm_qmm_prepacked(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    const void* sb_image,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t sb_batch_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream);
+
+/*
  * mlxrocm_qmm without the workspace argument, for callers that cannot
  * allocate device memory at all (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the

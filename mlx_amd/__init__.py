@@ -3,6 +3,11 @@
 with the reference's operator names and semantics, backed by hand-written HIP
 kernels through the C ABI declared in ``include/mlx_rocm_qmm.h``."""
 from . import nn
-from .ops import dequantize, gather_qmm, quantize, quantized_matmul, quantized_swiglu
+from .ops import (
+    dequantize, gather_qmm, quantize, quantized_matmul, quantized_matmul_sb_image, quantized_swiglu,
+)
 
-__all__ = ["quantize", "dequantize", "quantized_matmul", "quantized_swiglu", "gather_qmm", "nn"]
+__all__ = [
+    "quantize", "dequantize", "quantized_matmul", "quantized_matmul_sb_image", "quantized_swiglu",
+    "gather_qmm", "nn",
+]

@@ -35,6 +35,12 @@ SIGNATURES = {
         _i,
         [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p, _sz, _p],
     ),
+    "mlxrocm_qmm_sb_image_size": (_sz, [_i] * 5),
+    "mlxrocm_qmm_sb_image": (_i, [_p, _p, _p, _i, _i, _i, _i64, _i, _i, _p]),
+    "mlxrocm_qmm_prepacked": (
+        _i,
+        [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p, _sz, _p],
+    ),
     "mlxrocm_qmm_static": (
         _i,
         [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _p],

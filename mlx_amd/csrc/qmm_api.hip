@@ -124,6 +124,9 @@ struct Scratch {
   size_t bytes = 0;
   bool dry = false;
   size_t need = 0;
+  // Optional: the caller's transposed image of scales and biases
+  // (mlxrocm_qmm_sb_image); the prefill path then skips its pre-pass.
+  const void* sb_image = nullptr;
 };
 
 constexpr size_t kScratchAlign = 256;
@@ -270,24 +273,33 @@ int run_qmm_t_transposed_sb(
     const QmmArgs& a, int gs, int bits, int dtype, int k_splits, Scratch& sc, hipStream_t s) {
   const int G = a.K / gs;
   const int batches = a.sb_batch_stride == 0 ? 1 : a.L;
-  const size_t sb_bytes = (qmm_n_sb_bytes(a.N, G, batches, dtype) + 255) / 256 * 256;
+  const bool prepacked = sc.sb_image != nullptr;
+  const size_t sb_bytes =
+      prepacked ? 0 : (qmm_n_sb_bytes(a.N, G, batches, dtype) + 255) / 256 * 256;
   const size_t plane = static_cast<size_t>(a.M) * a.N;
   const size_t partial_bytes = k_splits > 1 ? plane * k_splits * sizeof(float) : 0;
   void* region = nullptr;
-  int rc = claim(sc, sb_bytes + partial_bytes, &region);
+  int rc = MLXROCM_OK;
+  if (sb_bytes + partial_bytes != 0) {
+    rc = claim(sc, sb_bytes + partial_bytes, &region);
+  }
   if (rc != MLXROCM_OK || sc.dry) {
     return rc;
   }
-  // rows of the source are the N rows of W, columns its G groups
-  rc = transpose_sb_for_qmm_n(
-      a.scales, a.biases, region, a.N, G, batches, a.sb_batch_stride, dtype, s);
-  if (rc != MLXROCM_OK) {
-    return rc;
+  const void* sb = sc.sb_image;
+  if (!prepacked) {
+    // rows of the source are the N rows of W, columns its G groups
+    rc = transpose_sb_for_qmm_n(
+        a.scales, a.biases, region, a.N, G, batches, a.sb_batch_stride, dtype, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    sb = region;
   }
   const size_t image = static_cast<size_t>(a.N) * G;
   QmmArgs part = a;
-  part.scales = region;
-  part.biases = static_cast<char*>(region) + image * dtype_size(dtype);
+  part.scales = sb;
+  part.biases = static_cast<const char*>(sb) + image * dtype_size(dtype);
   part.sb_batch_stride = batches == 1 ? 0 : static_cast<int64_t>(2 * image);
   part.sb_transposed = 1;
   if (k_splits <= 1) {
@@ -778,6 +790,73 @@ extern "C" int mlxrocm_qmm(
   Scratch sc;
   sc.base = static_cast<char*>(workspace);
   sc.bytes = workspace != nullptr ? workspace_bytes : 0;
+  return qmm_entry(
+      x, wq, scales, biases, out, M, N, K, L, x_batch_stride, w_batch_stride,
+      sb_batch_stride, group_size, bits, dtype, transpose, sc,
+      static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t mlxrocm_qmm_sb_image_size(int N, int K, int batches, int group_size, int dtype) {
+  if (N <= 0 || K <= 0 || batches <= 0 || group_size <= 0 || K % group_size != 0) {
+    return 0;
+  }
+  return qmm_n_sb_bytes(N, K / group_size, batches, dtype);
+}
+
+extern "C" int mlxrocm_qmm_sb_image(
+    const void* scales,
+    const void* biases,
+    void* image,
+    int N,
+    int K,
+    int batches,
+    int64_t sb_batch_stride,
+    int group_size,
+    int dtype,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_qmm_sb_image");
+  if (N <= 0 || K <= 0 || batches <= 0 || (group_size != 32 && group_size != 64 && group_size != 128) ||
+      K % group_size != 0 || sb_batch_stride < 0 ||
+      (dtype != MLXROCM_FLOAT32 && dtype != MLXROCM_FLOAT16 && dtype != MLXROCM_BFLOAT16)) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[qmm_sb_image] invalid shape or dtype");
+  }
+  if (!scales || !biases || !image) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[qmm_sb_image] null device pointer");
+  }
+  return transpose_sb_for_qmm_n(
+      scales, biases, image, N, K / group_size, batches, sb_batch_stride, dtype,
+      static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mlxrocm_qmm_prepacked(
+    const void* x,
+    const uint32_t* wq,
+    const void* scales,
+    const void* biases,
+    const void* sb_image,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t sb_batch_stride,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_qmm_prepacked");
+  if (sb_image != nullptr && (reinterpret_cast<uintptr_t>(sb_image) & 15u) != 0) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] the image must be 16-byte aligned");
+  }
+  Scratch sc;
+  sc.base = static_cast<char*>(workspace);
+  sc.bytes = workspace != nullptr ? workspace_bytes : 0;
+  sc.sb_image = transpose != 0 ? sb_image : nullptr;
   return qmm_entry(
       x, wq, scales, biases, out, M, N, K, L, x_batch_stride, w_batch_stride,
       sb_batch_stride, group_size, bits, dtype, transpose, sc,

@@ -60,9 +60,23 @@ class QuantizedLinear(torch.nn.Module):
         return (f"input_dims={in_dims}, output_dims={out_dims}, bias={self.bias is not None}, "
                 f"group_size={self.group_size}, bits={self.bits}, mode={self.mode}")
 
+    def prepack(self) -> "QuantizedLinear":
+        """Keeps the transposed image of scales and biases that prefill calls
+        (512 rows of x and more) would otherwise rebuild on every call.  Not in
+        the reference; call again after changing the weights."""
+        self._sb_image = ops.quantized_matmul_sb_image(self.scales, self.biases, self.group_size)
+        self._sb_image_of = (self.scales.data_ptr(), self.biases.data_ptr())
+        return self
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        image = getattr(self, "_sb_image", None)
+        if image is not None and (
+                self._sb_image_of != (self.scales.data_ptr(), self.biases.data_ptr())
+                or torch.promote_types(x.dtype, self.scales.dtype) != image.dtype):
+            image = None  # weights replaced, or a product in another type
         y = ops.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
-                                 group_size=self.group_size, bits=self.bits, mode=self.mode)
+                                 group_size=self.group_size, bits=self.bits, mode=self.mode,
+                                 sb_image=image)
         if self.bias is not None:
             y = y + self.bias
         return y

@@ -327,8 +327,13 @@ def quantized_matmul(
     group_size: Optional[int] = None,
     bits: Optional[int] = None,
     mode: str = "affine",
+    *,
+    sb_image: Optional[torch.Tensor] = None,
 ):
-    """``mx.quantized_matmul`` (mlx/ops.cpp:4784-4834)."""
+    """``mx.quantized_matmul`` (mlx/ops.cpp:4784-4834).  ``sb_image`` (not in
+    the reference): the result of :func:`quantized_matmul_sb_image` for these
+    scales and biases, which saves prefill calls their transposition pre-pass;
+    results do not depend on it."""
     dtype, mode = _validate_mode_with_type("quantized_matmul", scales, biases, None, mode)
     group_size, bits = _params_from_mode(mode, group_size, bits)
     _, w_outer = _extract_dims(
@@ -380,15 +385,57 @@ def quantized_matmul(
     )
     # a temporary of the call, like the ones eval_gpu hands to add_temporary
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    if sb_image is not None:
+        want = lib.mlxrocm_qmm_sb_image_size(
+            w_outer, K, L if sb_stride else 1, group_size, code)
+        if (not transpose or sb_image.dtype != dtype or sb_image.device != x.device
+                or not sb_image.is_contiguous() or sb_image.numel() * sb_image.element_size() != want):
+            raise ValueError(
+                "[quantized_matmul] sb_image does not belong to these scales and biases "
+                "(quantized_matmul_sb_image with the same dtype, transpose=True)"
+            )
     _lib.check(
-        lib.mlxrocm_qmm(
-            xb.data_ptr(), wb.data_ptr(), sb.data_ptr(), bb.data_ptr(), out.data_ptr(),
+        lib.mlxrocm_qmm_prepacked(
+            xb.data_ptr(), wb.data_ptr(), sb.data_ptr(), bb.data_ptr(),
+            sb_image.data_ptr() if sb_image is not None else None, out.data_ptr(),
             M, w_outer, K, L, M * K, w_stride, sb_stride, group_size, bits,
             code, int(bool(transpose)),
             ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x),
         )
     )
     return out
+
+
+def quantized_matmul_sb_image(
+    scales: torch.Tensor,
+    biases: torch.Tensor,
+    group_size: int = 64,
+    dtype: Optional[torch.dtype] = None,
+) -> torch.Tensor:
+    """Scales and biases of ``[..., N, K / group_size]`` weights transposed to the
+    ``[K / group_size][N]`` image the prefill kernels read, to be kept beside a
+    weight and passed to ``quantized_matmul(..., sb_image=...)``.  ``dtype``: the
+    type the product will run in (that of x after promotion; default: that of
+    the scales).  No counterpart in the reference."""
+    dtype = dtype or scales.dtype
+    _require_gpu("quantized_matmul_sb_image", scales, biases)
+    if scales.shape != biases.shape or scales.dim() < 2:
+        raise ValueError("[quantized_matmul_sb_image] scales and biases must have one shape")
+    lib = _lib.load()
+    s = _contiguous(_astype(scales, dtype))
+    b = _contiguous(_astype(biases, dtype))
+    N, G = s.shape[-2], s.shape[-1]
+    batches = s.numel() // (N * G)
+    code = _DTYPE_CODE[dtype]
+    nbytes = lib.mlxrocm_qmm_sb_image_size(N, G * group_size, batches, group_size, code)
+    image = torch.empty(nbytes // s.element_size(), dtype=dtype, device=s.device)
+    _lib.check(
+        lib.mlxrocm_qmm_sb_image(
+            s.data_ptr(), b.data_ptr(), image.data_ptr(), N, G * group_size, batches,
+            N * G, group_size, code, _stream_ptr(s),
+        )
+    )
+    return image
 
 
 def _indices_or_default(tag, indices, t):

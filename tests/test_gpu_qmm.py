@@ -519,3 +519,32 @@ def test_prefill_call_replays_from_a_hip_graph(oracle, gpu):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {i}"
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_qmm_prepacked_scale_image(gpu, dtype):
+    """A prefill call that is handed the transposed scale / bias image of its
+    weight skips the pre-pass and returns the bits of the plain call; shapes that
+    read no image ignore it; an image of another weight shape is refused."""
+    N, K, gs = 1024, 2048, 64
+    w = normal_weights((N, K), dtype, std=0.05).to(gpu)
+    wq, s, b = mlx_amd.quantize(w, gs, 4)
+    image = mlx_amd.quantized_matmul_sb_image(s, b, gs)
+    assert image.numel() == 2 * N * (K // gs) and image.dtype == dtype
+    # the image is the two arrays transposed, scales first
+    assert torch.equal(image[: N * (K // gs)].reshape(K // gs, N), s.T.contiguous())
+    assert torch.equal(image[N * (K // gs):].reshape(K // gs, N), b.T.contiguous())
+    for M in (1, 8, 600, 2048):
+        x = activations((M, K), dtype).to(gpu)
+        plain = mlx_amd.quantized_matmul(x, wq, s, b, True, gs, 4)
+        packed = mlx_amd.quantized_matmul(x, wq, s, b, True, gs, 4, sb_image=image)
+        assert torch.equal(plain, packed), M
+    with pytest.raises(ValueError):
+        mlx_amd.quantized_matmul(x, wq, s, b, True, gs, 4, sb_image=image[:-8])
+    # the layer keeps the image and drops it when the weights are replaced
+    lin = mlx_amd.nn.QuantizedLinear(K, N, bias=False, device=gpu, dtype=dtype)
+    x = activations((640, K), dtype).to(gpu)
+    before = lin(x)
+    assert torch.equal(lin.prepack()(x), before)
+    lin._set_quantized(w)
+    assert torch.equal(lin(x), mlx_amd.quantized_matmul(x, wq, s, b, True, gs, 4))
