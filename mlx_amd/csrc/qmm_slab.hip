@@ -823,6 +823,314 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// ---------------------------------------------------------------------------
+// Up to 8 rows of x with all of K resident: the same arithmetic without ranges,
+// planes or a unit list.  A workgroup of 4 wavefronts owns 64 rows of W (one
+// 16-row tile per wavefront) and keeps the rows of x for the whole of K in LDS
+// (M * K * 2 bytes <= 64 KiB), so every element of y is finished where it is
+// computed.  Scales and biases of a wavefront's 16 rows go to LDS by DMA once,
+// the packed codes through a ring of four 256-code steps.  Grid: N / 64
+// workgroups per problem -- one per compute unit for the shapes it is used for.
+constexpr int kR8Tiles = 4;              // 16-row tiles of W per workgroup
+constexpr int kR8Rows = 16 * kR8Tiles;
+constexpr int kR8SlotBytes = 16 * kSlStep / 2;
+constexpr int kR8MaxXBytes = 64 * 1024;
+
+// kw: wavefronts per tile (each takes 1 / kw of the K steps); stages: ring slots
+// per wavefront
+inline size_t rows8_smem_bytes(int M, int K, int gs, int kw, int stages) {
+  const size_t groups = K / gs;
+  const size_t sums = (static_cast<size_t>(M) * (groups + 1) * 4 + 15) / 16 * 16;
+  return static_cast<size_t>(M) * (2 * K + 16) + sums +
+      static_cast<size_t>(kR8Tiles) * kw * stages * kR8SlotBytes +
+      static_cast<size_t>(kR8Tiles) * 2 * 16 * groups * 2;
+}
+
+__device__ __forceinline__ floatx4 quad_transpose4(floatx4 v, int lane) {
+  const bool odd = (lane & 1) != 0;
+  const bool high = (lane & 2) != 0;
+  float sx = odd ? v[0] : v[1];
+  float sy = odd ? v[2] : v[3];
+  const float px = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, sx), 0xB1, 0xf, 0xf, true));
+  const float py = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, sy), 0xB1, 0xf, 0xf, true));
+  if (odd) {
+    v[0] = px;
+    v[2] = py;
+  } else {
+    v[1] = px;
+    v[3] = py;
+  }
+  sx = high ? v[0] : v[2];
+  sy = high ? v[1] : v[3];
+  const float qx = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, sx), 0x4E, 0xf, 0xf, true));
+  const float qy = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, sy), 0x4E, 0xf, 0xf, true));
+  if (high) {
+    v[0] = qx;
+    v[1] = qy;
+  } else {
+    v[2] = qx;
+    v[3] = qy;
+  }
+  return v;
+}
+
+template <typename T, int GS, int KW, int kR8Stages>
+__global__ __launch_bounds__(64 * kR8Tiles * KW) void qmm_rows8_kernel(const QmmArgs a) {
+  constexpr int kR8Threads = 64 * kR8Tiles * KW;
+  using Shape = SlabShape<GS>;
+  constexpr int GPS = Shape::kGroupsPerStep;
+  constexpr int DW = Shape::kDwords;
+  constexpr int kChunks = GPS * DW;
+  constexpr int kAhead = (kR8Stages - 1) * 2;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15;
+  const int q = lane >> 4;
+  const int M = a.M;
+  const int N = a.N;
+  const int K = a.K;
+  const int groups = K / GS;
+  const int row_bytes = K / 2;
+  const int rbk = groups * 2;          // bytes of a row's scales
+  const int x_stride = 2 * K + 16;     // bytes
+  const int xs_stride = groups + 1;    // floats
+  const int nsteps = K / kSlStep / KW;      // steps of this wavefront
+  const int tile = wave % kR8Tiles;
+  const int kpart = wave / kR8Tiles;
+  const int step0 = kpart * nsteps;
+  const QmmProblem<T> p = resolve_problem<T>(a, blockIdx.y);
+
+  uint8_t* xl = smem;
+  float* xsum = reinterpret_cast<float*>(smem + M * x_stride);
+  uint8_t* rings = reinterpret_cast<uint8_t*>(xsum) + (M * xs_stride * 4 + 15) / 16 * 16;
+  uint8_t* ring = rings + wave * (kR8Stages * kR8SlotBytes);
+  // [16 rows][groups] scales, then biases, of the tile (fetched by its first wavefront)
+  uint8_t* sbbuf = rings + kR8Tiles * KW * (kR8Stages * kR8SlotBytes) + tile * (2 * 16 * rbk);
+  const uint32_t ring_lds = lds_address(ring);
+  const uint32_t sb_lds = lds_address(sbbuf);
+
+  const int n0 = blockIdx.x * kR8Rows + tile * 16;
+  // ---- scales and biases of the tile's rows: rbk / 64 DMAs per array,
+  // lane -> 16-byte piece (i * 64 + lane) of the [16][rbk] block
+  if (kpart == 0) {
+    const int per_row = rbk >> 4;
+    const int dmas = rbk >> 6;
+    for (int i = 0; i < dmas; ++i) {
+      const int piece = i * 64 + lane;
+      const int r = piece / per_row;
+      const int c = piece - r * per_row;
+      int n = n0 + r;
+      n = n < N ? n : N - 1;
+      const uint32_t off = static_cast<uint32_t>(n) * static_cast<uint32_t>(rbk) + c * 16;
+      dma16(p.scales, off, sb_lds + i * 1024);
+      dma16(p.biases, off, sb_lds + 16 * rbk + i * 1024);
+    }
+  }
+  // ---- W: DMA i of a step fetches tile row 8 i + lane / 8, LDS piece lane % 8
+  // <- global piece (lane % 8) ^ (row / 2 % 8)
+  uint32_t w_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = 8 * i + (lane >> 3);
+    int n = n0 + r;
+    n = n < N ? n : N - 1;
+    const int piece = (lane & 7) ^ ((r >> 1) & 7);
+    w_off[i] = static_cast<uint32_t>(n) * static_cast<uint32_t>(row_bytes) + piece * 16;
+  }
+  auto fetch = [&](int j, int slot) {
+    const int jc = step0 + (j < nsteps ? j : nsteps - 1); // past the end: again, into a free slot
+    const uint8_t* wb = p.w + jc * (kSlStep / 2);
+    const uint32_t m0 = ring_lds + slot * kR8SlotBytes;
+    dma16(wb, w_off[0], m0);
+    dma16(wb, w_off[1], m0 + 1024);
+  };
+#pragma unroll
+  for (int i = 0; i < kR8Stages - 1; ++i) {
+    fetch(i, i);
+  }
+
+  // ---- x into LDS: rows in the widened order and their group sums
+  {
+    const int per_row = K >> 3; // 16-byte pieces per row
+    const int pieces = M * per_row;
+    for (int c0 = 0; c0 < pieces; c0 += 4 * kR8Threads) {
+      uint4 xv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = c0 + i * kR8Threads + tid;
+        xv[i] = make_uint4(0u, 0u, 0u, 0u);
+        if (c < pieces) {
+          xv[i] = *reinterpret_cast<const uint4*>(p.x + static_cast<size_t>(c) * 8);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = c0 + i * kR8Threads + tid;
+        const int m = c / per_row;
+        const int col = c - m * per_row;
+        const uint4 v = xv[i];
+        uint4 w;
+        w.x = (v.x & 0xffffu) | (v.z << 16);
+        w.y = (v.x >> 16) | (v.z & 0xffff0000u);
+        w.z = (v.y & 0xffffu) | (v.w << 16);
+        w.w = (v.y >> 16) | (v.w & 0xffff0000u);
+        const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          s += to_f32(__builtin_bit_cast(T, static_cast<uint16_t>(words[k] & 0xffffu)));
+          s += to_f32(__builtin_bit_cast(T, static_cast<uint16_t>(words[k] >> 16)));
+        }
+#pragma unroll
+        for (int d = 1; d < GS / 8; d *= 2) {
+          s += __shfl_xor(s, d);
+        }
+        if (c < pieces) {
+          *reinterpret_cast<uint4*>(xl + m * x_stride + col * 16) = w;
+          if ((lane & (GS / 8 - 1)) == 0) {
+            xsum[m * xs_stride + col / (GS / 8)] = s;
+          }
+        }
+      }
+    }
+  }
+  wait_vm<kAhead>(); // the tile's scales and biases are in LDS before the barrier
+  __syncthreads();
+
+  const int xrow = r16 < M ? r16 : M - 1; // rows past M repeat the last one; their results are dropped
+  const int lane_byte = q * (GS / 8);
+  const uint32_t w_lane = r16 * 128 + ((((lane_byte >> 4) ^ (r16 >> 1)) & 7) << 4) + (lane_byte & 15);
+  const uint8_t* x_lane = xl + xrow * x_stride + 2 * (GS / 4) * q;
+  const float* xs_lane = xsum + xrow * xs_stride;
+  const uint8_t* sb_lane = sbbuf + r16 * rbk;
+  uint32_t wmask = 0x000f000fu;
+  uint32_t wmagic = WidenMagic<T>::kBits;
+  asm volatile("" : "+v"(wmask), "+v"(wmagic));
+
+  floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  int slot = 0;
+  int fslot = kR8Stages - 1;
+  for (int j = 0; j < nsteps; ++j) {
+    fetch(j + kR8Stages - 1, fslot);
+    fslot = fslot + 1 == kR8Stages ? 0 : fslot + 1;
+    const uint8_t* xs = x_lane + (step0 + j) * (2 * kSlStep);
+    uint4 xf[kChunks];
+#pragma unroll
+    for (int G = 0; G < GPS; ++G) {
+#pragma unroll
+      for (int d = 0; d < DW; ++d) {
+        xf[G * DW + d] = *reinterpret_cast<const uint4*>(xs + 2 * (GS * G + 8 * d));
+      }
+    }
+    constexpr int kCorr = (GPS + 3) / 4;
+    float xa[kCorr];
+    bool live[kCorr];
+    int gcl[kCorr];
+#pragma unroll
+    for (int h = 0; h < kCorr; ++h) {
+      const int g = 4 * h + q;
+      live[h] = g < GPS;
+      gcl[h] = live[h] ? g : 0;
+      xa[h] = xs_lane[(step0 + j) * GPS + gcl[h]];
+    }
+    wait_vm<kAhead>(); // this step's codes (and, the first time, scales and biases) have landed
+    uint32_t raw[GPS / 2];
+    T cs[kCorr], cb[kCorr];
+    {
+      const uint8_t* sp = sb_lane + (step0 + j) * (2 * GPS);
+      if constexpr (GPS == 8) {
+        const uint4 v = *reinterpret_cast<const uint4*>(sp);
+        raw[0] = v.x; raw[1] = v.y; raw[2] = v.z; raw[3] = v.w;
+      } else if constexpr (GPS == 4) {
+        const uint2 v = *reinterpret_cast<const uint2*>(sp);
+        raw[0] = v.x; raw[1] = v.y;
+      } else {
+        raw[0] = *reinterpret_cast<const uint32_t*>(sp);
+      }
+#pragma unroll
+      for (int h = 0; h < kCorr; ++h) {
+        cs[h] = *reinterpret_cast<const T*>(sp + 2 * gcl[h]);
+        cb[h] = *reinterpret_cast<const T*>(sp + 2 * gcl[h] + 16 * rbk);
+      }
+    }
+    const uint8_t* sl = ring + slot * kR8SlotBytes;
+    uint32_t wq[GPS][DW];
+#pragma unroll
+    for (int G = 0; G < GPS; ++G) {
+      const uint8_t* wp = sl + (w_lane ^ (G * (GS / 2)));
+      if constexpr (DW == 4) {
+        const uint4 v = *reinterpret_cast<const uint4*>(wp);
+        wq[G][0] = v.x; wq[G][1] = v.y; wq[G][2] = v.z; wq[G][3] = v.w;
+      } else if constexpr (DW == 2) {
+        const uint2 v = *reinterpret_cast<const uint2*>(wp);
+        wq[G][0] = v.x; wq[G][1] = v.y;
+      } else {
+        wq[G][0] = *reinterpret_cast<const uint32_t*>(wp);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int G = 0; G < GPS; ++G) {
+      floatx4 chain;
+#pragma unroll
+      for (int d = 0; d < DW; ++d) {
+        const uint4 wf = widen8(wq[G][d], wmask, wmagic);
+        const floatx4 c0 = d == 0 ? floatx4{0.0f, 0.0f, 0.0f, 0.0f} : chain;
+        chain = mfma16<T>(xf[G * DW + d], wf, c0);
+      }
+      const float scale = to_f32(__builtin_bit_cast(
+          T, static_cast<uint16_t>((raw[G / 2] >> (16 * (G & 1))) & 0xffffu)));
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        acc[r] = fmaf(scale, chain[r], acc[r]);
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < kCorr; ++h) {
+      float c = fmaf(-WidenMagic<T>::kOffset, to_f32(cs[h]), to_f32(cb[h]));
+      c = live[h] ? c : 0.0f;
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[h], c, acc, 0, 0, 0);
+    }
+    wait_lds_reads();
+    slot = slot + 1 == kR8Stages ? 0 : slot + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the refetches past the end
+
+  // the K parts of a tile meet in LDS (the ring is free now)
+  if constexpr (KW > 1) {
+    __syncthreads();
+    float* part = reinterpret_cast<float*>(rings) + (wave * 64 + lane) * 4;
+    if (kpart != 0) {
+      *reinterpret_cast<floatx4*>(part) = acc;
+    }
+    __syncthreads();
+    if (kpart != 0) {
+      return;
+    }
+#pragma unroll
+    for (int k = 1; k < KW; ++k) {
+      acc += *reinterpret_cast<const floatx4*>(part + k * kR8Tiles * 64 * 4);
+    }
+  }
+  // lane i of quad c: y[m = 4 q + i][n0 + 4 c .. + 3]
+  const floatx4 v = quad_transpose4(acc, lane);
+  const int m = 4 * q + (lane & 3);
+  const int n = n0 + (r16 & ~3);
+  if (m < M && n < N) {
+    uint2 packed;
+    packed.x = p.valid ? pack2<T>(v[0], v[1]) : 0u;
+    packed.y = p.valid ? pack2<T>(v[2], v[3]) : 0u;
+    *reinterpret_cast<uint2*>(p.out + static_cast<size_t>(m) * N + n) = packed;
+  }
+}
+
 // y[perm[pos]] (grouped) = sum over the K ranges of plane[range][pos]
 template <typename T>
 __global__ __launch_bounds__(256) void slab_reduce_grouped_kernel(
@@ -983,6 +1291,79 @@ int launch_qmm_slab_grouped(
   }
   MLXROCM_HIP_TRY(hipGetLastError());
   return MLXROCM_OK;
+}
+
+// Wavefronts per tile: as many as K has pairs of steps, at most 4.
+int rows8_kw(int K) {
+  const int steps = K / kSlStep;
+  return steps % 4 == 0 && steps >= 8 ? 4 : (steps % 2 == 0 && steps >= 4 ? 2 : 1);
+}
+
+// Ring slots per wavefront: as many as LDS leaves (2..4 with four wavefronts
+// per tile, 3 otherwise); 0: does not fit.
+int rows8_stages(int M, int K, int gs, int kw) {
+  const int steps = K / kSlStep / kw;
+  for (int st = kw == 4 ? 4 : 3; st >= (kw == 4 ? 2 : 3); --st) {
+    if (st <= steps + 1 && rows8_smem_bytes(M, K, gs, kw, st) <= 160 * 1024) {
+      return st;
+    }
+  }
+  return 0;
+}
+
+// Up to 8 rows of x whose whole K fits LDS (qmm_rows8_kernel).
+bool qmm_rows8_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose) {
+  if (!transpose || bits != 4 || dtype == MLXROCM_FLOAT32) {
+    return false;
+  }
+  if (a.M < 1 || a.M > 8 || a.N < 4 || a.N % 4 != 0 || a.L > 65535) {
+    return false;
+  }
+  // whole 64-piece DMAs of a 16-row block of scales; whole steps
+  if (a.K < 32 * gs || a.K % (32 * gs) != 0 || a.K % kSlStep != 0) {
+    return false;
+  }
+  if (static_cast<size_t>(a.M) * (2 * a.K + 16) > kR8MaxXBytes + 8 * 16 ||
+      rows8_stages(a.M, a.K, gs, rows8_kw(a.K)) == 0) {
+    return false;
+  }
+  return static_cast<int64_t>(a.N) * (a.K / 2) < (int64_t{1} << 32);
+}
+
+int launch_qmm_rows8(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  (void)bits;
+  const int kw = rows8_kw(a.K);
+  const int stages = rows8_stages(a.M, a.K, gs, kw);
+  const size_t smem = rows8_smem_bytes(a.M, a.K, gs, kw, stages);
+  const dim3 grid((a.N + kR8Rows - 1) / kR8Rows, a.L);
+  auto go = [&](auto kern) -> int {
+    static bool configured = false; // per instantiation
+    if (!configured) {
+      MLXROCM_HIP_TRY(hipFuncSetAttribute(
+          reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+          160 * 1024));
+      configured = true;
+    }
+    kern<<<grid, 64 * kR8Tiles * kw, smem, s>>>(a);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
+  };
+  auto run = [&](auto tval) -> int {
+    using T = decltype(tval);
+    auto with = [&](auto kwv, auto stv) -> int {
+      constexpr int KW = decltype(kwv)::value;
+      constexpr int ST = decltype(stv)::value;
+      return gs == 32 ? go(qmm_rows8_kernel<T, 32, KW, ST>)
+                      : (gs == 64 ? go(qmm_rows8_kernel<T, 64, KW, ST>)
+                                  : go(qmm_rows8_kernel<T, 128, KW, ST>));
+    };
+    if (kw == 4) {
+      return stages == 4 ? with(IntC<4>{}, IntC<4>{})
+                         : (stages == 3 ? with(IntC<4>{}, IntC<3>{}) : with(IntC<4>{}, IntC<2>{}));
+    }
+    return kw == 2 ? with(IntC<2>{}, IntC<3>{}) : with(IntC<1>{}, IntC<3>{});
+  };
+  return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
 }
 
 } // namespace mlxrocm

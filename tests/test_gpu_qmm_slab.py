@@ -119,3 +119,30 @@ def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T):
     keep = torch.ones((T, 2), dtype=torch.bool, device=gpu)
     keep[7, 1] = False
     assert torch.equal(got_bad[keep], got[keep])
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("gs,K", ((64, 4096), (64, 2048), (32, 1024), (128, 4096)))
+def test_rows8_all_of_k_resident(oracle, gpu, dtype, gs, K):
+    """5..8 rows of x kept in LDS for the whole of K: four, two (K = 2048) or one
+    (K = 1024) wavefronts per 16-row tile of W, N with a ragged last workgroup."""
+    N = 8200
+    w = normal_weights((N, K), dtype, std=0.05)
+    quantized = oracle.quantize(w, gs, 4)
+    for M in (5, 8):
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, None, gs, 4, rows=torch.tensor([M - 1]), quantized=quantized)
+        ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, 4, CODE[dtype], 1)
+        assert ws == 0, "the shape did not take the kernel without K ranges"
+
+
+def test_rows8_batched(oracle, gpu):
+    L, M, N, K = 3, 7, 4096, 4096
+    dtype = torch.bfloat16
+    w = normal_weights((L, N, K), dtype, std=0.05)
+    wq, s, b = oracle.quantize(w, 64, 4)
+    x = activations((L, M, K), dtype)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq.to(gpu), s.to(gpu), b.to(gpu), True, 64, 4).cpu()
+    w_hat = exact_affine_weights(wq, s, b, 64, 4)
+    exact = torch.einsum("lmk,lnk->lmn", x.double(), w_hat)
+    assert float((got.double() - exact).abs().max()) <= exact_tolerance(dtype, K, x, w_hat, exact)
