@@ -400,11 +400,12 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
   // workgroups fill their last round of compute units (4096, 11008, 12288 or
   // 28672 rows at K = 4096); at 6144 or 14336 rows the last round is half
   // empty and the 32-row MFMA GEMV is 4-12 % ahead.
-  // 5..8 rows of 4-bit codes whose x fits LDS for all of K: no K ranges, no
-  // planes (14336 x 4096: 11.7-12.2 us against 15.3-15.7 for the kernels below,
-  // 8192 x 2048: 6.8-7.2 against 8.5-8.9; with up to 4 rows the 4x4x4 kernel stays
+  // 5..16 rows of 4-bit codes whose x fits LDS for all of K (8 rows at K = 4096,
+  // 16 at K = 2048): no K ranges, no planes (14336 x 4096: 11.7-12.2 us against
+  // 15.3-15.7 for the kernels below, 8192 x 2048: 6.8-7.4 against 8.5-10.4,
+  // 16384 x 2048, 16 rows: 9.0 against 15.0; with up to 4 rows the 4x4x4 kernel stays
   // ahead, and 4096 x 4096 has too few 64-row workgroups: 9.8 against 7.1 us)
-  if (transpose && a.M >= 5 && a.M <= 8 && a.lhs_indices == nullptr && a.w_alt == nullptr &&
+  if (transpose && a.M >= 5 && a.M <= 16 && a.lhs_indices == nullptr && a.w_alt == nullptr &&
       a.group_tiles == nullptr && qmm_rows8_supported(a, gs, bits, dtype, transpose) &&
       2L * ((a.N + 63) / 64) * a.L >= compute_units()) {
     return MLXROCM_LAUNCH(sc, launch_qmm_rows8(a, gs, bits, dtype, s));

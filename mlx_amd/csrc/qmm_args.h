@@ -127,7 +127,7 @@ int launch_qmm_skinny_grouped(const QmmArgs& a, int gs, int bits, int dtype, hip
 // K range the partial sums go through fp32 planes (`planes`, *_plane_bytes()).
 bool qmm_slab_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 bool qmm_slab_shape_ok(int rows, int N, int K, int gs, int bits);
-// Up to 8 rows of x with M * K * 2 bytes <= 64 KiB of LDS: all of K resident, no planes.
+// Up to 16 rows of x with M * K * 2 bytes <= 64 KiB of LDS: all of K resident, no planes.
 bool qmm_rows8_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmm_rows8(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 long qmm_slab_units(const QmmArgs& a); // work items of a plain call

@@ -824,7 +824,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
 }
 
 // ---------------------------------------------------------------------------
-// Up to 8 rows of x with all of K resident: the same arithmetic without ranges,
+// Up to 16 rows of x with all of K resident: the same arithmetic without ranges,
 // planes or a unit list.  A workgroup of 4 wavefronts owns 64 rows of W (one
 // 16-row tile per wavefront) and keeps the rows of x for the whole of K in LDS
 // (M * K * 2 bytes <= 64 KiB), so every element of y is finished where it is
@@ -1311,19 +1311,19 @@ int rows8_stages(int M, int K, int gs, int kw) {
   return 0;
 }
 
-// Up to 8 rows of x whose whole K fits LDS (qmm_rows8_kernel).
+// Up to 16 rows of x whose whole K fits LDS (qmm_rows8_kernel).
 bool qmm_rows8_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose) {
   if (!transpose || bits != 4 || dtype == MLXROCM_FLOAT32) {
     return false;
   }
-  if (a.M < 1 || a.M > 8 || a.N < 4 || a.N % 4 != 0 || a.L > 65535) {
+  if (a.M < 1 || a.M > 16 || a.N < 4 || a.N % 4 != 0 || a.L > 65535) {
     return false;
   }
   // whole 64-piece DMAs of a 16-row block of scales; whole steps
   if (a.K < 32 * gs || a.K % (32 * gs) != 0 || a.K % kSlStep != 0) {
     return false;
   }
-  if (static_cast<size_t>(a.M) * (2 * a.K + 16) > kR8MaxXBytes + 8 * 16 ||
+  if (static_cast<size_t>(a.M) * (2 * a.K + 16) > kR8MaxXBytes + 16 * 16 ||
       rows8_stages(a.M, a.K, gs, rows8_kw(a.K)) == 0) {
     return false;
   }

@@ -124,12 +124,13 @@ def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T):
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
 @pytest.mark.parametrize("gs,K", ((64, 4096), (64, 2048), (32, 1024), (128, 4096)))
 def test_rows8_all_of_k_resident(oracle, gpu, dtype, gs, K):
-    """5..8 rows of x kept in LDS for the whole of K: four, two (K = 2048) or one
-    (K = 1024) wavefronts per 16-row tile of W, N with a ragged last workgroup."""
+    """5..8 rows of x (up to 16 at K <= 2048) kept in LDS for the whole of K, the
+    K steps split over the wavefronts of a tile; N with a ragged last workgroup."""
     N = 8200
     w = normal_weights((N, K), dtype, std=0.05)
     quantized = oracle.quantize(w, gs, 4)
-    for M in (5, 8):
+    rows = (5, 8) + ((12, 16) if K <= 2048 else ())  # M * K * 2 bytes <= 64 KiB
+    for M in rows:
         x = activations((M, K), dtype, seed=M)
         _check_qmm(oracle, gpu, x, None, gs, 4, rows=torch.tensor([M - 1]), quantized=quantized)
         ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, 4, CODE[dtype], 1)
