@@ -1,21 +1,23 @@
-// qmm_slab.hip -- transpose=true products of 4-bit weights with up to 32 rows of
-// x per weight matrix (16-bit element types): 9..32 rows of a plain call and the
+// qmm_slab.hip -- transpose=true products of 4-bit weights with a few rows of x
+// per weight matrix (16-bit element types): 5..32 rows of a plain call and the
 // small expert groups of a gather.
 //
 //   y[M, N] = x[M, K] * dequant(W)[N, K]^T
 //
 // The weights are read once and the work is bound by that stream.  What the
-// kernel is built around:
+// kernels here are built around:
 //   * packed codes go from HBM to LDS without passing through registers
 //     (global_load_lds_dwordx4): a wavefront instruction fetches 8 rows x 128
-//     bytes, whole cache lines, into a ring of four 256-code steps that is
-//     private to the wavefront -- no workgroup barrier in the loop, the only
+//     bytes, whole cache lines, into a ring of 256-code steps that is private
+//     to the wavefront -- no workgroup barrier in the loop, the only
 //     synchronisation is the wavefront's own vmcnt;
-//   * x does not move while weights stream: a workgroup keeps MT x 16 rows of
-//     one K range (1024 or 2048 codes) in LDS and walks the slabs of 128 weight
-//     rows with it; a launch is a flat list of units (x rows, K range, slab)
-//     cut into equal consecutive pieces, one per workgroup, so that x is staged
-//     once or twice per workgroup;
+//   * x does not move while weights stream.  qmm_slab_kernel: a workgroup of 8
+//     wavefronts keeps 16 or 32 rows of one 1024-code K range in LDS and walks
+//     slabs of 256 weight rows with it; a launch is a flat list of units (x rows
+//     of a problem or expert tile, K range, slab) cut into equal consecutive
+//     pieces, one per workgroup, so that x is staged once or twice per
+//     workgroup.  qmm_rows8_kernel: up to 16 rows of x whose whole K fits LDS,
+//     one launch workgroup per 64 weight rows, no K ranges;
 //   * codes are widened without arithmetic (OR into the mantissa of 128.0 /
 //     1024.0) and multiplied as they are: per quantization group one chain of
 //     v_mfma_f32_16x16x32 starting from zero, then acc += scale * chain (four
@@ -23,8 +25,12 @@
 //     sum_g X[m][g] * (bias[n][g] - offset * scale[n][g]) with X the sums of x
 //     over a group, is one v_mfma_f32_16x16x4_f32 per tile and four groups on
 //     exact fp32 operands;
+//   * scales and biases arrive once per unit (whole 32- or 64-byte runs of a
+//     row per load), results leave one step after their unit ended (stores
+//     count in vmcnt like loads);
 //   * the K ranges of a row of y are added up from fp32 planes by a second
-//     small kernel (one range: written directly).
+//     small kernel (one range: written directly);
+//   * a gather of up to 512 index pairs is grouped by expert inside the kernel.
 // LDS reads are free of bank conflicts by construction: the 16-byte pieces of a
 // weight row are stored at piece ^ (row / 2 % 8), rows of x are 16 bytes longer
 // than a power of two.
