@@ -319,7 +319,7 @@ def sweep(torch, mlx_amd, dev) -> list:
     E, n, k = 8, 14336, 4096
     wq, sc, bi = mlx_amd.quantize(
         (torch.randn((E, n, k), generator=g, dtype=torch.float32) * 0.02).to(bf16).to(dev), 64, 4)
-    for T in (1, 64, 2048):
+    for T in (1, 8, 64, 2048):
         x = torch.randn((T, 1, 1, k), generator=g, dtype=torch.float32).to(bf16).to(dev)
         idx = torch.randint(0, E, (T, 2), generator=torch.Generator().manual_seed(0)).to(dev)
         ms = timed(lambda i: mlx_amd.gather_qmm(x, wq, sc, bi, rhs_indices=idx, transpose=True,

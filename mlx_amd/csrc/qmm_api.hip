@@ -959,22 +959,42 @@ extern "C" int mlxrocm_qmm_static(
       static_cast<hipStream_t>(stream));
 }
 
+// Small expert groups of 4-bit weights run on the slab kernel, whose K ranges
+// meet in fp32 planes behind the grouping tables.
+bool group_gather_small(int K, int n_indices, int n_experts) {
+  return K % 128 == 0 && static_cast<int64_t>(n_indices) <= 64 * static_cast<int64_t>(n_experts);
+}
+bool group_gather_slab(int N, int K, int n_indices, int n_experts, int gs, int bits) {
+  return group_gather_small(K, n_indices, n_experts) && qmm_slab_shape_ok(32, N, K, gs, bits);
+}
+
 // Grouping by expert pays when every expert's weights are shared by several
 // index pairs; it needs one row of x per pair, the matrix-core GEMM, 32-bit
 // element offsets into x and a workspace for the sorted order.
+// (Where the slab kernel groups the pairs itself there is no planning launch
+// to pay for, and a pair that shares its expert with no other still costs what
+// its own GEMV would: grouping pays from 8 pairs on -- 8 experts of
+// [14336, 4096], top-2: 8 tokens 52 us against 98 us one GEMV per pair, 12
+// tokens 53 against 155, 4 tokens 46 against 44, 2 tokens 34 against 24.)
 bool group_gather(
     int M,
+    int N,
     int K,
     int n_indices,
     int n_experts,
     int x_batches,
     int64_t x_batch_stride,
+    int group_size,
+    int bits,
     int dtype,
     bool transpose) {
   if (M != 1 || !transpose || dtype == MLXROCM_FLOAT32 || K % 64 != 0 || K < 64) {
     return false;
   }
-  if (n_indices < 32 || static_cast<int64_t>(n_indices) < 4 * static_cast<int64_t>(n_experts)) {
+  const bool few = n_indices >= 8 && qmm_slab_plans_in_kernel(n_indices, n_experts) &&
+      group_gather_slab(N, K, n_indices, n_experts, group_size, bits);
+  if (!few &&
+      (n_indices < 32 || static_cast<int64_t>(n_indices) < 4 * static_cast<int64_t>(n_experts))) {
     return false;
   }
   if (static_cast<int64_t>(x_batches) * x_batch_stride + K >= (int64_t(1) << 32)) {
@@ -984,15 +1004,6 @@ bool group_gather(
     return false;
   }
   return gather_group_workspace_bytes(n_indices, n_experts) > 0;
-}
-
-// Small expert groups of 4-bit weights run on the slab kernel, whose K ranges
-// meet in fp32 planes behind the grouping tables.
-bool group_gather_small(int K, int n_indices, int n_experts) {
-  return K % 128 == 0 && static_cast<int64_t>(n_indices) <= 64 * static_cast<int64_t>(n_experts);
-}
-bool group_gather_slab(int N, int K, int n_indices, int n_experts, int gs, int bits) {
-  return group_gather_small(K, n_indices, n_experts) && qmm_slab_shape_ok(32, N, K, gs, bits);
 }
 
 extern "C" size_t mlxrocm_gather_qmm_workspace_size(
@@ -1008,7 +1019,7 @@ extern "C" size_t mlxrocm_gather_qmm_workspace_size(
     int /*rhs_sorted*/) {
   // x_batches / stride are unknown here; mlxrocm_gather_qmm checks them and
   // falls back to the ungrouped launch if they rule grouping out.
-  if (!group_gather(M, K, n_indices, n_experts, 1, 0, dtype, transpose != 0)) {
+  if (!group_gather(M, N, K, n_indices, n_experts, 1, 0, group_size, bits, dtype, transpose != 0)) {
     return 0;
   }
   size_t bytes = gather_group_workspace_bytes(n_indices, n_experts);
@@ -1089,7 +1100,8 @@ extern "C" int mlxrocm_gather_qmm(
   }
   if (workspace != nullptr &&
       group_gather(
-          M, K, n_indices, n_experts, x_batches, x_batch_stride, dtype, transpose != 0) &&
+          M, N, K, n_indices, n_experts, x_batches, x_batch_stride, group_size, bits, dtype,
+          transpose != 0) &&
       workspace_bytes >= gather_group_workspace_bytes(n_indices, n_experts)) {
     if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) {
       return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qmm] workspace must be 4-byte aligned");
