@@ -357,6 +357,28 @@ def sweep(torch, mlx_amd, dev) -> list:
         torch.cuda.synchronize()
         ms = hip_event_ms(lib, launcher, 40 if small else 10)
         add("cfg4", f"gather T={T} top-2 of 8, unsorted, C ABI" + (" (2 experts, cache-resident)" if T == 1 else ""), ms, flops=4.0 * T * n * k)
+        if T in (8, 64):
+            # the same launch over three expert stacks in rotation (792 MB): the rows
+            # above re-read one 264 MB stack, about the size of the Infinity Cache
+            stacks = [(wq, sc, bi)] + [tuple(t.clone() for t in (wq, sc, bi)) for _ in range(2)]
+
+            def gstep3(i, stream):
+                wq_, sc_, bi_ = stacks[i % 3]
+                rc = lib.mlxrocm_gather_qmm(
+                    xb.data_ptr(), wq_.data_ptr(), sc_.data_ptr(), bi_.data_ptr(), lhs_u.data_ptr(),
+                    rhs_u.data_ptr(), out.data_ptr(), 1, n, k, n_idx, T, E, k, wq_.stride(0),
+                    sc_.stride(0), 64, 4, 2, 1, 0, ws.data_ptr() if ws_bytes else None, ws_bytes,
+                    stream)
+                if rc != 0:
+                    raise RuntimeError(_lib.last_error())
+
+            launcher = Launcher(torch, gstep3, 6, True)
+            launcher.run(6)
+            torch.cuda.synchronize()
+            ms = hip_event_ms(lib, launcher, 42)
+            add("cfg4", f"gather T={T} top-2 of 8, unsorted, C ABI, three expert stacks in rotation",
+                ms, flops=4.0 * T * n * k)
+            del stacks
     del wq, sc, bi
     # Cfg5: odd code widths, group 32, Llama-2-7B MLP shapes
     for dtype in (bf16, f32):

@@ -1137,6 +1137,25 @@ __global__ __launch_bounds__(64 * kR8Tiles * KW) void qmm_rows8_kernel(const Qmm
   }
 }
 
+// y = sum over the K ranges of plane[range] (plain call): one thread per four
+// outputs, the planes read as one stream each.
+template <typename T>
+__global__ __launch_bounds__(256) void slab_reduce_kernel(
+    const float* planes, int ranges, int64_t plane_elems, T* out) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i >= plane_elems) {
+    return;
+  }
+  floatx4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int r = 0; r < ranges; ++r) {
+    s += *reinterpret_cast<const floatx4*>(planes + r * plane_elems + i);
+  }
+  uint2 packed;
+  packed.x = pack2<T>(s[0], s[1]);
+  packed.y = pack2<T>(s[2], s[3]);
+  *reinterpret_cast<uint2*>(out + i) = packed;
+}
+
 // y[perm[pos]] (grouped) = sum over the K ranges of plane[range][pos]
 template <typename T>
 __global__ __launch_bounds__(256) void slab_reduce_grouped_kernel(
@@ -1255,8 +1274,22 @@ int launch_qmm_slab(const QmmArgs& a, int gs, int bits, int dtype, void* planes,
   if (rc != MLXROCM_OK || pl.ranges <= 1) {
     return rc;
   }
-  return reduce_planes(
-      pl.planes, a.out, static_cast<size_t>(pl.plane_elems), pl.ranges, dtype, s);
+  if (pl.ranges >= 8 && pl.plane_elems < (int64_t{1} << 20)) {
+    // many planes of a small y: the reduction that spreads the planes over threads
+    return reduce_planes(
+        pl.planes, a.out, static_cast<size_t>(pl.plane_elems), pl.ranges, dtype, s);
+  }
+  const int64_t quads = pl.plane_elems / 4; // (the caller checks plane_elems % 4 == 0)
+  const unsigned blocks = static_cast<unsigned>((quads + 255) / 256);
+  if (dtype == MLXROCM_BFLOAT16) {
+    slab_reduce_kernel<bf16_t><<<blocks, 256, 0, s>>>(
+        pl.planes, pl.ranges, pl.plane_elems, static_cast<bf16_t*>(a.out));
+  } else {
+    slab_reduce_kernel<f16_t><<<blocks, 256, 0, s>>>(
+        pl.planes, pl.ranges, pl.plane_elems, static_cast<f16_t*>(a.out));
+  }
+  MLXROCM_HIP_TRY(hipGetLastError());
+  return MLXROCM_OK;
 }
 
 // Gather grouped by expert in tiles of up to 32 rows (`a` carries the tile
