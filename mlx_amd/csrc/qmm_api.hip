@@ -407,7 +407,11 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
   // ahead, and 4096 x 4096 has too few 64-row workgroups: 9.8 against 7.1 us)
   if (transpose && a.M >= 5 && a.M <= 16 && a.lhs_indices == nullptr && a.w_alt == nullptr &&
       a.group_tiles == nullptr && qmm_rows8_supported(a, gs, bits, dtype, transpose) &&
-      2L * ((a.N + 63) / 64) * a.L >= compute_units()) {
+      2L * ((a.N + 63) / 64) * a.L >= compute_units() &&
+      // (every workgroup stages all of x: beyond 1.75 workgroups per compute unit the
+      // kernel below, which stages x once per workgroup of a persistent grid, is
+      // ahead -- 57344 x 4096, 8 rows: 42.9 against 39.8 us, 128256 x 4096: 88 against 76)
+      4L * ((a.N + 63) / 64) * a.L <= 7L * compute_units()) {
     return MLXROCM_LAUNCH(sc, launch_qmm_rows8(a, gs, bits, dtype, s));
   }
   if (transpose && a.M <= 8 && qmv_quad_supported(a, gs, bits, dtype)) {
