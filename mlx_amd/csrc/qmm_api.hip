@@ -969,7 +969,9 @@ bool group_gather_small(int K, int n_indices, int n_experts) {
   return K % 128 == 0 && static_cast<int64_t>(n_indices) <= 64 * static_cast<int64_t>(n_experts);
 }
 bool group_gather_slab(int N, int K, int n_indices, int n_experts, int gs, int bits) {
-  return group_gather_small(K, n_indices, n_experts) && qmm_slab_shape_ok(32, N, K, gs, bits);
+  // (32-wide groups only in the 16-row tiles of the kernel's own grouping)
+  const int rows = gs == 32 && qmm_slab_plans_in_kernel(n_indices, n_experts) ? 16 : 32;
+  return group_gather_small(K, n_indices, n_experts) && qmm_slab_shape_ok(rows, N, K, gs, bits);
 }
 
 // Grouping by expert pays when every expert's weights are shared by several

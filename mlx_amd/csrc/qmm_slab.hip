@@ -60,7 +60,7 @@ constexpr int kSlXStride = 2 * kSlKr + 16;           // bytes per staged row of 
 // microseconds.
 constexpr int kSlPlanPairs = kSlThreads;  // one pair per thread
 constexpr int kSlPlanExperts = 64;
-constexpr int kSlPlanTiles = kSlPlanPairs / 32 + kSlPlanExperts;
+constexpr int kSlPlanTiles = kSlPlanPairs / 16 + kSlPlanExperts; // tiles of 16 rows at worst
 constexpr int kSlPlanInts = kSlPlanPairs + kSlWaves * (kSlPlanExperts + 1) +
     3 * (kSlPlanExperts + 1) + 3 * kSlPlanTiles + 4;
 constexpr int kSlPlanBytes = (kSlPlanInts * 4 + 255) / 256 * 256;
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
         lpos[ee] = pos;
         lfirst[ee] = tile;
         pos += lcnt[ee];
-        tile += (lcnt[ee] + 31) / 32;
+        tile += (lcnt[ee] + XR - 1) / XR;
       }
       lnum[0] = tile;
       lnum[1] = pos;
@@ -288,10 +288,10 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
     if (tid < E) {
       const int c = lcnt[tid];
       int t = lfirst[tid];
-      for (int r = 0; r < c; r += 32, ++t) {
+      for (int r = 0; r < c; r += XR, ++t) { // tiles of as many rows as x is staged with
         ltiles[3 * t + 0] = tid;
         ltiles[3 * t + 1] = lpos[tid] + r;
-        ltiles[3 * t + 2] = c - r < 32 ? c - r : 32;
+        ltiles[3 * t + 2] = c - r < XR ? c - r : XR;
       }
     }
     if (e < E) {
@@ -1307,12 +1307,18 @@ int launch_qmm_slab_grouped(
     const QmmArgs& a, int gs, int bits, int dtype, void* planes, bool plan_in_kernel,
     hipStream_t s) {
   (void)bits;
-  SlabPlan pl = make_plan(
-      a.N, a.K, gather_group_max_tiles(a.L, a.n_experts, kGroupSmallTile));
+  // Few pairs per expert (8 on average at most) and the kernel's own grouping:
+  // 16-row tiles, which leave LDS for a third ring slot; an expert that does get
+  // more than 16 rows is then read once per tile.  32-wide groups have no
+  // two-tile form at all.
+  const bool one_tile = plan_in_kernel &&
+      (gs == 32 || static_cast<int64_t>(a.L) <= 8 * static_cast<int64_t>(a.n_experts));
+  const int tile_rows = one_tile ? 16 : kGroupSmallTile;
+  SlabPlan pl = make_plan(a.N, a.K, gather_group_max_tiles(a.L, a.n_experts, tile_rows));
   pl.planes = static_cast<float*>(planes);
   pl.plane_elems = static_cast<int64_t>(a.L) * a.N;
-  // (mode 1 never runs with one tile of x: instantiating it would only cost build time)
-  int rc = plan_in_kernel ? launch_any<2>(a, pl, gs, dtype, 2, s)
+  // (mode 1 never runs with one tile of x: the planning kernel makes 32-row tiles)
+  int rc = plan_in_kernel ? launch_any<2>(a, pl, gs, dtype, one_tile ? 1 : 2, s)
                           : launch_any<1>(a, pl, gs, dtype, 2, s);
   if (rc != MLXROCM_OK || pl.ranges <= 1) {
     return rc;

@@ -66,7 +66,8 @@ def test_slab_batched_weights(oracle, gpu):
 
 
 @pytest.mark.parametrize("E,T", ((8, 6), (8, 64), (16, 320)))
-@pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 64), (torch.float16, 64), (torch.bfloat16, 128)))
+@pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 64), (torch.float16, 64), (torch.bfloat16, 128),
+                                      (torch.bfloat16, 32)))
 def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T):
     """T tokens x top-2 of E experts of [520, 2048] (two K ranges, a ragged
     slab).  6 tokens: grouping already pays from 8 pairs on; 64 tokens over 8
@@ -89,7 +90,8 @@ def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T):
         assert int(counts.max()) > 32
     gx, gwq, gsc, gb, gidx = (t.to(gpu) for t in (x, wq, s, b, idx))
     ws = _lib.load().mlxrocm_gather_qmm_workspace_size(1, N, K, 2 * T, E, gs, 4, CODE[dtype], 1, 0)
-    assert ws >= (K // 1024) * 2 * T * N * 4, "the call did not take the slab kernel"
+    if gs != 32 or 2 * T <= 512:  # (32-wide groups: only where the kernel groups the pairs itself)
+        assert ws >= (K // 1024) * 2 * T * N * 4, "the call did not take the slab kernel"
     got = mlx_amd.gather_qmm(gx, gwq, gsc, gb, rhs_indices=gidx, transpose=True,
                              group_size=gs, bits=4)
     assert got.shape == (T, 2, 1, N)
@@ -101,8 +103,11 @@ def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T):
     exact = torch.einsum("tk,tjnk->tjn", x.reshape(T, K).double(), w_hat[idx]).reshape(T, 2, 1, N)
     assert float((got.cpu().double() - exact).abs().max()) <= exact_tolerance(
         dtype, K, x, w_hat, exact)
-    assert float((got.cpu().double() - ref.double()).abs().max()) <= matmul_tolerance(
-        dtype, K, x, w_hat)
+    # (the CPU reference accumulates 16-bit types in the element type,
+    # cpu/quantized.cpp:177-206: its own distance from the exact product is
+    # discounted; the fp64 check above is the strict one)
+    tol_ref = matmul_tolerance(dtype, K, x, w_hat) + float((ref.double() - exact).abs().max())
+    assert float((got.cpu().double() - ref.double()).abs().max()) <= tol_ref
     # sorted by expert: same rows, bit for bit
     flat = gidx.reshape(-1)
     order = torch.argsort(flat, stable=True)
