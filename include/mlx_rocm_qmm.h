@@ -162,8 +162,8 @@ int mlxrocm_gguf_repack(
  * transpose == 0 call on the matrix cores (a transposed copy of scales and
  * biases, 4 * N * K / group_size bytes); transpose == 0 calls with 1..4 rows of
  * x and K > 64 (one fp32 plane of the output per 64 rows of K); 5..32 rows of
- * x over 4-bit weights with transpose != 0 and K a multiple of 1024 beyond
- * 1024 (one fp32 plane of the output per 1024 codes of K).  Calls with one to
+ * x over 4-bit weights with transpose != 0 and K a multiple of 256 beyond
+ * 1024 (one fp32 plane of the output per started 1024 codes of K).  Calls with one to
  * four rows of x and transpose != 0 never use one.  The call only enqueues work: it allocates
  * nothing, takes no lock and does not synchronize, so it can be captured in a
  * HIP graph.  A workspace that is too small is MLXROCM_INVALID_ARGUMENT.
@@ -331,7 +331,7 @@ int mlxrocm_qmm_swiglu(
  * mlxrocm_gather_qmm_workspace_size(...) bytes and may be NULL when that is 0:
  * with many index pairs per expert (M == 1, 16-bit types) the pairs are sorted
  * by expert into it and every expert's weights are read once for all its rows
- * (small expert groups of 4-bit weights also keep K / 1024 fp32 planes of
+ * (small expert groups of 4-bit weights also keep ceil(K / 1024) fp32 planes of
  * [n_indices, N] there; the pointer must then be 16-byte aligned);
  * without a workspace the call falls back to one product per pair.  Index
  * values are range-checked on the device; an out-of-range pair produces zeros

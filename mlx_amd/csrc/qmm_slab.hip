@@ -29,7 +29,8 @@
 //     row per load), results leave one step after their unit ended (stores
 //     count in vmcnt like loads);
 //   * the K ranges of a row of y are added up from fp32 planes by a second
-//     small kernel (one range: written directly);
+//     small kernel (one range: written directly); K is a multiple of 256, the
+//     last range of a row may be 512 or 768 codes long (not 256);
 //   * a gather of up to 512 index pairs is grouped by expert inside the kernel.
 // LDS reads are free of bank conflicts by construction: the 16-byte pieces of a
 // weight row are stored at piece ^ (row / 2 % 8), rows of x are 16 bytes longer
@@ -66,7 +67,7 @@ constexpr int kSlPlanInts = kSlPlanPairs + kSlWaves * (kSlPlanExperts + 1) +
 constexpr int kSlPlanBytes = (kSlPlanInts * 4 + 255) / 256 * 256;
 
 struct SlabPlan {
-  int ranges;          // K / 1024
+  int ranges;          // ceil(K / 1024); the last one may hold 2 or 3 steps instead of 4
   int n_slabs;         // ceil(N / 256)
   int workgroups;      // the launch's grid
   float* planes;       // ranges > 1: fp32 [ranges][rows][N]
@@ -335,7 +336,12 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
     return;
   }
   const int my_units = static_cast<int>(u1 - u0);
-  const int my_steps = my_units * kSlSteps;
+  // steps of a unit: four, fewer in the last K range when K is no multiple of 1024
+  const int last_steps = K / kSlStep - (R - 1) * kSlSteps;
+  auto unit_steps = [&](int range) { return range == R - 1 ? last_steps : kSlSteps; };
+  // the last range reads the last GPR groups of a row (whole 16-byte pieces that
+  // end where the row ends): its groups start this far into that window
+  const int last_shift = R * GPR - groups;
 
   auto resolve = [&](SlabUnit<T>& u) {
     int64_t e = u.owner;
@@ -401,8 +407,9 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   };
   InFlight4 sbq[kSbInstrs]; // in flight within one loop iteration only
   auto fetch_sb = [&](const SlabUnit<T>& u) {
-    const T* sp = u.scales + u.range * GPR;
-    const T* bp = u.biases + u.range * GPR;
+    const int g0 = u.range * GPR - (u.range == R - 1 ? last_shift : 0);
+    const T* sp = u.scales + g0;
+    const T* bp = u.biases + g0;
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       sbq[i].load(sp, sb_off[i]);
@@ -453,6 +460,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
     constexpr int cshift = kSlKrShift - 3; // 16-byte pieces per row = 1 << cshift
     constexpr int kPasses = (XR << cshift) / kSlThreads;
     const T* xbase = static_cast<const T*>(a.x) + (u.range << kSlKrShift);
+    const int valid_k = unit_steps(u.range) * kSlStep; // codes of this range
     // all loads first: one memory latency for the whole tile
     uint4 xv[kPasses];
 #pragma unroll
@@ -461,7 +469,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
       const int m = c >> cshift;
       const int col = c & ((1 << cshift) - 1);
       xv[i] = make_uint4(0u, 0u, 0u, 0u);
-      if (m < M) {
+      if (m < M && col * 8 < valid_k) {
         xv[i] = *reinterpret_cast<const uint4*>(xbase + xoff[m] + col * 8);
       }
     }
@@ -507,6 +515,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   uint32_t wmagic = WidenMagic<T>::kBits;
   asm volatile("" : "+v"(wmask), "+v"(wmagic)); // keep both in vector registers
 
+  int sb_shift = 0; // first group of the compute unit inside its scale window
   floatx4 acc[2][MT];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
@@ -591,7 +600,7 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
     T cs[kCorr][2], cb[kCorr][2];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
-      const uint8_t* sp = sbbuf + (nt * 16 + r16) * RB + j * (2 * GPS);
+      const uint8_t* sp = sbbuf + (nt * 16 + r16) * RB + (j * GPS + sb_shift) * 2;
       if constexpr (GPS == 8) {
         const uint4 v = *reinterpret_cast<const uint4*>(sp);
         raw[nt][0] = v.x; raw[nt][1] = v.y; raw[nt][2] = v.z; raw[nt][3] = v.w;
@@ -740,25 +749,30 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   first_unit(fu);
   cu = fu;
   fetch_offsets(fu);
-  int fj = 0;        // step of fu to fetch next
-  int fetched = 0;   // steps fetched so far
+  int fj = 0;          // step of fu to fetch next
+  int funit = 0;       // which of this workgroup's units fu is
+  bool fdone = false;  // every step has been fetched
   int fslot = 0;
   // Fetches the next step; true when it is the first step of a unit, whose
   // scales and biases were then requested ahead of its weights.  Past the end:
   // the last step again (lands in a free slot, never read), so that the
   // outstanding-load count of every wait is the same.
   auto fetch_next = [&]() {
-    const bool enters = fj == 0 && fetched != 0 && fetched < my_steps;
+    const bool enters = fj == 0 && funit != 0 && !fdone;
     if (enters) {
       fetch_sb(fu);
     }
     fetch_w(fu, fj, fslot);
     fslot = fslot + 1 == kStages ? 0 : fslot + 1;
-    if (++fetched < my_steps) {
-      if (++fj == kSlSteps) {
+    if (!fdone && ++fj == unit_steps(fu.range)) {
+      if (funit + 1 < my_units) {
         fj = 0;
+        ++funit;
         next_unit(fu);
         fetch_offsets(fu);
+      } else {
+        fdone = true;
+        --fj;
       }
     }
     return enters;
@@ -781,7 +795,9 @@ __global__ __launch_bounds__(kSlThreads, 2) void qmm_slab_kernel(const QmmArgs a
   bool have_sb = false;
   int cslot = 0;
   for (int un = 0; un < my_units; ++un) {
-    for (int j = 0; j < kSlSteps; ++j) {
+    const int usteps = unit_steps(cu.range);
+    sb_shift = cu.range == R - 1 ? last_shift : 0;
+    for (int j = 0; j < usteps; ++j) {
       const bool entered = fetch_next();
       const bool two = MT == 2 && M > 16;
       if (entered) {
@@ -1225,7 +1241,7 @@ int launch_any(const QmmArgs& a, const SlabPlan& pl, int gs, int dtype, int mt, 
 SlabPlan make_plan(int N, int K, long owners) {
   SlabPlan pl{};
   pl.n_slabs = (N + kSlRows - 1) / kSlRows;
-  pl.ranges = K >> kSlKrShift;
+  pl.ranges = (K + kSlKr - 1) >> kSlKrShift;
   const long units = owners * pl.ranges * pl.n_slabs;
   const long cus = compute_units();
   pl.workgroups = static_cast<int>(units < cus ? (units > 0 ? units : 1) : cus);
@@ -1239,7 +1255,9 @@ bool qmm_slab_shape_ok(int rows, int N, int K, int gs, int bits) {
   if (bits != 4 || rows < 1 || rows > 32 || (gs == 32 && rows > 16)) {
     return false;
   }
-  if (K < kSlKr || K % kSlKr != 0 || N < 4 || N % 4 != 0) {
+  // whole 256-code steps; a last K range of 2..4 of them (one step would be
+  // shorter than the fetch distance of the ring)
+  if (K < kSlKr || K % kSlStep != 0 || (K / kSlStep) % kSlSteps == 1 || N < 4 || N % 4 != 0) {
     return false;
   }
   // 32-bit byte offsets of a matrix's rows
@@ -1254,13 +1272,13 @@ bool qmm_slab_supported(const QmmArgs& a, int gs, int bits, int dtype, bool tran
 }
 
 long qmm_slab_units(const QmmArgs& a) {
-  return static_cast<long>(a.L) * (a.K >> kSlKrShift) * ((a.N + kSlRows - 1) / kSlRows);
+  return static_cast<long>(a.L) * ((a.K + kSlKr - 1) >> kSlKrShift) * ((a.N + kSlRows - 1) / kSlRows);
 }
 
 // Plain call (no index arrays).  With more than one K range `planes` must hold
 // qmm_slab_plane_bytes() bytes.
 size_t qmm_slab_plane_bytes(const QmmArgs& a) {
-  const int ranges = a.K >> kSlKrShift;
+  const int ranges = (a.K + kSlKr - 1) >> kSlKrShift;
   return ranges <= 1 ? 0 : static_cast<size_t>(ranges) * a.L * a.M * a.N * sizeof(float);
 }
 
@@ -1295,7 +1313,7 @@ int launch_qmm_slab(const QmmArgs& a, int gs, int bits, int dtype, void* planes,
 // Gather grouped by expert in tiles of up to 32 rows (`a` carries the tile
 // list).  planes: qmm_slab_grouped_plane_bytes() bytes.
 size_t qmm_slab_grouped_plane_bytes(int n_indices, int N, int K) {
-  const int ranges = K >> kSlKrShift;
+  const int ranges = (K + kSlKr - 1) >> kSlKrShift;
   return ranges <= 1 ? 0 : static_cast<size_t>(ranges) * n_indices * N * sizeof(float);
 }
 

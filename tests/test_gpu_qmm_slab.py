@@ -17,7 +17,7 @@ CODE = {torch.float16: 1, torch.bfloat16: 2}
 
 
 def _planes_bytes(M, N, K, L=1):
-    return (K // 1024) * L * M * N * 4 if K > 1024 else 0
+    return -(-K // 1024) * L * M * N * 4 if K > 1024 else 0
 
 
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
@@ -49,6 +49,29 @@ def test_slab_ragged_and_single_range(oracle, gpu, N, K):
         assert ws == _planes_bytes(M, N, K)
 
 
+@pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32)))
+@pytest.mark.parametrize("N,K", ((16384, 1536), (8200, 3584), (4096, 11008)))
+def test_slab_short_last_range(oracle, gpu, dtype, gs, N, K):
+    """K a multiple of 256 but not of 1024: the last K range has two or three
+    steps instead of four (1536 = 4 + 2, 3584 = 4 + 4 + 4 + 2, 11008 = 10 x 4 + 3);
+    its scales are fetched from a window that ends with the row, x beyond K
+    stays zero in LDS."""
+    w = normal_weights((N, K), dtype, std=0.05)
+    quantized = oracle.quantize(w, gs, 4)
+    for M in (9, 16):
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, None, gs, 4, rows=torch.tensor([M - 1]), quantized=quantized)
+        ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, 4, CODE[dtype], 1)
+        assert ws == _planes_bytes(M, N, K), "the shape did not take the slab kernel"
+
+
+def test_slab_one_step_last_range_is_refused(gpu):
+    """A last range of a single step (K = 1280, 5376 ...) is not built: such
+    shapes stay on the other kernels and ask for no planes."""
+    for K in (1280, 5376):
+        assert _lib.load().mlxrocm_qmm_workspace_size(16, 16384, K, 1, 0, 64, 4, 2, 1) == 0
+
+
 def test_slab_batched_weights(oracle, gpu):
     """Eight problems of [4096, 1024] with their own weights: the unit list runs
     over problems, every workgroup restages x when it crosses into the next one."""
@@ -65,18 +88,19 @@ def test_slab_batched_weights(oracle, gpu):
     assert float((got.double() - ref.double()).abs().max()) <= matmul_tolerance(dtype, K, x, w_hat)
 
 
+@pytest.mark.parametrize("K", (2048, 1792))
 @pytest.mark.parametrize("E,T", ((8, 6), (8, 64), (16, 320)))
 @pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 64), (torch.float16, 64), (torch.bfloat16, 128),
                                       (torch.bfloat16, 32)))
-def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T):
-    """T tokens x top-2 of E experts of [520, 2048] (two K ranges, a ragged
-    slab).  6 tokens: grouping already pays from 8 pairs on; 64 tokens over 8
+def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T, K):
+    """T tokens x top-2 of E experts of [520, K] (two K ranges, the second one
+    short at K = 1792; a ragged slab).  6 tokens: grouping already pays from 8 pairs on; 64 tokens over 8
     experts: the kernel groups the pairs itself, experts end up with fewer and
     with more than 16 rows; 320 tokens over 16 experts: the planning kernel runs
     first, experts have more than one tile.  One pair names
     an expert that does not exist (zero row), and the run on expert-sorted pairs
     reproduces the unsorted one bit for bit."""
-    N, K = 520, 2048
+    N = 520
     w = normal_weights((E, N, K), dtype, std=0.5)
     wq, s, b = oracle.quantize(w, gs, 4)
     x = activations((T, 1, 1, K), dtype)
@@ -91,7 +115,7 @@ def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T):
     gx, gwq, gsc, gb, gidx = (t.to(gpu) for t in (x, wq, s, b, idx))
     ws = _lib.load().mlxrocm_gather_qmm_workspace_size(1, N, K, 2 * T, E, gs, 4, CODE[dtype], 1, 0)
     if gs != 32 or 2 * T <= 512:  # (32-wide groups: only where the kernel groups the pairs itself)
-        assert ws >= (K // 1024) * 2 * T * N * 4, "the call did not take the slab kernel"
+        assert ws >= -(-K // 1024) * 2 * T * N * 4, "the call did not take the slab kernel"
     got = mlx_amd.gather_qmm(gx, gwq, gsc, gb, rhs_indices=gidx, transpose=True,
                              group_size=gs, bits=4)
     assert got.shape == (T, 2, 1, N)
