@@ -379,6 +379,17 @@ def sweep(torch, mlx_amd, dev) -> list:
             add("cfg4", f"gather T={T} top-2 of 8, unsorted, C ABI, three expert stacks in rotation",
                 ms, flops=4.0 * T * n * k)
             del stacks
+    # transpose=False over the same stack (the input gradient of the expert layer,
+    # GatherQMM::vjp): cotangent rows [1, 14336] x W as [14336, 4096]
+    for T in (64, 2048):
+        cot = torch.randn((T, 2, 1, n), generator=g, dtype=torch.float32).to(bf16).to(dev)
+        idx = torch.randint(0, E, (T, 2), generator=torch.Generator().manual_seed(0)).to(dev)
+        lhs = torch.arange(2 * T, device=dev).reshape(T, 2)
+        ms = timed(lambda i: mlx_amd.gather_qmm(cot, wq, sc, bi, lhs_indices=lhs,
+                                                rhs_indices=idx, transpose=False,
+                                                group_size=64, bits=4))
+        add("f3", f"gather transpose=False T={T} top-2 of 8 (x [1,{n}] per pair, W [{n},{k}])", ms,
+            flops=4.0 * T * n * k)
     del wq, sc, bi
     # Cfg5: odd code widths, group 32, Llama-2-7B MLP shapes
     for dtype in (bf16, f32):

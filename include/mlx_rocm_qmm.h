@@ -332,7 +332,10 @@ int mlxrocm_qmm_swiglu(
  * with many index pairs per expert (M == 1, 16-bit types) the pairs are sorted
  * by expert into it and every expert's weights are read once for all its rows
  * (small expert groups of 4-bit weights also keep ceil(K / 1024) fp32 planes of
- * [n_indices, N] there; the pointer must then be 16-byte aligned);
+ * [n_indices, N] there; the pointer must then be 16-byte aligned; with
+ * transpose == 0, 4- or 8-bit codes and at least four pairs the [group][k]
+ * images of every expert's scales and biases follow the tables, 16-byte
+ * aligned as well);
  * without a workspace the call falls back to one product per pair.  Index
  * values are range-checked on the device; an out-of-range pair produces zeros
  * instead of a wild access.

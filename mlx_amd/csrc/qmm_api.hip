@@ -1012,6 +1012,45 @@ bool group_gather(
   return gather_group_workspace_bytes(n_indices, n_experts) > 0;
 }
 
+// transpose=false (what the backward pass of an expert layer asks for): the
+// pairs are sorted by expert in 256-row tiles for the tile GEMM's column
+// loader, which reads scales and biases from [group][k] images -- those of all
+// experts are made behind the grouping tables first.
+constexpr size_t kGroupTablesAlign = 256;
+size_t group_gather_n_tables(int n_indices, int n_experts) {
+  return (gather_group_workspace_bytes(n_indices, n_experts) + kGroupTablesAlign - 1) /
+      kGroupTablesAlign * kGroupTablesAlign;
+}
+bool group_gather_n(
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int n_experts,
+    int x_batches,
+    int64_t x_batch_stride,
+    int bits,
+    int dtype,
+    bool transpose) {
+  if (M != 1 || transpose || dtype == MLXROCM_FLOAT32 || K % 64 != 0 || K < 64 || N < 8 ||
+      (bits != 4 && bits != 8)) {
+    return false;
+  }
+  // (one product per pair has no fast kernel with [K, N] weights: 8 experts of
+  // [14336, 4096], 32 pairs: 5.5 ms against 0.37 ms grouped, which is what a
+  // single 256-row tile per expert costs -- grouping pays from a few pairs on)
+  if (n_indices < 4) {
+    return false;
+  }
+  if (static_cast<int64_t>(x_batches) * x_batch_stride + K >= (int64_t(1) << 32)) {
+    return false;
+  }
+  if (gather_group_max_tiles(n_indices, n_experts, kGroupLargeTile) > 65535) {
+    return false;
+  }
+  return gather_group_workspace_bytes(n_indices, n_experts) > 0;
+}
+
 extern "C" size_t mlxrocm_gather_qmm_workspace_size(
     int M,
     int N,
@@ -1025,6 +1064,10 @@ extern "C" size_t mlxrocm_gather_qmm_workspace_size(
     int /*rhs_sorted*/) {
   // x_batches / stride are unknown here; mlxrocm_gather_qmm checks them and
   // falls back to the ungrouped launch if they rule grouping out.
+  if (group_gather_n(M, N, K, n_indices, n_experts, 1, 0, bits, dtype, transpose != 0)) {
+    return group_gather_n_tables(n_indices, n_experts) +
+        qmm_n_sb_bytes(K, N / group_size, n_experts, dtype);
+  }
   if (!group_gather(M, N, K, n_indices, n_experts, 1, 0, group_size, bits, dtype, transpose != 0)) {
     return 0;
   }
@@ -1135,6 +1178,29 @@ extern "C" int mlxrocm_gather_qmm(
     }
     return small ? launch_qmm_skinny_grouped(a, group_size, bits, dtype, s)
                  : launch_qmm_mfma_grouped(a, group_size, bits, dtype, s);
+  }
+  if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0 &&
+      group_gather_n(
+          M, N, K, n_indices, n_experts, x_batches, x_batch_stride, bits, dtype, transpose != 0)) {
+    const int G = N / group_size;
+    const int images = sb_expert_stride == 0 ? 1 : n_experts;
+    const size_t tables = group_gather_n_tables(n_indices, n_experts);
+    if (workspace_bytes >= tables + qmm_n_sb_bytes(K, G, images, dtype)) {
+      rc = launch_gather_group(a, dtype, kGroupLargeTile, workspace, s);
+      if (rc != MLXROCM_OK) {
+        return rc;
+      }
+      char* image = static_cast<char*>(workspace) + tables;
+      rc = transpose_sb_for_qmm_n(scales, biases, image, K, G, images, sb_expert_stride, dtype, s);
+      if (rc != MLXROCM_OK) {
+        return rc;
+      }
+      const size_t one = static_cast<size_t>(K) * G; // elements of one [G][K] image
+      a.scales = image;
+      a.biases = image + one * dtype_size(dtype);
+      a.sb_batch_stride = images == 1 ? 0 : static_cast<int64_t>(2 * one);
+      return launch_qmm_mfma_grouped_n(a, group_size, bits, dtype, s);
+    }
   }
   // One grid z-slot per index pair; large index lists go in slices.
   constexpr int kMaxZ = 65535;

@@ -193,6 +193,8 @@ long qmv_quad_workgroups_two_sets(const QmmArgs& a, int bits);
 int launch_qmm_mfma_ksplit(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
 int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int dtype, hipStream_t s);
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+// transpose=false form: scales / biases are the [group][k] images of all experts
+int launch_qmm_mfma_grouped_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 
 // Compute units of the current device (read once).
 inline int compute_units() {

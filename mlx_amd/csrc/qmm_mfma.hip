@@ -217,7 +217,7 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const int k_splits) {
   constexpr bool kSplit = !std::is_same<T, TS>::value;
   static_assert(!(kSplit && GROUPED), "the grouped gather runs on 16-bit types only");
-  static_assert(!(WN && (kSplit || GROUPED)), "[K, N] weights: plain 16-bit problems only");
+  static_assert(!(WN && kSplit), "[K, N] weights: 16-bit problems only");
   static_assert(!WN || BITS == 4 || BITS == 8, "[K, N] weights: 4- and 8-bit codes");
   constexpr int kBN = 32 * NT;
   constexpr int kNS = 8 * NT; // MFMAs per wavefront per K-step
@@ -1172,6 +1172,24 @@ int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipSt
       constexpr int B = decltype(bval)::value;
       return launch_variant<T, T, T, B, kNT, true>(a, gs_shift, grid, s);
     });
+  };
+  return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
+}
+
+// The same for [K, N] weights (transpose=false): a.scales / a.biases point at
+// the transposed images of all experts (transpose_sb_for_qmm_n), a.sb_batch_stride
+// is the distance between two experts' images.
+int launch_qmm_mfma_grouped_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  constexpr int kNT = 6;
+  const int gs_shift = shift_of(gs);
+  const dim3 grid(
+      (a.N + 32 * kNT - 1) / (32 * kNT), gather_group_max_tiles(a.L, a.n_experts, kGroupLargeTile), 1);
+  auto run = [&](auto tval) -> int {
+    using T = decltype(tval);
+    if (bits == 4) {
+      return launch_variant<T, T, T, 4, kNT, true, true>(a, gs_shift, grid, s);
+    }
+    return launch_variant<T, T, T, 8, kNT, true, true>(a, gs_shift, grid, s);
   };
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
 }

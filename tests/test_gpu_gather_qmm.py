@@ -167,6 +167,60 @@ def test_gather_qmm_grouped_by_expert(oracle, gpu, dtype, bits, gs):
     assert float((got[sub].double() - ref.double()).abs().max()) <= tol
 
 
+@pytest.mark.parametrize("bits,gs", ((4, 64), (8, 32), (4, 128)))
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_gather_qmm_grouped_by_expert_not_transposed(oracle, gpu, dtype, bits, gs):
+    """transpose=False (weights [K, N], what GatherQMM::vjp asks for,
+    mlx/primitives.cpp:3718-3837) with many pairs per expert: sorted by expert
+    into 256-row tiles of the column-loading tile GEMM.  Skewed routing (one
+    expert with more than one tile, one unused), x rows reused, N no multiple
+    of the tile width, one expert index out of range (zero row); a shared
+    scale/bias set (stride 0) is not part of the Python surface and not taken."""
+    from mlx_amd import _lib
+    E, N, K, T = 5, 384, 320, 700
+    code = {torch.float16: 1, torch.bfloat16: 2}[dtype]
+    ws = _lib.load().mlxrocm_gather_qmm_workspace_size(1, N, K, T, E, gs, bits, code, 0, 0)
+    assert ws >= 2 * E * K * (N // gs) * 2, "the grouped path is not taken"
+    w = normal_weights((E, K, N), dtype, std=0.5)
+    wq, s, b = oracle.quantize(w, gs, bits)
+    X = 64
+    x = activations((X, 1, K), dtype)
+    g = torch.Generator().manual_seed(1)
+    rhs = torch.multinomial(torch.tensor([0.6, 0.0, 0.25, 0.1, 0.05]), T,
+                            replacement=True, generator=g)
+    lhs = torch.randint(0, X, (T,), generator=g)
+    assert int((rhs == 0).sum()) > 256 and int((rhs == 1).sum()) == 0
+    gx, gwq, gsc, gb, glhs, grhs = _to(gpu, x, wq, s, b, lhs, rhs)
+    got = mlx_amd.gather_qmm(gx, gwq, gsc, gb, glhs, grhs, False, gs, bits).cpu()
+    assert got.shape == (T, 1, N)
+    w_hat = exact_affine_weights(wq, s, b, gs, bits)  # [E, K, N]
+    exact = torch.einsum("tk,tkn->tn", x.reshape(X, K).double()[lhs], w_hat[rhs])
+    err = float((got.reshape(T, N).double() - exact).abs().max())
+    assert err <= exact_tolerance(dtype, K, x, w_hat, exact)
+    # against the oracle on a subsample of the pairs (the oracle is scalar and
+    # accumulates in the element type: its own distance from exact is discounted)
+    sub = torch.arange(0, T, 23)
+    ref = oracle.gather_qmm(x, wq, s, b, lhs[sub], rhs[sub], False, gs, bits)
+    tol = matmul_tolerance(dtype, K, x, w_hat) + float(
+        (ref.reshape(-1, N).double() - exact[sub]).abs().max())
+    assert float((got[sub].double() - ref.double()).abs().max()) <= tol
+    # two pairs at a time stay on one product per pair: same rows up to rounding
+    parts = [
+        mlx_amd.gather_qmm(gx, gwq, gsc, gb, glhs[i:i + 2], grhs[i:i + 2], False, gs, bits)
+        for i in range(0, 64, 2)
+    ]
+    single = torch.cat(parts).cpu()
+    eps = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    assert float((got[:64].double() - single.double()).abs().max()) <= 2 * eps * float(exact.abs().max())
+    bad = grhs.clone()
+    bad[7] = E + 2
+    got_bad = mlx_amd.gather_qmm(gx, gwq, gsc, gb, glhs, bad, False, gs, bits).cpu()
+    assert bool((got_bad[7] == 0).all())
+    keep = torch.ones(T, dtype=torch.bool)
+    keep[7] = False
+    assert torch.equal(got_bad[keep], got[keep])
+
+
 @pytest.mark.parametrize("index_dtype", (torch.int64, torch.int32, torch.uint32, torch.int16))
 def test_gather_qmm_many_pairs_and_index_types(gpu, index_dtype):
     """More than 16384 pairs take the three-kernel grouping (fewer take the
