@@ -42,11 +42,12 @@ def test_slab_ragged_and_single_range(oracle, gpu, N, K):
     and a long K (14 ranges)."""
     dtype = torch.bfloat16
     w = normal_weights((N, K), dtype, std=0.05)
-    for M in (9, 24):
+    for M in (6, 9, 24):
         x = activations((M, K), dtype, seed=M)
         _check_qmm(oracle, gpu, x, w, 64, 4, rows=torch.tensor([M - 1]))
         ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, 64, 4, 2, 1)
-        assert ws == _planes_bytes(M, N, K)
+        if M >= 9 or K >= 8192:  # (5..8 rows: only over a long K)
+            assert ws == _planes_bytes(M, N, K)
 
 
 @pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32)))
