@@ -424,10 +424,12 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
       // a single round, or more than 7/8 of the slots of all rounds in use
       many_rows = a.K >= 8192 || gs == 32 ||
           (wgs > 0 && (rounds <= 1 || wgs * 8 > rounds * cus * 7));
-      // (a long K that the slab kernel below takes: 4096 x 14336, 8 rows: 13.5 us
-      // there against 16.1 here, 8192 x 8192: 13.9 against 17.3, 5120 x 13824: 20.5
-      // against 29.6)
-      if (a.K >= 8192 && a.lhs_indices == nullptr && a.group_tiles == nullptr &&
+      // (not where the slab kernel below takes the shape, a single K range
+      // excepted: 4096 x 14336, 8 rows: 13.5 us there against 16.1 here,
+      // 8192 x 8192: 13.9 against 17.3, 5120 x 13824: 20.5 against 29.6,
+      // 128256 x 4096: 63 against 104, 151936 x 3584: 73 against 143, 32000 x 4096:
+      // 19.9 against 28.1; but 32768 x 1024 with 32-wide groups: 10.4 against 8.9)
+      if (a.K >= 2048 && a.lhs_indices == nullptr && a.group_tiles == nullptr &&
           a.w_alt == nullptr && qmm_slab_supported(a, gs, bits, dtype, transpose) &&
           2 * qmm_slab_units(a) >= cus &&
           (qmm_slab_plane_bytes(a) == 0 || (static_cast<int64_t>(a.L) * a.M * a.N) % 4 == 0)) {

@@ -35,18 +35,19 @@ def test_slab_rows_and_groups(oracle, gpu, dtype, gs, M):
         assert ws == _planes_bytes(M, N, K), "the shape did not take the slab kernel"
 
 
-@pytest.mark.parametrize("N,K", ((8000, 4096), (32772, 1024), (4096, 14336)))
+@pytest.mark.parametrize("N,K", ((8000, 4096), (32772, 1024), (4096, 14336), (32000, 2048)))
 def test_slab_ragged_and_single_range(oracle, gpu, N, K):
     """N that is no multiple of the 256-row slab (the last slab's rows are
-    clamped and never written), a single K range (written directly, no planes)
-    and a long K (14 ranges)."""
+    clamped and never written), a single K range (written directly, no planes),
+    a long K (14 ranges) and a tall matrix (more workgroups than the kernel
+    with all of K in LDS is used for, so 5..8 rows come here as well)."""
     dtype = torch.bfloat16
     w = normal_weights((N, K), dtype, std=0.05)
     for M in (6, 9, 24):
         x = activations((M, K), dtype, seed=M)
         _check_qmm(oracle, gpu, x, w, 64, 4, rows=torch.tensor([M - 1]))
         ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, 64, 4, 2, 1)
-        if M >= 9 or K >= 8192:  # (5..8 rows: only over a long K)
+        if M >= 9 or K >= 8192 or N >= 32000:  # (5..8 rows: a long K or many rows of W)
             assert ws == _planes_bytes(M, N, K)
 
 
