@@ -161,9 +161,10 @@ int mlxrocm_gguf_repack(
  * is split; fp32 partial results); 16-bit prefill calls with M >= 512 and every
  * transpose == 0 call on the matrix cores (a transposed copy of scales and
  * biases, 4 * N * K / group_size bytes); transpose == 0 calls with 1..4 rows of
- * x and K > 64 (one fp32 plane of the output per 64 rows of K); 5..32 rows of
+ * x and K > 64 (one fp32 plane of the output per 64 rows of K); 5..64 rows of
  * x over 4-bit weights with transpose != 0 and K a multiple of 256 beyond
- * 1024 (one fp32 plane of the output per started 1024 codes of K).  Calls with one to
+ * 1024 (one fp32 plane of the output per started 1024 codes of K; 33..64
+ * rows take the same path 32 rows at a time and need what 32 rows need).  Calls with one to
  * four rows of x and transpose != 0 never use one.  The call only enqueues work: it allocates
  * nothing, takes no lock and does not synchronize, so it can be captured in a
  * HIP graph.  A workspace that is too small is MLXROCM_INVALID_ARGUMENT.

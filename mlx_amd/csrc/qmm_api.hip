@@ -464,6 +464,42 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
       return MLXROCM_LAUNCH(sc, launch_qmm_slab(a, gs, bits, dtype, region, s));
     }
   }
+  // 33..64 rows: the same kernel twice, 32 rows and the rest; the second
+  // pass finds weights in the Infinity Cache where they fit.  The 256-row tile
+  // GEMM below costs the same whatever M (graph replays, 64 rows: 14336 x 4096:
+  // 37 us, twice the slab kernel: 31; 4096 x 14336: 46.5 against 35; 28672 x 4096:
+  // 60 against 50; 128256 x 4096: 270 against 180); from 65 rows on it is ahead.
+  if (transpose && a.M > 32 && a.M <= 64 && a.L == 1 && gs != 32 && a.lhs_indices == nullptr &&
+      a.group_tiles == nullptr && a.w_alt == nullptr) {
+    const int first = 32;
+    QmmArgs head = a;
+    head.M = first;
+    QmmArgs tail = a;
+    tail.M = a.M - first;
+    tail.x = static_cast<const char*>(a.x) + static_cast<size_t>(first) * a.K * dtype_size(dtype);
+    tail.out = static_cast<char*>(a.out) + static_cast<size_t>(first) * a.N * dtype_size(dtype);
+    if (qmm_slab_supported(head, gs, bits, dtype, transpose) &&
+        qmm_slab_supported(tail, gs, bits, dtype, transpose) &&
+        2 * qmm_slab_units(head) >= compute_units()) {
+      // both passes use the same planes, one after the other on the stream
+      const size_t plane_bytes = qmm_slab_plane_bytes(head);
+      void* region = nullptr;
+      if (plane_bytes != 0) {
+        const int rc = claim(sc, plane_bytes, &region);
+        if (rc != MLXROCM_OK) {
+          return rc;
+        }
+      }
+      if (sc.dry) {
+        return MLXROCM_OK;
+      }
+      const int rc = launch_qmm_slab(head, gs, bits, dtype, region, s);
+      if (rc != MLXROCM_OK) {
+        return rc;
+      }
+      return launch_qmm_slab(tail, gs, bits, dtype, region, s);
+    }
+  }
   // (two rows of 8-bit codes over a long K: the streaming kernel's dot products
   // are issue-bound there, 28 us against 20 us for the wide kernel at K = 14336)
   const bool few_rows = a.M >= 3 || !qmv_stream_supported(a, gs, bits, dtype) ||

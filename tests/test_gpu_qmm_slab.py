@@ -67,6 +67,24 @@ def test_slab_short_last_range(oracle, gpu, dtype, gs, N, K):
         assert ws == _planes_bytes(M, N, K), "the shape did not take the slab kernel"
 
 
+@pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 64), (torch.float16, 128)))
+def test_slab_two_passes_for_33_to_64_rows(oracle, gpu, dtype, gs):
+    """33..64 rows run the kernel twice (32 rows, then the rest) over the same
+    planes; 65 rows and 32-wide groups stay on the tile GEMM."""
+    N, K = 8200, 3584
+    w = normal_weights((N, K), dtype, std=0.05)
+    quantized = oracle.quantize(w, gs, 4)
+    lib = _lib.load()
+    for M in (33, 47, 64):
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, None, gs, 4, rows=torch.tensor([0, 31, 32, M - 1]),
+                   quantized=quantized)
+        ws = lib.mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, 4, CODE[dtype], 1)
+        assert ws == _planes_bytes(32, N, K), "the shape did not take the slab kernel twice"
+    assert lib.mlxrocm_qmm_workspace_size(65, N, K, 1, 0, gs, 4, CODE[dtype], 1) != _planes_bytes(32, N, K)
+    assert lib.mlxrocm_qmm_workspace_size(40, N, K, 1, 0, 32, 4, CODE[dtype], 1) != _planes_bytes(32, N, K)
+
+
 def test_slab_one_step_last_range_is_refused(gpu):
     """A last range of a single step (K = 1280, 5376 ...) is not built: such
     shapes stay on the other kernels and ask for no planes."""
