@@ -376,6 +376,24 @@ int run_qmm_n(const QmmArgs& a, int gs, int bits, int dtype, Scratch& sc, hipStr
   return reduce_k_splits(partial, a.out, plane, k_splits, dtype, s);
 }
 
+// Where the slab kernel is worth its launch: its units (K ranges x 256-row
+// slabs) fill at least half the compute units -- or, with fewer, the weights
+// are large enough that the kernels it replaces take longer than its floor of
+// 12 us (9..16 rows) or 15 us (17..32 rows, where they run twice).  Graph
+// replays, 24 rows: 6144 x 4096: 15.3 against 21.0 us, 5120 x 5120: 15.5
+// against 24.5, 2048 x 8192: 14.3 against 20.4; but 4096 x 4096: 14.7 against
+// 13.0, 8192 x 2048: 14.2 against 11.6; 12 rows: 5120 x 5120: 12.5 against 14.0.
+bool slab_pays(const QmmArgs& a) {
+  if (2 * qmm_slab_units(a) >= compute_units()) {
+    return true;
+  }
+  const int64_t codes = static_cast<int64_t>(a.L) * a.N * a.K;
+  if (a.M > 16) {
+    return codes >= 25000000 || (a.K >= 8192 && codes >= 16000000);
+  }
+  return a.M > 8 && codes >= 26000000;
+}
+
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& sc, hipStream_t s) {
   // w [K, N] with a few rows of x: the streaming kernel (the tile kernel
   // needs 60-70 us for one row of a 4096 x 14336 weight)
@@ -451,7 +469,7 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
   if (transpose && a.M >= 5 && a.M <= 32 && a.lhs_indices == nullptr &&
       a.group_tiles == nullptr && a.w_alt == nullptr &&
       qmm_slab_supported(a, gs, bits, dtype, transpose) &&
-      2 * qmm_slab_units(a) >= compute_units()) {
+      slab_pays(a)) {
     const size_t plane_bytes = qmm_slab_plane_bytes(a);
     if (plane_bytes == 0 || (static_cast<int64_t>(a.L) * a.M * a.N) % 4 == 0) {
       void* region = nullptr;
@@ -532,7 +550,13 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
   const bool narrow_long = a.M > 16 && a.K > 8192 &&
       static_cast<long>((a.N + 63) / 64) * a.L < compute_units() / 2 &&
       a.lhs_indices == nullptr && a.group_tiles == nullptr;
-  const bool staged = (a.M > 16 || (a.M > 8 && a.N >= 8192)) && !narrow_long;
+  // (8-bit codes, 3..8 rows over 64 MB of weights or more: the staged kernel is
+  // ahead of the MFMA GEMV as it is from 9 rows on -- graph replays, 8 rows:
+  // 28672 x 4096: 26 against 37 us, 8192 x 8192: 32 against 45, 49152 x 4096: 38
+  // against 55; level at 14336 x 4096 and 128256 x 4096)
+  const bool many_bytes = bits == 8 && a.M >= 3 && a.N >= 8192 &&
+      static_cast<int64_t>(a.N) * a.K >= (int64_t{64} << 20);
+  const bool staged = (a.M > 16 || (a.M > 8 && a.N >= 8192) || many_bytes) && !narrow_long;
   // one row at a width the row-streaming GEMV does not cover (2/3/5/6 bits): the
   // fp32-arithmetic streaming kernel
   if (transpose && a.M == 1 && few_rows && qmv_f32_supported(a, gs, bits, dtype)) {

@@ -213,6 +213,19 @@ def test_qmm_few_rows_kernels(oracle, gpu, dtype, bits):
             _check_qmm(oracle, gpu, x, w, gs, bits)
 
 
+@pytest.mark.parametrize("dtype,gs", ((torch.bfloat16, 128), (torch.float16, 64)))
+def test_qmm_few_rows_of_8_bit_over_many_bytes(oracle, gpu, dtype, gs):
+    """3..8 rows over 64 MB of 8-bit codes or more take the LDS-staged 32-row
+    kernel (as 9..32 rows do): ragged N, every row checked against fp64, the
+    first and the last against the CPU reference."""
+    N, K = 8200, 8192
+    w = normal_weights((N, K), dtype, std=0.05)
+    quantized = oracle.quantize(w, gs, 8)
+    for M in (3, 8):
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, None, gs, 8, rows=torch.tensor([0, M - 1]), quantized=quantized)
+
+
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
 @pytest.mark.parametrize("bits,gs", ((4, 32), (4, 64), (8, 64), (8, 128)))
 def test_qmm_n_on_the_matrix_path(oracle, gpu, dtype, bits, gs):

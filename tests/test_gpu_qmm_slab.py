@@ -85,6 +85,22 @@ def test_slab_two_passes_for_33_to_64_rows(oracle, gpu, dtype, gs):
     assert lib.mlxrocm_qmm_workspace_size(40, N, K, 1, 0, 32, 4, CODE[dtype], 1) != _planes_bytes(32, N, K)
 
 
+def test_slab_below_half_occupancy_for_large_weights(oracle, gpu):
+    """Fewer units than half the compute units, but weights large enough that
+    the kernels it replaces would be slower than its floor: 17..32 rows at
+    6144 x 4096 (96 units) and 2048 x 8192 (64 units, long K) take it; 4096 x
+    4096 (64 units) and 12 rows at 6144 x 4096 do not."""
+    lib = _lib.load()
+    dtype = torch.bfloat16
+    for (N, K) in ((6144, 4096), (2048, 8192)):
+        w = normal_weights((N, K), dtype, std=0.05)
+        x = activations((24, K), dtype)
+        _check_qmm(oracle, gpu, x, w, 64, 4, rows=torch.tensor([0, 23]))
+        assert lib.mlxrocm_qmm_workspace_size(24, N, K, 1, 0, 64, 4, 2, 1) == _planes_bytes(24, N, K)
+    assert lib.mlxrocm_qmm_workspace_size(24, 4096, 4096, 1, 0, 64, 4, 2, 1) == 0
+    assert lib.mlxrocm_qmm_workspace_size(12, 6144, 4096, 1, 0, 64, 4, 2, 1) == 0
+
+
 def test_slab_one_step_last_range_is_refused(gpu):
     """A last range of a single step (K = 1280, 5376 ...) is not built: such
     shapes stay on the other kernels and ask for no planes."""
