@@ -429,7 +429,11 @@ int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& 
       // (every workgroup stages all of x: beyond 1.75 workgroups per compute unit the
       // kernel below, which stages x once per workgroup of a persistent grid, is
       // ahead -- 57344 x 4096, 8 rows: 42.9 against 39.8 us, 128256 x 4096: 88 against 76)
-      4L * ((a.N + 63) / 64) * a.L <= 7L * compute_units()) {
+      4L * ((a.N + 63) / 64) * a.L <= 7L * compute_units() &&
+      // (32-wide groups: twice the scales in LDS; a second round of workgroups
+      // costs more than the kernel below -- 18432..28672 x 4096, 5..7 rows: 25-28
+      // against 21 us)
+      (gs != 32 || static_cast<long>((a.N + 63) / 64) * a.L <= compute_units())) {
     return MLXROCM_LAUNCH(sc, launch_qmm_rows8(a, gs, bits, dtype, s));
   }
   if (transpose && a.M <= 8 && qmv_quad_supported(a, gs, bits, dtype)) {
