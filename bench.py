@@ -315,6 +315,9 @@ def sweep(torch, mlx_amd, dev) -> list:
     for M in (1, 512, 2048):
         matmul_case("f3", M, 14336, 4096, 4, 64, bf16, transpose=False)
         matmul_case("f3", M, 4096, 14336, 8, 128, bf16, transpose=False)
+    # ... at an odd width (codes repacked at 4 bits first)
+    for M in (1, 512):
+        matmul_case("f3", M, 11008, 4096, 3, 32, bf16, transpose=False)
     # Cfg4: 8 experts, top-2 routing
     E, n, k = 8, 14336, 4096
     wq, sc, bi = mlx_amd.quantize(

@@ -161,7 +161,9 @@ int mlxrocm_gguf_repack(
  * is split; fp32 partial results); 16-bit prefill calls with M >= 512 and every
  * transpose == 0 call on the matrix cores (a transposed copy of scales and
  * biases, 4 * N * K / group_size bytes); transpose == 0 calls with 1..4 rows of
- * x and K > 64 (one fp32 plane of the output per 64 rows of K); 5..64 rows of
+ * x and K > 64 (one fp32 plane of the output per 64 rows of K); transpose == 0
+ * calls at 2, 3, 5 or 6 bits (the codes repacked at 4 or 8 bits: K * N / 2 or
+ * K * N bytes per weight matrix, plus what the call needs at that width); 5..64 rows of
  * x over 4-bit weights with transpose != 0 and K a multiple of 256 beyond
  * 1024 (one fp32 plane of the output per started 1024 codes of K; 33..64
  * rows take the same path 32 rows at a time and need what 32 rows need).  Calls with one to

@@ -394,7 +394,58 @@ bool slab_pays(const QmmArgs& a) {
   return a.M > 8 && codes >= 26000000;
 }
 
+int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& sc, hipStream_t s);
+
+// transpose=false at 2, 3, 5 or 6 bits: the [K, N] kernels read whole words
+// per 8 codes, which these widths do not offer, so the codes are first repacked
+// at 4 or 8 bits into the workspace (same values, same scales and biases) and
+// the call goes on at that width -- 4096 x 4096 at 3 bits, one row: 1.4 ms on
+// the scalar kernel, two launches of a few microseconds this way.
+int run_widened(const QmmArgs& a, int gs, int bits, int dtype, Scratch& sc, hipStream_t s) {
+  const int wide = widened_bits(bits);
+  const int batches = a.w_batch_stride == 0 ? 1 : a.L;
+  const size_t codes = static_cast<size_t>(a.K) * a.N;
+  const size_t words_out = codes / 32 * wide;
+  const size_t repack_bytes =
+      (batches * words_out * sizeof(uint32_t) + kScratchAlign - 1) / kScratchAlign * kScratchAlign;
+  QmmArgs inner = a;
+  Scratch probe;
+  probe.dry = true;
+  int rc = run(inner, gs, wide, dtype, false, probe, s);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  void* region = nullptr;
+  rc = claim(sc, repack_bytes + probe.need, &region);
+  if (rc != MLXROCM_OK || sc.dry) {
+    return rc;
+  }
+  uint32_t* packed = static_cast<uint32_t*>(region);
+  const int64_t words_in = static_cast<int64_t>(codes / 32) * bits;
+  if (batches == 1 || a.w_batch_stride == words_in) {
+    rc = launch_widen_codes(a.w, packed, codes * batches, bits, s);
+  } else {
+    for (int l = 0; l < batches && rc == MLXROCM_OK; ++l) {
+      rc = launch_widen_codes(a.w + l * a.w_batch_stride, packed + l * words_out, codes, bits, s);
+    }
+  }
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  inner.w = packed;
+  inner.w_batch_stride = batches == 1 ? 0 : static_cast<int64_t>(words_out);
+  Scratch rest;
+  rest.base = static_cast<char*>(region) + repack_bytes;
+  rest.bytes = sc.bytes - repack_bytes;
+  return run(inner, gs, wide, dtype, false, rest, s);
+}
+
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& sc, hipStream_t s) {
+  if (!transpose && widened_bits(bits) != 0 && a.lhs_indices == nullptr &&
+      a.group_tiles == nullptr && a.N % 32 == 0 &&
+      (a.M <= 4 || (dtype != MLXROCM_FLOAT32 && a.K % 64 == 0 && a.K >= 64))) {
+    return run_widened(a, gs, bits, dtype, sc, s);
+  }
   // w [K, N] with a few rows of x: the streaming kernel (the tile kernel
   // needs 60-70 us for one row of a 4096 x 14336 weight)
   if (!transpose && qmv_n_supported(a, gs, bits, dtype)) {

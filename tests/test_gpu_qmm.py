@@ -256,6 +256,47 @@ def test_qvm_streaming_kernel(oracle, gpu, dtype, bits, gs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits,gs", ((2, 32), (3, 64), (5, 32), (6, 128)))
+def test_transpose_false_odd_widths_are_repacked(oracle, gpu, dtype, bits, gs):
+    """transpose=False at 2/3/5/6 bits: the codes are repacked at 4 or 8 bits
+    into the workspace first (same values, same scales) and the call goes on on
+    the kernels of that width -- one row and four (streaming kernel, every
+    element type), a ragged M and a long K on the matrix cores (16-bit types;
+    float32 with more than four rows stays on the scalar kernel)."""
+    from mlx_amd import _lib
+
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    lib = _lib.load()
+    for M, K, N in ((1, 512, 384), (4, 1000, 1152), (70, 2048, 640), (9, 64, 4096)):
+        w = normal_weights((K, N), dtype, seed=bits + gs + M)
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, w, gs, bits, transpose=False)
+        ws = lib.mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, bits, code, 0)
+        repacked = K * N * (4 if bits < 4 else 8) // 8
+        if M <= 4 or (dtype != torch.float32 and K % 64 == 0):
+            assert ws >= repacked, "the call did not repack the codes"
+        else:
+            assert ws == 0
+
+
+def test_transpose_false_odd_width_batched_weights(oracle, gpu):
+    """Three problems with their own 3-bit [K, N] weights: every matrix is
+    repacked, the batch stride of the repacked stack is the new one; the same
+    with a strided (every other) selection of a larger stack."""
+    dtype = torch.bfloat16
+    L, M, K, N = 3, 20, 256, 320
+    w = normal_weights((2 * L, K, N), dtype, seed=1)
+    wq, s, b = oracle.quantize(w, 64, 3)
+    x = activations((L, M, K), dtype, seed=2)
+    for sel in (slice(0, L), slice(0, 2 * L, 2)):
+        got = mlx_amd.quantized_matmul(
+            x.to(gpu), wq.to(gpu)[sel], s.to(gpu)[sel], b.to(gpu)[sel], False, 64, 3).cpu()
+        w_hat = exact_affine_weights(wq[sel], s[sel], b[sel], 64, 3)  # [L, K, N]
+        exact = torch.einsum("lmk,lkn->lmn", x.double(), w_hat)
+        assert float((got.double() - exact).abs().max()) <= exact_tolerance(dtype, K, x, w_hat, exact)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_transpose_false_odd_k(oracle, gpu, dtype):
     # K need not be a multiple of anything when w is [K, N]: rows of x then start
     # at unaligned addresses (7 rows: the generic kernel; 3 rows: the streaming one)
