@@ -160,7 +160,7 @@ int mlxrocm_gguf_repack(
  * matrix cores); 16-bit calls whose tile grid would leave compute units idle (K
  * is split; fp32 partial results); 16-bit prefill calls with M >= 512 and every
  * transpose == 0 call on the matrix cores (a transposed copy of scales and
- * biases, 4 * N * K / group_size bytes); transpose == 0 calls with 1..4 rows of
+ * biases, 4 * N * K / group_size bytes); transpose == 0 calls with 1..8 rows of
  * x and K > 64 (one fp32 plane of the output per 64 rows of K); transpose == 0
  * calls at 2, 3, 5 or 6 bits (the codes repacked at 4 or 8 bits: K * N / 2 or
  * K * N bytes per weight matrix, plus what the call needs at that width); 5..64 rows of

@@ -443,13 +443,33 @@ int run_widened(const QmmArgs& a, int gs, int bits, int dtype, Scratch& sc, hipS
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& sc, hipStream_t s) {
   if (!transpose && widened_bits(bits) != 0 && a.lhs_indices == nullptr &&
       a.group_tiles == nullptr && a.N % 32 == 0 &&
-      (a.M <= 4 || (dtype != MLXROCM_FLOAT32 && a.K % 64 == 0 && a.K >= 64))) {
+      (a.M <= 4 || (a.M <= 8 && a.L == 1) ||
+       (dtype != MLXROCM_FLOAT32 && a.K % 64 == 0 && a.K >= 64))) {
     return run_widened(a, gs, bits, dtype, sc, s);
   }
   // w [K, N] with a few rows of x: the streaming kernel (the tile kernel
   // needs 60-70 us for one row of a 4096 x 14336 weight)
   if (!transpose && qmv_n_supported(a, gs, bits, dtype)) {
     return run_qmv_n(a, gs, bits, dtype, sc, s);
+  }
+  // ... and 5..8 rows: the same kernel twice, four rows and the rest, over the
+  // same planes (graph replays, W [14336, 4096] 4-bit: 41-52 us against 65 for the
+  // tile kernel, which costs the same whatever M; W [4096, 4096]: 20-25 against 25)
+  if (!transpose && a.M >= 5 && a.M <= 8 && a.L == 1) {
+    QmmArgs head = a;
+    head.M = 4;
+    QmmArgs tail = a;
+    tail.M = a.M - 4;
+    tail.x = static_cast<const char*>(a.x) + static_cast<size_t>(4) * a.K * dtype_size(dtype);
+    tail.out = static_cast<char*>(a.out) + static_cast<size_t>(4) * a.N * dtype_size(dtype);
+    if (qmv_n_supported(head, gs, bits, dtype) && qmv_n_supported(tail, gs, bits, dtype)) {
+      // (the first pass needs the larger workspace: it is the one a dry run sizes)
+      const int rc = run_qmv_n(head, gs, bits, dtype, sc, s);
+      if (rc != MLXROCM_OK || sc.dry) {
+        return rc;
+      }
+      return run_qmv_n(tail, gs, bits, dtype, sc, s);
+    }
   }
   // A few rows of x, beyond what the row-streaming GEMV keeps in registers.
   // Measured on gate/up and down projection shapes (4- and 8-bit):

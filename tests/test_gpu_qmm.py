@@ -256,13 +256,32 @@ def test_qvm_streaming_kernel(oracle, gpu, dtype, bits, gs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits,gs", ((4, 64), (8, 128), (3, 32)))
+def test_qvm_streaming_kernel_twice_for_5_to_8_rows(oracle, gpu, dtype, bits, gs):
+    """transpose=False with 5..8 rows of x: the row-streaming kernel runs twice
+    (four rows, then the rest) over the same planes of the workspace."""
+    from mlx_amd import _lib
+
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    K, N = 1088, 1152
+    w = normal_weights((K, N), dtype, seed=bits + gs)
+    quantized = oracle.quantize(w, gs, bits)
+    for M in (5, 7, 8):
+        x = activations((M, K), dtype, seed=M)
+        _check_qmm(oracle, gpu, x, None, gs, bits, transpose=False, quantized=quantized)
+        ws4 = _lib.load().mlxrocm_qmm_workspace_size(4, N, K, 1, 0, gs, bits, code, 0)
+        ws = _lib.load().mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, bits, code, 0)
+        assert ws == ws4 and ws > 0, "the call is not sized like its four-row pass"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("bits,gs", ((2, 32), (3, 64), (5, 32), (6, 128)))
 def test_transpose_false_odd_widths_are_repacked(oracle, gpu, dtype, bits, gs):
     """transpose=False at 2/3/5/6 bits: the codes are repacked at 4 or 8 bits
     into the workspace first (same values, same scales) and the call goes on on
     the kernels of that width -- one row and four (streaming kernel, every
     element type), a ragged M and a long K on the matrix cores (16-bit types;
-    float32 with more than four rows stays on the scalar kernel)."""
+    float32 with more than eight rows stays on the scalar kernel)."""
     from mlx_amd import _lib
 
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
@@ -273,7 +292,7 @@ def test_transpose_false_odd_widths_are_repacked(oracle, gpu, dtype, bits, gs):
         _check_qmm(oracle, gpu, x, w, gs, bits, transpose=False)
         ws = lib.mlxrocm_qmm_workspace_size(M, N, K, 1, 0, gs, bits, code, 0)
         repacked = K * N * (4 if bits < 4 else 8) // 8
-        if M <= 4 or (dtype != torch.float32 and K % 64 == 0):
+        if M <= 8 or (dtype != torch.float32 and K % 64 == 0):
             assert ws >= repacked, "the call did not repack the codes"
         else:
             assert ws == 0
