@@ -156,7 +156,7 @@ int mlxrocm_gguf_repack(
  * bytes, 256-byte aligned, owned by the caller (an eval_gpu body allocates it
  * like any other temporary and keeps it until the stream has passed the call);
  * it may be NULL when that size is 0.  Shapes that use it: float32 operands
- * with M > 8 and transpose != 0 (x split into two bfloat16 parts for the
+ * with M > 16 (M > 8 in a batch of problems) and transpose != 0 (x split into two bfloat16 parts for the
  * matrix cores); 16-bit calls whose tile grid would leave compute units idle (K
  * is split; fp32 partial results); 16-bit prefill calls with M >= 512 and every
  * transpose == 0 call on the matrix cores (a transposed copy of scales and

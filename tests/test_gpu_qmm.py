@@ -433,13 +433,18 @@ def test_qmv_float32_streaming(oracle, gpu, bits):
 def test_qmv_float32_few_rows(oracle, gpu, bits):
     """2..4 rows of float32 x in one launch of the fp32 streaming GEMV (K up to
     8192), and the shapes beyond it (5..16 rows, K > 8192 with two rows, a batch
-    of problems with five rows) on the generic kernels and the matrix path."""
+    of problems with five rows) on the generic kernels; 9..16 rows run them
+    twice (eight rows, then the rest) and need no workspace, 17 rows take the
+    matrix path."""
     cases = ((64, 2, 100, 512), (32, 3, 70, 4096), (128, 4, 33, 8192), (64, 7, 64, 2048),
              (64, 16, 48, 4096), (32, 13, 40, 6144), (64, 2, 24, 10240))
     for gs, M, N, K in cases:
         w = normal_weights((N, K), torch.float32, seed=bits + gs + M)
         x = activations((M, K), torch.float32, seed=K + M)
         _check_qmm(oracle, gpu, x, w, gs, bits)
+    from mlx_amd import _lib
+    assert _lib.load().mlxrocm_qmm_workspace_size(13, 4096, 4096, 1, 0, 64, bits, 0, 1) == 0
+    assert _lib.load().mlxrocm_qmm_workspace_size(17, 4096, 4096, 1, 0, 64, bits, 0, 1) > 0
     # batched, five rows
     L, M, N, K, gs = 2, 5, 40, 1024, 64
     ws = [normal_weights((N, K), torch.float32, seed=30 + l) for l in range(L)]
