@@ -14,7 +14,17 @@ enum class Family { Qmv, QmmT, QmmN, QmmNaive };
 // weight row is read once and reused across the few rows of x.
 constexpr int kQmvMaxM = 8;
 
-Family choose_family(int M, int /*N*/, int K, int /*L*/, int bits, int dtype, bool transpose) {
+// transpose=false at 2/3/5/6 bits: whether the codes are repacked at 4 or 8 bits
+// first (run_widened) so that the fast [K, N] kernels apply.
+bool widens_codes(int M, int N, int K, int L, int bits, int dtype, bool transpose) {
+  return !transpose && widened_bits(bits) != 0 && N % 32 == 0 &&
+      (M <= 4 || (M <= 8 && L == 1) || (dtype != MLXROCM_FLOAT32 && K % 64 == 0 && K >= 64));
+}
+
+Family choose_family(int M, int N, int K, int L, int bits, int dtype, bool transpose) {
+  if (widens_codes(M, N, K, L, bits, dtype, transpose)) {
+    bits = widened_bits(bits);
+  }
   if (transpose && M <= kQmvMaxM) {
     return Family::Qmv;
   }
@@ -441,10 +451,8 @@ int run_widened(const QmmArgs& a, int gs, int bits, int dtype, Scratch& sc, hipS
 }
 
 int run(const QmmArgs& a, int gs, int bits, int dtype, bool transpose, Scratch& sc, hipStream_t s) {
-  if (!transpose && widened_bits(bits) != 0 && a.lhs_indices == nullptr &&
-      a.group_tiles == nullptr && a.N % 32 == 0 &&
-      (a.M <= 4 || (a.M <= 8 && a.L == 1) ||
-       (dtype != MLXROCM_FLOAT32 && a.K % 64 == 0 && a.K >= 64))) {
+  if (a.lhs_indices == nullptr && a.group_tiles == nullptr &&
+      widens_codes(a.M, a.N, a.K, a.L, bits, dtype, transpose)) {
     return run_widened(a, gs, bits, dtype, sc, s);
   }
   // w [K, N] with a few rows of x: the streaming kernel (the tile kernel

@@ -70,7 +70,8 @@ def test_kernel_choice(lib):
     assert name(2048, 14336, 4096, 1, 64, 4, 0, 1) == b"qmm_t"        # float32: split bf16
     assert name(2048, 14336, 4000, 1, 32, 4, 0, 1) == b"qmm_generic"  # K not a multiple of 64
     assert name(64, 512, 256, 1, 64, 4, 2, 0) == b"qmm_n"             # transpose=False, 4/8-bit
-    assert name(64, 512, 256, 1, 64, 3, 2, 0) == b"qmm_generic"       # transpose=False, odd width
+    assert name(64, 512, 256, 1, 64, 3, 2, 0) == b"qmm_n"             # ... odd width: repacked at 4 bits
+    assert name(64, 512, 256, 1, 64, 3, 0, 0) == b"qmm_generic"       # ... odd width, float32, many rows
     assert name(64, 512, 256, 1, 64, 4, 0, 0) == b"qmm_generic"       # transpose=False, float32
     assert name(64, 512, 250, 1, 64, 4, 2, 1) is None
 
