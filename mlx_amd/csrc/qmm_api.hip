@@ -1170,8 +1170,10 @@ bool group_gather(
   }
   const bool few = n_indices >= 8 && qmm_slab_plans_in_kernel(n_indices, n_experts) &&
       group_gather_slab(N, K, n_indices, n_experts, group_size, bits);
+  // (from one pair per expert on average: 64 experts of [2048, 1408], top-6, 32
+  // tokens: 99 us one GEMV per pair, 47 us grouped; 8-bit, 16 tokens: 88 against 50)
   if (!few &&
-      (n_indices < 32 || static_cast<int64_t>(n_indices) < 4 * static_cast<int64_t>(n_experts))) {
+      (n_indices < 32 || static_cast<int64_t>(n_indices) < static_cast<int64_t>(n_experts))) {
     return false;
   }
   if (static_cast<int64_t>(x_batches) * x_batch_stride + K >= (int64_t(1) << 32)) {
