@@ -356,10 +356,11 @@ def mixtral_stack(gpu):
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("T", (1, 64))
+@pytest.mark.parametrize("T", (1, 8, 64))
 def test_gather_qmm_full_size_moe_few_tokens(oracle, gpu, mixtral_stack, T):
     """The expert-routed decode shapes at full size: T tokens, top-2 of 8 experts
-    drawn uniformly (seeded), unsorted and pre-sorted by expert.  Every index
+    drawn uniformly (seeded), unsorted and pre-sorted by expert (8 tokens: 16
+    pairs, grouped inside the kernel in 16-row tiles; 64: in 32-row tiles).  Every index
     pair against the fp64 product; a subsample of the pairs against the CPU
     oracle; sorted and unsorted runs agree bit for bit after un-permuting."""
     wq, s, b, w_hat = mixtral_stack

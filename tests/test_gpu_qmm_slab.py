@@ -130,7 +130,8 @@ def test_slab_batched_weights(oracle, gpu):
                                       (torch.bfloat16, 32)))
 def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T, K):
     """T tokens x top-2 of E experts of [520, K] (two K ranges, the second one
-    short at K = 1792; a ragged slab).  6 tokens: grouping already pays from 8 pairs on; 64 tokens over 8
+    short at K = 1792; a ragged slab).  6 tokens: grouping pays from 8 pairs on over large experts, these small
+    ones are multiplied pair by pair; 64 tokens over 8
     experts: the kernel groups the pairs itself, experts end up with fewer and
     with more than 16 rows; 320 tokens over 16 experts: the planning kernel runs
     first, experts have more than one tile.  One pair names
@@ -150,7 +151,13 @@ def test_slab_grouped_gather(oracle, gpu, dtype, gs, E, T, K):
         assert int(counts.max()) > 32
     gx, gwq, gsc, gb, gidx = (t.to(gpu) for t in (x, wq, s, b, idx))
     ws = _lib.load().mlxrocm_gather_qmm_workspace_size(1, N, K, 2 * T, E, gs, 4, CODE[dtype], 1, 0)
-    if gs != 32 or 2 * T <= 512:  # (32-wide groups: only where the kernel groups the pairs itself)
+    if T == 6:
+        # 12 pairs: grouped only over experts of 4 MB and more (one GEMV over a
+        # smaller one takes about a microsecond); these stay on one GEMV per pair
+        assert ws == 0
+        big = _lib.load().mlxrocm_gather_qmm_workspace_size(1, 4096, 4096, 12, E, gs, 4, CODE[dtype], 1, 0)
+        assert big >= 4 * 12 * 4096 * 4, "12 pairs over large experts are not grouped"
+    elif gs != 32 or 2 * T <= 512:  # (32-wide groups: only where the kernel groups the pairs itself)
         assert ws >= -(-K // 1024) * 2 * T * N * 4, "the call did not take the slab kernel"
     got = mlx_amd.gather_qmm(gx, gwq, gsc, gb, rhs_indices=gidx, transpose=True,
                              group_size=gs, bits=4)
