@@ -115,11 +115,36 @@ def hip_event_ms(lib, launcher: "Launcher", steps: int) -> float:
 
 
 # Timing protocol of the headline figures: after at least MIN_WARMUP untimed
-# launches, REPEATS timed regions of max(--steps, MIN_LAUNCHES) launches each,
-# HIP events around every region; the median region is the figure.
+# launches, REPEATS timed regions, HIP events around every region; the median
+# region is the figure.  A qmv region is max(--steps, QMV_MIN_LAUNCHES) launches
+# rounded up to whole passes over the weight ring: a graph replay costs a few
+# microseconds of host time, and with only a handful of replays per region (plus
+# a shorter tail graph) that cost showed up as 6-8 % on an 8 us kernel.  A
+# qmm_t region (200 us per call, launched one by one) is at least MIN_LAUNCHES.
 REPEATS = 7
+QMV_MIN_LAUNCHES = 1800
 MIN_LAUNCHES = 100
 MIN_WARMUP = 10
+
+
+def read_only_floor() -> dict | None:
+    """Runs the read-only probe (mlx_amd/lib/read_probe --floor) in a child
+    process and returns its figures: what a launch that only loads the decode
+    weight's 33 MB costs in the same launch chain, what it costs from the
+    cache, and what an empty grid costs.  Called before this process touches
+    the GPU.  None when the probe is not built or fails."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "mlx_amd", "lib", "read_probe")
+    if not os.path.isfile(exe):
+        return None
+    try:
+        proc = subprocess.run([exe, "--floor"], capture_output=True, text=True, timeout=120)
+        if proc.returncode != 0:
+            return None
+        return json.loads(proc.stdout.strip().splitlines()[-1])
+    except (OSError, ValueError, IndexError, subprocess.TimeoutExpired):
+        return None
 
 
 def median_event_ms(lib, launcher: "Launcher", launches: int, repeats: int = REPEATS):
@@ -457,6 +482,8 @@ def main() -> int:
     ap.add_argument("--only", choices=("qmv", "qmm_t"), default=None)
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying a HIP graph")
+    ap.add_argument("--no-floor", action="store_true",
+                    help="skip the read-only probe (roofline.read_only_floor_us)")
     ap.add_argument("--sweep", action="store_true",
                     help="time the other synthetic configurations of the path instead of "
                          "the headline pair; prints one JSON line {\"sweep\": [...]}")
@@ -468,6 +495,12 @@ def main() -> int:
         print("bench.py measures one GPU; this build has no multi-GPU path "
               "(run with --gpus 1)", file=sys.stderr)
         return 2
+
+    # the load-only floor of a 33 MB launch, measured by a child process before
+    # this one initialises the GPU
+    floor = None
+    if not (args.copy_probe or args.sweep or args.no_floor) and args.only in (None, "qmv"):
+        floor = read_only_floor()
 
     import torch
 
@@ -540,7 +573,7 @@ def main() -> int:
     if args.only in (None, "qmv"):
         launcher = Launcher(torch, qmv_step, RING, not args.no_graph)
         warmup = max(args.warmup, MIN_WARMUP)
-        launches = max(args.steps, MIN_LAUNCHES)
+        launches = -(-max(args.steps, QMV_MIN_LAUNCHES) // RING) * RING
         launcher.prepare(warmup)
         launcher.prepare(launches)
         launcher.run(warmup)
@@ -592,6 +625,17 @@ def main() -> int:
                 "llc_resident_gbps": round(nbytes / (llc_ms * 1e-3) / 1e9, 2),
             },
         })
+        if floor is not None:
+            # the same bytes through a kernel that only loads, same launch chain
+            result["roofline"].update({
+                "read_only_floor_us": floor["read_only_floor_us"],
+                "read_only_floor_frac": round(
+                    floor["bytes"] / (floor["read_only_floor_us"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                "read_only_cache_resident_us": floor["read_only_cache_resident_us"],
+                "empty_launch_us": floor["empty_launch_us"],
+                "floor_source": "mlx_amd/lib/read_probe --floor (child process, before this "
+                                "process initialised the GPU)",
+            })
 
     # ---------------------------------------------------------------- qmm_t
     if args.only in (None, "qmm_t"):

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MLXROCM_ABI_VERSION 2
+#define MLXROCM_ABI_VERSION 3
 
 typedef enum {
   MLXROCM_OK = 0,
@@ -392,6 +392,57 @@ const char* mlxrocm_qmm_kernel_name(
     int bits,
     int dtype,
     int transpose);
+
+/*
+ * What mlxrocm_qmm would do for a shape, without touching a device: the call
+ * is rehearsed -- same argument checks, same kernel choice, the same workspace
+ * claims against `workspace_bytes` -- and every launch is recorded instead of
+ * issued.  `plan` receives the record as text, "[rule]+kernel(params)+kernel..."
+ * ("[rule]" = the entry of the dispatch table that took the shape; a call that
+ * re-enters the table, e.g. after repacking odd code widths, shows every
+ * entry), truncated to plan_bytes - 1 characters.  Returns what the call would
+ * return: MLXROCM_INVALID_ARGUMENT when workspace_bytes is too small.  No
+ * counterpart in the reference (its CUDA backend picks kernels in
+ * mlx/backend/cuda/quantized/quantized.cpp:95-136 and qmm/qmm.cu:64-100 without
+ * an introspection hook); it exists so that the kernel choice and the
+ * workspace sizes can be tested on a machine without a GPU.
+ */
+int mlxrocm_qmm_plan(
+    int M,
+    int N,
+    int K,
+    int L,
+    int batched_weights,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    size_t workspace_bytes,
+    char* plan,
+    size_t plan_bytes);
+
+/* The same for mlxrocm_gather_qmm. */
+int mlxrocm_gather_qmm_plan(
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int group_size,
+    int bits,
+    int dtype,
+    int transpose,
+    size_t workspace_bytes,
+    char* plan,
+    size_t plan_bytes);
+
+/* The dispatch table of mlxrocm_qmm, first match wins: number of entries, and
+ * entry i's name and the measurements its thresholds rest on (static strings;
+ * NULL beyond the table). */
+int mlxrocm_qmm_rule_count(void);
+const char* mlxrocm_qmm_rule_name(int i);
+const char* mlxrocm_qmm_rule_evidence(int i);
 
 /* ------------------------------------------------------------------------ */
 /* Element copies with dtype conversion                                      */

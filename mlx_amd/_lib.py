@@ -53,6 +53,11 @@ SIGNATURES = {
     ),
     "mlxrocm_gather_qmm_workspace_size": (_sz, [_i] * 10),
     "mlxrocm_qmm_kernel_name": (ctypes.c_char_p, [_i] * 8),
+    "mlxrocm_qmm_plan": (_i, [_i] * 9 + [_sz, ctypes.c_char_p, _sz]),
+    "mlxrocm_gather_qmm_plan": (_i, [_i] * 10 + [_sz, ctypes.c_char_p, _sz]),
+    "mlxrocm_qmm_rule_count": (_i, []),
+    "mlxrocm_qmm_rule_name": (ctypes.c_char_p, [_i]),
+    "mlxrocm_qmm_rule_evidence": (ctypes.c_char_p, [_i]),
     "mlxrocm_malloc": (_i, [ctypes.POINTER(_p), _sz]),
     "mlxrocm_free": (_i, [_p]),
     "mlxrocm_buffer_size": (_sz, [_p]),
@@ -110,10 +115,45 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
-    if lib.mlxrocm_abi_version() != 2:
+    if lib.mlxrocm_abi_version() != 3:
         raise ImportError("libmlx_rocm_qmm.so ABI version mismatch")
     _lib = lib
     return lib
+
+
+def qmm_plan(M, N, K, L=1, batched_weights=False, group_size=64, bits=4, dtype=BFLOAT16,
+             transpose=True, workspace_bytes=None):
+    """(status, record) of a rehearsed mlxrocm_qmm call: the dispatch rules it
+    takes and the kernels it would launch, e.g.
+    "[qmm_t_tile_sb_transposed]+transpose_sb+qmm_t_tile(nt=7)".  Runs without a
+    GPU.  workspace_bytes=None rehearses with exactly mlxrocm_qmm_workspace_size."""
+    lib = load()
+    args = (M, N, K, L, int(batched_weights), group_size, bits, dtype, int(transpose))
+    if workspace_bytes is None:
+        workspace_bytes = lib.mlxrocm_qmm_workspace_size(*args)
+    buf = ctypes.create_string_buffer(1024)
+    rc = lib.mlxrocm_qmm_plan(*args, workspace_bytes, buf, len(buf))
+    return rc, buf.value.decode()
+
+
+def gather_qmm_plan(M, N, K, n_indices, x_batches, n_experts, group_size=64, bits=4,
+                    dtype=BFLOAT16, transpose=True, workspace_bytes=None):
+    """The same for mlxrocm_gather_qmm."""
+    lib = load()
+    if workspace_bytes is None:
+        workspace_bytes = lib.mlxrocm_gather_qmm_workspace_size(
+            M, N, K, n_indices, n_experts, group_size, bits, dtype, int(transpose), 0)
+    buf = ctypes.create_string_buffer(1024)
+    rc = lib.mlxrocm_gather_qmm_plan(M, N, K, n_indices, x_batches, n_experts, group_size, bits,
+                                     dtype, int(transpose), workspace_bytes, buf, len(buf))
+    return rc, buf.value.decode()
+
+
+def dispatch_rules():
+    """[(name, evidence)] of the dispatch table of mlxrocm_qmm, in match order."""
+    lib = load()
+    return [(lib.mlxrocm_qmm_rule_name(i).decode(), lib.mlxrocm_qmm_rule_evidence(i).decode())
+            for i in range(lib.mlxrocm_qmm_rule_count())]
 
 
 def last_error() -> str:

@@ -31,6 +31,29 @@ class ApiRange {
   bool open_;
 };
 
+// Rehearsal of a call: the entry point walks its whole host path -- argument
+// checks, kernel choice, workspace claims against the size it was given -- but
+// every launcher records its name (and the parameters that shape its launch)
+// instead of launching.  Nothing touches the device, so the choice of kernels
+// can be listed and tested without a GPU (mlxrocm_qmm_plan).  Thread-local.
+class RehearsalScope {
+ public:
+  RehearsalScope(char* buf, size_t cap);
+  ~RehearsalScope();
+  RehearsalScope(const RehearsalScope&) = delete;
+  RehearsalScope& operator=(const RehearsalScope&) = delete;
+};
+bool rehearsing();
+// Appends "name" to the rehearsal's record ("a+b+c"); returns MLXROCM_OK.
+int note_launch(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+// At the top of a launcher: in a rehearsal, record and return.
+#define MLXROCM_REHEARSE(...)                    \
+  do {                                           \
+    if (::mlxrocm::rehearsing()) {               \
+      return ::mlxrocm::note_launch(__VA_ARGS__); \
+    }                                            \
+  } while (0)
+
 #define MLXROCM_HIP_TRY(expr)                    \
   do {                                           \
     hipError_t err__ = (expr);                   \

@@ -22,6 +22,54 @@ int fail(int status, const char* fmt, ...) {
   return status;
 }
 
+namespace {
+struct Rehearsal {
+  char* buf = nullptr;
+  size_t cap = 0;
+  size_t len = 0;
+  bool active = false;
+};
+thread_local Rehearsal g_rehearsal;
+} // namespace
+
+RehearsalScope::RehearsalScope(char* buf, size_t cap) {
+  g_rehearsal.buf = buf;
+  g_rehearsal.cap = cap;
+  g_rehearsal.len = 0;
+  g_rehearsal.active = true;
+  if (buf != nullptr && cap > 0) {
+    buf[0] = '\0';
+  }
+}
+
+RehearsalScope::~RehearsalScope() {
+  g_rehearsal = Rehearsal{};
+}
+
+bool rehearsing() {
+  return g_rehearsal.active;
+}
+
+int note_launch(const char* fmt, ...) {
+  Rehearsal& r = g_rehearsal;
+  if (!r.active || r.buf == nullptr || r.len + 2 >= r.cap) {
+    return MLXROCM_OK;
+  }
+  if (r.len > 0) {
+    r.buf[r.len++] = '+';
+  }
+  va_list args;
+  va_start(args, fmt);
+  const int n = vsnprintf(r.buf + r.len, r.cap - r.len, fmt, args);
+  va_end(args);
+  if (n > 0) {
+    const size_t room = r.cap - r.len - 1;
+    r.len += static_cast<size_t>(n) < room ? static_cast<size_t>(n) : room;
+  }
+  r.buf[r.len] = '\0';
+  return MLXROCM_OK;
+}
+
 int hip_fail(hipError_t err, const char* what) {
   snprintf(
       g_last_error,

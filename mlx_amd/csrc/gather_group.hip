@@ -274,6 +274,7 @@ int launch_gather_group(QmmArgs& a, int dtype, int tile_rows, void* workspace, h
   a.group_tiles = tiles;
   a.group_perm = perm;
   a.group_ntiles = n_tiles;
+  MLXROCM_REHEARSE(n <= kFusedMaxPairs ? "gather_group(fused)" : "gather_group(3 kernels)");
   a.group_tile_rows = tile_rows;
   if (n <= kFusedMaxPairs) {
     if (dtype == MLXROCM_BFLOAT16) {

@@ -130,7 +130,8 @@ bool qmm_slab_shape_ok(int rows, int N, int K, int gs, int bits);
 // Up to 16 rows of x with M * K * 2 bytes <= 64 KiB of LDS: all of K resident, no planes.
 // widen_codes.hip: 2/3-bit codes repacked as 4-bit, 5/6-bit as 8-bit (values kept)
 int widened_bits(int bits);
-int launch_widen_codes(const uint32_t* src, uint32_t* dst, size_t codes, int bits, hipStream_t s);
+int launch_widen_codes(
+    const uint32_t* src, uint32_t* dst, size_t dst_words, size_t codes, int bits, hipStream_t s);
 bool qmm_rows8_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmm_rows8(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 long qmm_slab_units(const QmmArgs& a); // work items of a plain call

@@ -169,6 +169,7 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint16_t* p, size_t n) {
 // memset node, so the call can be captured into a HIP graph.  Only degenerate
 // K == 0 products come here.
 int launch_zero_fill(void* p, size_t bytes, hipStream_t s) {
+  MLXROCM_REHEARSE("zero_fill");
   const size_t n = bytes / 2;
   const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
   zero_fill_kernel<<<blocks, 256, 0, s>>>(static_cast<uint16_t*>(p), n);
@@ -187,6 +188,7 @@ int launch_qmv_generic(
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
+  MLXROCM_REHEARSE("qmv_generic");
   return dispatch_dtype(dtype, [&](auto tval) {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
@@ -213,6 +215,7 @@ int launch_qmm_naive(
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
+  MLXROCM_REHEARSE(transpose ? "qmm_naive_t" : "qmm_naive_n");
   return dispatch_dtype(dtype, [&](auto tval) {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {

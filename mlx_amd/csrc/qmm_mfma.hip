@@ -800,12 +800,12 @@ constexpr size_t qmm_smem_bytes() {
 
 // Tile width (in units of 32 columns) that finishes first: a workgroup needs
 // time ~ NT per tile and the tiles run in ceil(tiles / CUs) rounds.
-int choose_nt(int M, int N, int L) {
+int choose_nt(int M, int N, int L, int min_nt = 5) {
   const long cus = compute_units();
   const long mt = (M + kBM - 1) / kBM;
   int best = 7;
   long best_cost = -1;
-  for (int nt = 7; nt >= 5; --nt) {
+  for (int nt = 7; nt >= min_nt; --nt) {
     const long tiles = mt * ((N + 32 * nt - 1) / (32 * nt)) * L;
     const long rounds = (tiles + cus - 1) / cus;
     const long cost = rounds * (nt * 8 + 3); // + fixed per-tile prologue/epilogue
@@ -929,6 +929,7 @@ int transpose_sb_for_qmm_n(
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] K=%d or batch=%d exceed the grid", K, batches);
   }
+  MLXROCM_REHEARSE("transpose_sb");
   if (dtype == MLXROCM_FLOAT32) {
     transpose_sb_kernel<float><<<grid, 256, 0, s>>>(
         static_cast<const float*>(scales), static_cast<const float*>(biases),
@@ -950,6 +951,7 @@ int transpose_sb_for_qmm_n(
 // / a.biases point at the transposed images made by transpose_sb_for_qmm_n.
 int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s) {
   const int gs_shift = shift_of(gs);
+  MLXROCM_REHEARSE("qmm_n_tile(ksplit=%d)", k_splits);
   if (k_splits > 1) {
     const dim3 grid((a.N + 32 * 6 - 1) / (32 * 6), (a.M + kBM - 1) / kBM, k_splits);
     return dtype == MLXROCM_BFLOAT16
@@ -969,13 +971,19 @@ int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_split
 
 int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
   const int gs_shift = shift_of(gs);
-  const int nt = choose_nt(a.M, a.N, a.L);
+  // (128-wide tiles as well: 4096 columns are 32 of them, so 2048 rows of x make
+  // exactly one round of 256 workgroups, where 160-wide tiles leave a fifth of
+  // the compute units idle)
+  const int nt = choose_nt(a.M, a.N, a.L, 4);
+  MLXROCM_REHEARSE("qmm_t_tile(nt=%d)", nt);
   const dim3 grid((a.N + 32 * nt - 1) / (32 * nt), (a.M + kBM - 1) / kBM, a.L);
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
       constexpr int B = decltype(bval)::value;
       switch (nt) {
+        case 4:
+          return launch_variant<T, T, T, B, 4, false>(a, gs_shift, grid, s);
         case 5:
           return launch_variant<T, T, T, B, 5, false>(a, gs_shift, grid, s);
         case 6:
@@ -1022,6 +1030,7 @@ int launch_qmm_mfma_ksplit(
   constexpr int kNT = 7;
   const int gs_shift = shift_of(gs);
   const dim3 grid((a.N + 32 * kNT - 1) / (32 * kNT), (a.M + kBM - 1) / kBM, k_splits);
+  MLXROCM_REHEARSE("qmm_t_tile(ksplit=%d)", k_splits);
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
@@ -1081,6 +1090,7 @@ int reduce_k_splits(const void* partial, void* out, size_t n, int k_splits, int 
   if (blocks > 0x7fffffffull) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] output too large for the split-K reduction");
   }
+  MLXROCM_REHEARSE("reduce_k_splits(%d)", k_splits);
   const float* p = static_cast<const float*>(partial);
   const unsigned g = static_cast<unsigned>(blocks);
   if (dtype == MLXROCM_FLOAT32) {
@@ -1103,6 +1113,7 @@ int launch_qmm_mfma_split(const QmmArgs& a, int gs, int bits, hipStream_t s, int
   const int gs_shift = shift_of(gs);
   const dim3 grid(
       (a.N + 32 * kNT - 1) / (32 * kNT), (a.M + kBM - 1) / kBM, k_splits > 1 ? k_splits : a.L);
+  MLXROCM_REHEARSE("qmm_t_tile_split_fp32(ksplit=%d)", k_splits);
   return dispatch_bits(bits, [&](auto bval) {
     constexpr int B = decltype(bval)::value;
     return launch_variant<bf16_t, float, float, B, kNT, false>(a, gs_shift, grid, s, k_splits);
@@ -1155,6 +1166,7 @@ int split_x_for_mfma(const void* x, void* xs, size_t rows, int K, hipStream_t s)
   if (blocks > 0x7fffffffull) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] x is too large to split");
   }
+  MLXROCM_REHEARSE("split_x");
   split_x_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(
       static_cast<const float*>(x), static_cast<bf16_t*>(xs), rows, K);
   MLXROCM_HIP_TRY(hipGetLastError());
@@ -1164,6 +1176,7 @@ int split_x_for_mfma(const void* x, void* xs, size_t rows, int K, hipStream_t s)
 // Gather grouped by expert: `a` carries the tile list; one grid row per
 // possible tile, rows past the device-side tile count exit at once.
 int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  MLXROCM_REHEARSE("qmm_t_tile_grouped");
   constexpr int kNT = 7;
   const int gs_shift = shift_of(gs);
   const dim3 grid(
@@ -1182,6 +1195,7 @@ int launch_qmm_mfma_grouped(const QmmArgs& a, int gs, int bits, int dtype, hipSt
 // the transposed images of all experts (transpose_sb_for_qmm_n), a.sb_batch_stride
 // is the distance between two experts' images.
 int launch_qmm_mfma_grouped_n(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s) {
+  MLXROCM_REHEARSE("qmm_n_tile_grouped");
   constexpr int kNT = 6;
   const int gs_shift = shift_of(gs);
   const dim3 grid(

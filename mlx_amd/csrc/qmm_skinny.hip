@@ -310,6 +310,7 @@ int launch_qmm_skinny(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] batch=%d exceeds the grid", a.L);
   }
+  MLXROCM_REHEARSE("qmm_skinny");
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {
@@ -345,6 +346,7 @@ int launch_qmm_skinny_grouped(const QmmArgs& a, int gs, int bits, int dtype, hip
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[gather_qmm] %d index pairs exceed the grid", a.L);
   }
+  MLXROCM_REHEARSE("qmm_skinny_grouped");
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {

@@ -1288,6 +1288,7 @@ int launch_qmm_slab(const QmmArgs& a, int gs, int bits, int dtype, void* planes,
   SlabPlan pl = make_plan(a.N, a.K, a.L);
   pl.planes = static_cast<float*>(planes);
   pl.plane_elems = static_cast<int64_t>(a.L) * a.M * a.N;
+  MLXROCM_REHEARSE("qmm_slab(tiles=%d,ranges=%d)", mt, pl.ranges);
   int rc = launch_any<0>(a, pl, gs, dtype, mt, s);
   if (rc != MLXROCM_OK || pl.ranges <= 1) {
     return rc;
@@ -1335,6 +1336,9 @@ int launch_qmm_slab_grouped(
   SlabPlan pl = make_plan(a.N, a.K, gather_group_max_tiles(a.L, a.n_experts, tile_rows));
   pl.planes = static_cast<float*>(planes);
   pl.plane_elems = static_cast<int64_t>(a.L) * a.N;
+  MLXROCM_REHEARSE(
+      "qmm_slab_grouped(%s,tile=%d,ranges=%d)", plan_in_kernel ? "plans" : "planned", tile_rows,
+      pl.ranges);
   // (mode 1 never runs with one tile of x: the planning kernel makes 32-row tiles)
   int rc = plan_in_kernel ? launch_any<2>(a, pl, gs, dtype, one_tile ? 1 : 2, s)
                           : launch_any<1>(a, pl, gs, dtype, 2, s);
@@ -1398,15 +1402,15 @@ int launch_qmm_rows8(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t 
   const int kw = rows8_kw(a.K);
   const int stages = rows8_stages(a.M, a.K, gs, kw);
   const size_t smem = rows8_smem_bytes(a.M, a.K, gs, kw, stages);
+  MLXROCM_REHEARSE("qmm_rows8(kw=%d,slots=%d)", kw, stages);
   const dim3 grid((a.N + kR8Rows - 1) / kR8Rows, a.L);
   auto go = [&](auto kern) -> int {
-    static bool configured = false; // per instantiation
-    if (!configured) {
-      MLXROCM_HIP_TRY(hipFuncSetAttribute(
-          reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-          160 * 1024));
-      configured = true;
-    }
+    // every instantiation decays to the same pointer type, so this lambda exists
+    // once: the attribute is set on each launch (a host-side table lookup), not
+    // behind a flag the kernels would share
+    MLXROCM_HIP_TRY(hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+        160 * 1024));
     kern<<<grid, 64 * kR8Tiles * kw, smem, s>>>(a);
     MLXROCM_HIP_TRY(hipGetLastError());
     return static_cast<int>(MLXROCM_OK);

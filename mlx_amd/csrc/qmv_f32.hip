@@ -232,6 +232,7 @@ int launch_qmv_f32(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s)
     pl.cpw = 1;
     pl.kw = need <= 1 ? 1 : (need <= 2 ? 2 : 4);
   }
+  MLXROCM_REHEARSE("qmv_f32");
   const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
   const int rows_per_wg = (kF32Threads / 64 / pl.kw) * kF32RowsInFlight;
   const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.L);

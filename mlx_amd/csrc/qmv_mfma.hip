@@ -528,6 +528,7 @@ int launch_qmv_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] batch=%d exceeds the grid", a.L);
   }
+  MLXROCM_REHEARSE("qmv_mfma");
   auto run = [&](auto tval, auto bval, auto gval) -> int {
     using T = decltype(tval);
     constexpr int B = decltype(bval)::value;

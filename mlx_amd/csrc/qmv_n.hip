@@ -252,6 +252,7 @@ int reduce_planes(const float* partial, void* out, size_t n, int splits, int dty
   if (n % 4 != 0 || blocks > 0x7fffffffull) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] output of %zu elements does not fit the plane reduction", n);
   }
+  MLXROCM_REHEARSE("reduce_planes(%d)", splits);
   const unsigned g = static_cast<unsigned>(blocks);
   return dispatch_dtype(dtype, [&](auto tval) {
     using T = decltype(tval);
@@ -294,6 +295,7 @@ int launch_qmv_n(const QmmArgs& a, int gs, int bits, int dtype, float* partial, 
   if (pl.splits > 1 && partial == nullptr) {
     return fail(MLXROCM_INVALID_ARGUMENT, "[qmv] the K ranges need a partial buffer");
   }
+  MLXROCM_REHEARSE("qmv_n(rows=%d,ranges=%d)", a.M, pl.splits);
   float* part = pl.splits > 1 ? partial : nullptr;
   auto go = [&](auto tval, auto bval, auto mval) -> int {
     using T = decltype(tval);

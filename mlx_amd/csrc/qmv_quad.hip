@@ -475,6 +475,7 @@ int launch_qmv_quad(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
   if (pl.kw == 0) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] K=%d is not covered by the quad kernel", a.K);
   }
+  MLXROCM_REHEARSE("qmv_quad(kw=%d,sets=%d)", pl.kw, a.M <= 4 ? 1 : 2);
   const int gs_shift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
   const int rw = 8 / pl.kw;
   const int mb = a.M <= 4 ? 1 : 2;

@@ -682,6 +682,7 @@ int launch_qmv_stream_glu(const QmmArgs& a, int gs, int bits, int dtype, hipStre
   if (!qmv_stream_glu_supported(a, gs, bits, dtype)) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] shape not covered by the gated GEMV");
   }
+  MLXROCM_REHEARSE("qmv_stream_glu");
   auto run = [&](auto tval, auto bval, auto gval) -> int {
     using T = decltype(tval);
     constexpr int B = decltype(bval)::value;
@@ -753,6 +754,7 @@ int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t
     if (grid.y > 65535u) {
       return fail(MLXROCM_UNSUPPORTED, "[qmv] batch=%d exceeds the grid", a.L);
     }
+    MLXROCM_REHEARSE("qmv_stream(rw=%d,kw=%d,rm=%d)", pl.rw, pl.kw, pl.rm);
     auto go = [&](auto mval, auto rwv, auto kwv, auto rmv) -> int {
       constexpr int M = decltype(mval)::value;
       constexpr int RW = decltype(rwv)::value;

@@ -286,6 +286,7 @@ int launch_qmv_wide(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmv] batch=%d exceeds the grid", a.L);
   }
+  MLXROCM_REHEARSE("qmv_wide");
   auto run = [&](auto tval) -> int {
     using T = decltype(tval);
     return dispatch_bits(bits, [&](auto bval) {

@@ -69,14 +69,27 @@ int widened_bits(int bits) {
   }
 }
 
-// `codes` codes (a multiple of 32) from src to dst.
-int launch_widen_codes(const uint32_t* src, uint32_t* dst, size_t codes, int bits, hipStream_t s) {
+// `codes` codes (a multiple of 32) from src to dst, which holds `dst_words`
+// words.  Thread t reads words [t bits, (t + 1) bits) and writes words
+// [t wide, (t + 1) wide), t < codes / 32: the last word read is
+// codes / 32 * bits - 1 (the packed matrix has exactly that many), the last
+// word written codes / 32 * wide - 1, checked against the region here.
+int launch_widen_codes(
+    const uint32_t* src, uint32_t* dst, size_t dst_words, size_t codes, int bits, hipStream_t s) {
   const size_t blocks = codes / 32;
   const size_t grid = (blocks + 255) / 256;
   if (codes % 32 != 0 || grid > 0x7fffffffull) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] cannot repack %zu codes of %d bits", codes, bits);
   }
+  const size_t wide = static_cast<size_t>(widened_bits(bits));
+  if (wide == 0 || blocks > SIZE_MAX / 8 / sizeof(uint32_t) || blocks * wide > dst_words) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[qmm] repacking %zu codes of %d bits writes %zu words; the region holds %zu",
+        codes, bits, blocks * wide, dst_words);
+  }
   const unsigned g = static_cast<unsigned>(grid);
+  MLXROCM_REHEARSE("widen_codes(%d->%d)", bits, widened_bits(bits));
   switch (bits) {
     case 2:
       widen_codes_kernel<2, 4><<<g, 256, 0, s>>>(src, dst, blocks);

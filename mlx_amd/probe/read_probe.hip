@@ -9,12 +9,17 @@
 //   rolling<D>  a persistent grid (4 workgroups per CU); each wave keeps D
 //               1 KiB loads in flight and walks the buffer with a grid stride
 //   empty       a grid of the same size whose waves exit at once (launch cost)
-// Built by mlx_amd/_build.py (build_read_probe); prints one table.
+// Built by mlx_amd/_build.py (build_read_probe) into mlx_amd/lib/read_probe.
+// Without arguments it prints the whole table; with --floor it times only the
+// 33 MB read, the same read from the cache and the empty grid, 1800 launches per
+// timed region like bench.py, and prints one JSON line -- bench.py runs it that
+// way in a child process and reports the figures beside the decode kernel's.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <string>
 #include <vector>
 
 #define HIP_OK(expr)                                                          \
@@ -130,7 +135,8 @@ struct Probe {
   }
 };
 
-int main() {
+int main(int argc, char** argv) {
+  const bool floor_only = argc > 1 && std::string(argv[1]) == "--floor";
   // W + scales + biases of the 4096 x 14336, 4-bit, group-64 decode weight,
   // rounded to whole KiB.
   const size_t unit = (static_cast<size_t>(4096) * 14336 / 2 + 2 * 2 * 4096 * 14336 / 64) / 1024 * 1024;
@@ -147,6 +153,24 @@ int main() {
   hipDeviceProp_t prop;
   HIP_OK(hipGetDeviceProperties(&prop, 0));
   const int cus = prop.multiProcessorCount;
+  if (floor_only) {
+    const size_t n_vec = unit / 16;
+    const unsigned grid = static_cast<unsigned>((n_vec / 64 / 4 + 3) / 4);
+    const float cold = probe.time(ring, 100, [&](int i, hipStream_t s) {
+      stream_kernel<4><<<grid, 256, 0, s>>>(bufs[i % ring], n_vec, sink);
+    });
+    const float hot = probe.time(ring, 100, [&](int, hipStream_t s) {
+      stream_kernel<4><<<grid, 256, 0, s>>>(bufs[0], n_vec, sink);
+    });
+    const float empty = probe.time(ring, 100, [&](int, hipStream_t s) {
+      empty_kernel<<<1792, 256, 0, s>>>(sink, 0);
+    });
+    std::printf(
+        "{\"bytes\": %zu, \"read_only_floor_us\": %.3f, \"read_only_cache_resident_us\": %.3f, "
+        "\"empty_launch_us\": %.3f, \"launches_per_region\": %d, \"repeats\": 7}\n",
+        unit, cold, hot, empty, ring * 100);
+    return 0;
+  }
   std::printf("device: %s, %d CUs; unit = %zu bytes\n", prop.name, cus, unit);
   std::printf("%-28s %8s %10s %10s\n", "kernel", "MB", "us/launch", "GB/s");
   auto row = [](const char* name, size_t bytes, float us) {

@@ -52,19 +52,35 @@ void CompletionQueue::thread_main(std::shared_ptr<Shared> shared) {
       shared->queue.pop_front();
       shared->running = true;
     }
-    int rc = mlxrocm_event_synchronize(batch.event);
+    // (a batch without an event was committed after the stream had been waited for)
+    int rc = batch.event != nullptr ? mlxrocm_event_synchronize(batch.event) : MLXROCM_OK;
     std::string message;
     if (rc != MLXROCM_OK) {
       message = mlxrocm_last_error();
     }
     // Handlers run even after an error: they balance task counters that the
-    // evaluating thread may be blocked on.
+    // evaluating thread may be blocked on.  One that throws must not end the
+    // process from this thread: its message reaches the next commit instead.
     for (auto& fn : batch.handlers) {
-      fn();
+      try {
+        fn();
+      } catch (const std::exception& e) {
+        if (rc == MLXROCM_OK) {
+          rc = MLXROCM_HIP_ERROR;
+          message = std::string("a completion handler threw: ") + e.what();
+        }
+      } catch (...) {
+        if (rc == MLXROCM_OK) {
+          rc = MLXROCM_HIP_ERROR;
+          message = "a completion handler threw";
+        }
+      }
     }
     batch.handlers.clear();
     batch.retained.clear(); // may free buffers: outside the lock
-    (void)mlxrocm_event_destroy(batch.event);
+    if (batch.event != nullptr) {
+      (void)mlxrocm_event_destroy(batch.event);
+    }
     {
       std::lock_guard<std::mutex> lock(shared->mtx);
       shared->running = false;
@@ -95,26 +111,47 @@ void CompletionQueue::rethrow_thread_error() {
 }
 
 void CompletionQueue::commit() {
-  rethrow_thread_error();
   if (!has_pending()) {
+    rethrow_thread_error();
     return;
   }
+  // The batch is handed to the completion thread whatever fails below: its
+  // handlers balance task counters that the evaluating thread may block on
+  // (scheduler::wait_for_one), so they must run even when this call throws.
   Batch batch;
-  check(mlxrocm_event_create_blocking(&batch.event));
-  int rc = mlxrocm_event_record(batch.event, stream_);
-  if (rc != MLXROCM_OK) {
-    (void)mlxrocm_event_destroy(batch.event);
-    check(rc);
-  }
   batch.retained = std::move(retained_);
   batch.handlers = std::move(handlers_);
   retained_.clear();
   handlers_.clear();
+  std::string failure;
+  int rc = mlxrocm_event_create_blocking(&batch.event);
+  if (rc == MLXROCM_OK) {
+    rc = mlxrocm_event_record(batch.event, stream_);
+    if (rc != MLXROCM_OK) {
+      failure = mlxrocm_last_error();
+      (void)mlxrocm_event_destroy(batch.event);
+      batch.event = nullptr;
+    }
+  } else {
+    failure = mlxrocm_last_error();
+    batch.event = nullptr;
+  }
+  if (batch.event == nullptr) {
+    // no event to wait for: the buffers may only be dropped once the stream is idle
+    (void)mlxrocm_stream_synchronize(stream_);
+  }
   {
     std::lock_guard<std::mutex> lock(shared_->mtx);
     shared_->queue.push_back(std::move(batch));
   }
   shared_->work.notify_one();
+  if (rc != MLXROCM_OK) {
+    if (rc == MLXROCM_INVALID_ARGUMENT) {
+      throw std::invalid_argument(failure);
+    }
+    throw std::runtime_error(failure);
+  }
+  rethrow_thread_error();
 }
 
 void CompletionQueue::synchronize() {

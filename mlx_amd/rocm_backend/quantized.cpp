@@ -9,6 +9,7 @@
 // retain what the kernels read.  Every arithmetic decision (kernel choice,
 // tiling) lives behind mlxrocm_qmm / mlxrocm_gather_qmm.
 #include <sstream>
+#include <limits>
 #include <stdexcept>
 
 #include "mlx/allocator.h"
@@ -89,6 +90,19 @@ int64_t matrix_stride(const array& a) {
   return a.strides()[a.ndim() - 3];
 }
 
+// A temporary of at least `bytes` bytes.  Shapes are 32-bit, so the array is
+// [rows, 1 MiB] of uint8: workspaces beyond 2 GiB keep an exact row count.
+array workspace_array(size_t bytes) {
+  constexpr size_t kRow = size_t(1) << 20;
+  const size_t rows = (bytes + kRow - 1) / kRow;
+  if (rows > static_cast<size_t>(std::numeric_limits<int>::max())) {
+    throw std::runtime_error("[quantized_matmul] workspace beyond 2^51 bytes");
+  }
+  array ws({static_cast<int>(rows), static_cast<int>(kRow)}, uint8, nullptr, {});
+  ws.set_data(allocator::malloc(rows * kRow));
+  return ws;
+}
+
 bool single_batch_stride(const array& a) {
   // true when element i of the flattened leading dims sits at i * stride
   int64_t expect = matrix_stride(a);
@@ -126,7 +140,11 @@ void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
   if (w.ndim() == 2 && L > 1) {
     // x is row-contiguous here, so the batch folds into its rows and the weight
     // is read once for all of them (mlx/backend/metal/quantized.cpp:1799-1801)
-    M *= L;
+    const int64_t rows = int64_t(M) * L;
+    if (rows > std::numeric_limits<int>::max()) {
+      throw std::runtime_error("[quantized_matmul] more than 2^31 - 1 rows of x");
+    }
+    M = static_cast<int>(rows);
     L = 1;
   }
   const int dt = dtype_code(x.dtype(), "quantized_matmul");
@@ -136,8 +154,7 @@ void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
       M, N, K, L, w.ndim() > 2, group_size_, bits_, dt, transpose_ ? 1 : 0);
   void* ws_ptr = nullptr;
   if (ws_bytes > 0) {
-    array ws({static_cast<int>(ws_bytes)}, uint8, nullptr, {});
-    ws.set_data(allocator::malloc(ws_bytes));
+    array ws = workspace_array(ws_bytes);
     enc.add_temporary(ws);
     ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
   }
@@ -200,8 +217,7 @@ void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
       M, N, K, n_idx, n_experts, group_size_, bits_, dt, transpose_, right_sorted_);
   void* ws_ptr = nullptr;
   if (ws_bytes > 0) {
-    array ws({static_cast<int>(ws_bytes)}, uint8, nullptr, {});
-    ws.set_data(allocator::malloc(ws_bytes));
+    array ws = workspace_array(ws_bytes);
     enc.add_temporary(ws);
     ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
   }

@@ -16,19 +16,30 @@ RocmBuffer::~RocmBuffer() {
 
 void* RocmBuffer::device_access(mlxrocm_stream_t stream, bool will_write) {
   std::lock_guard<std::mutex> lock(mtx_);
-  // A stale device side means host_access() ran last, and that waited for all
-  // GPU work on the buffer: the upload cannot overtake an older kernel.
+  // A stale device side means host_access() ran last, and that waited for every
+  // stream with work on the buffer: the upload cannot overtake an older kernel.
   if (!device_current_) {
     check(mlxrocm_memcpy_h2d(device_, host_, size_, stream));
     device_current_ = true;
   }
   if (will_write) {
     host_current_ = false;
+    last_stream_ = stream;
+  } else if (last_stream_ == nullptr) {
+    last_stream_ = stream;
   }
-  last_stream_ = stream;
-  gpu_work_pending_ = true;
+  note_pending(stream);
   touched_by_gpu_ = true;
   return device_;
+}
+
+void RocmBuffer::note_pending(mlxrocm_stream_t stream) {
+  for (mlxrocm_stream_t s : pending_streams_) {
+    if (s == stream) {
+      return;
+    }
+  }
+  pending_streams_.push_back(stream);
 }
 
 void* RocmBuffer::host_access() {
@@ -37,15 +48,17 @@ void* RocmBuffer::host_access() {
     check(mlxrocm_host_malloc(&host_, size_));
   }
   if (!host_current_ && touched_by_gpu_) {
-    // Ordered behind the kernels that produced the bytes: same stream.
+    // Ordered behind the kernels that produced the bytes: the last writer's stream.
     check(mlxrocm_memcpy_d2h(host_, device_, size_, last_stream_));
-    gpu_work_pending_ = true;
+    note_pending(last_stream_);
   }
-  if (gpu_work_pending_) {
-    // Also covers an upload still reading the mirror the caller may now write.
-    check(mlxrocm_stream_synchronize(last_stream_));
-    gpu_work_pending_ = false;
+  // Every stream that used the buffer since the last host access: writers,
+  // readers (the next upload must not overwrite what they still read) and an
+  // upload still reading the mirror the caller may now write.
+  for (mlxrocm_stream_t s : pending_streams_) {
+    check(mlxrocm_stream_synchronize(s));
   }
+  pending_streams_.clear();
   host_current_ = true;
   device_current_ = false;
   return host_;

@@ -30,6 +30,7 @@
 
 #include <cstddef>
 #include <mutex>
+#include <vector>
 
 #include "mlx_rocm_qmm.h"
 
@@ -54,6 +55,7 @@ class RocmBuffer {
   void* host_access();
 
  private:
+  void note_pending(mlxrocm_stream_t stream);
   std::mutex mtx_;
   size_t size_;
   void* device_{nullptr};
@@ -61,8 +63,10 @@ class RocmBuffer {
   bool device_current_{true}; // fresh memory: nothing to lose on either side
   bool host_current_{false};
   bool touched_by_gpu_{false}; // false: fresh memory, no bytes worth downloading
-  bool gpu_work_pending_{false}; // enqueued on last_stream_, not yet waited for
-  mlxrocm_stream_t last_stream_{nullptr};
+  // Streams with work on the buffer that host_access() has not waited for yet
+  // (a kernel that only reads may run on another stream than the last writer).
+  std::vector<mlxrocm_stream_t> pending_streams_;
+  mlxrocm_stream_t last_stream_{nullptr}; // orders the download behind the last writer
 };
 
 } // namespace mlx::core::rocm

@@ -154,6 +154,53 @@ void test_completion_error_reaches_the_caller_and_handlers_still_run() {
   q.synchronize(); // the error was consumed
 }
 
+void test_failed_commit_still_runs_the_handlers() {
+  // eval() counts the task before it commits (scheduler::notify_new_task), so a
+  // commit that cannot record its event must still hand the handlers over, or
+  // wait_for_one() would block for good.
+  CompletionQueue q;
+  TaskCounter tasks;
+  std::atomic<bool> kernel_done{false};
+  mock_launch(q.stream(), [&] {
+    std::this_thread::sleep_for(10ms);
+    kernel_done = true;
+  });
+  tasks.notify_new_task();
+  q.on_complete([&] { tasks.notify_task_completion(); });
+  mock_fail_event_record(1);
+  bool threw = false;
+  try {
+    q.commit();
+  } catch (const std::runtime_error& e) {
+    threw = std::strstr(e.what(), "hipEventRecord") != nullptr;
+  }
+  CHECK(threw);
+  // no later commit: the handler has to arrive by itself, behind the kernel
+  for (int i = 0; i < 200 && tasks.n_active() != 0; ++i) {
+    std::this_thread::sleep_for(5ms);
+  }
+  CHECK(tasks.n_active() == 0);
+  CHECK(kernel_done.load());
+  q.synchronize();
+}
+
+void test_throwing_handler_is_reported_not_fatal() {
+  CompletionQueue q;
+  std::atomic<bool> second_ran{false};
+  q.on_complete([] { throw std::runtime_error("handler failure"); });
+  q.on_complete([&] { second_ran = true; });
+  q.commit();
+  bool threw = false;
+  try {
+    q.synchronize();
+  } catch (const std::runtime_error& e) {
+    threw = std::strstr(e.what(), "handler failure") != nullptr;
+  }
+  CHECK(threw);
+  CHECK(second_ran.load());
+  q.synchronize();
+}
+
 void test_queue_destroyed_with_work_in_flight() {
   std::atomic<bool> released{false};
   {
@@ -327,6 +374,35 @@ void test_residency_transitions() {
   check(mlxrocm_stream_destroy(s));
 }
 
+void test_host_access_waits_for_readers_on_other_streams() {
+  mlxrocm_stream_t writer = nullptr, reader = nullptr;
+  check(mlxrocm_stream_create(&writer));
+  check(mlxrocm_stream_create(&reader));
+  {
+    RocmBuffer buf(sizeof(int));
+    *static_cast<int*>(buf.host_access()) = 7;
+    int* w = static_cast<int*>(buf.device_access(writer, /* will_write */ true));
+    mock_launch(writer, [w] { *w = 8; });
+    check(mlxrocm_stream_synchronize(writer));
+    // a slow kernel on another stream only reads the buffer ...
+    std::atomic<bool> read_done{false};
+    int seen = 0;
+    const int* r = static_cast<const int*>(buf.device_access(reader, false));
+    mock_launch(reader, [&, r] {
+      std::this_thread::sleep_for(30ms);
+      seen = *r;
+      read_done = true;
+    });
+    // ... and the CPU asks for the bytes: it must not get them (and the right to
+    // overwrite the device side at the next upload) before that kernel is done
+    int* host = static_cast<int*>(buf.host_access());
+    CHECK(read_done.load());
+    CHECK(seen == 8 && *host == 8);
+  }
+  check(mlxrocm_stream_destroy(writer));
+  check(mlxrocm_stream_destroy(reader));
+}
+
 void test_residency_is_safe_from_two_threads() {
   mlxrocm_stream_t s = nullptr;
   check(mlxrocm_stream_create(&s));
@@ -357,10 +433,13 @@ int main() {
   test_more_than_ten_active_tasks_do_not_deadlock();
   test_synchronize_waits_for_unbatched_work_too();
   test_completion_error_reaches_the_caller_and_handlers_still_run();
+  test_failed_commit_still_runs_the_handlers();
+  test_throwing_handler_is_reported_not_fatal();
   test_queue_destroyed_with_work_in_flight();
   test_signal_issued_before_and_after_the_wait();
   test_signal_orders_one_stream_behind_another();
   test_residency_transitions();
+  test_host_access_waits_for_readers_on_other_streams();
   test_residency_is_safe_from_two_threads();
   std::this_thread::sleep_for(50ms); // let a detached completion thread exit
   mock_shutdown();

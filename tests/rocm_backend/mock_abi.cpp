@@ -92,6 +92,7 @@ struct Registry {
   std::atomic<long> device_allocs{0}, host_allocs{0}, events{0};
   std::atomic<long> h2d{0}, d2h{0}, syncs{0};
   std::atomic<int> fail_event_sync{0};
+  std::atomic<int> fail_event_record{0};
 };
 
 Registry& reg() {
@@ -134,6 +135,10 @@ MockCounters mock_counters() {
 
 void mock_fail_event_synchronize(int n) {
   reg().fail_event_sync.store(n);
+}
+
+void mock_fail_event_record(int n) {
+  reg().fail_event_record.store(n);
 }
 
 void mock_shutdown() {
@@ -258,6 +263,12 @@ int mlxrocm_event_destroy(mlxrocm_event_t event) {
   return MLXROCM_OK;
 }
 int mlxrocm_event_record(mlxrocm_event_t event, mlxrocm_stream_t stream) {
+  int left = reg().fail_event_record.load();
+  while (left > 0 && !reg().fail_event_record.compare_exchange_weak(left, left - 1)) {
+  }
+  if (left > 0) {
+    return fail(MLXROCM_HIP_ERROR, "[mock] hipEventRecord failed");
+  }
   auto* e = static_cast<MockEvent*>(event);
   uint64_t gen;
   {

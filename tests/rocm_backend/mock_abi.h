@@ -22,5 +22,7 @@ struct MockCounters {
 MockCounters mock_counters();
 // Makes the next `n` mlxrocm_event_synchronize calls fail with MLXROCM_HIP_ERROR.
 void mock_fail_event_synchronize(int n);
+// Makes the next `n` mlxrocm_event_record calls fail with MLXROCM_HIP_ERROR.
+void mock_fail_event_record(int n);
 // Joins every mock stream thread (after draining it); call at the end of main.
 void mock_shutdown();

@@ -222,28 +222,32 @@ def test_gather_qmm_grouped_by_expert_not_transposed(oracle, gpu, dtype, bits, g
 
 
 @pytest.mark.parametrize("index_dtype", (torch.int64, torch.int32, torch.uint32, torch.int16))
-def test_gather_qmm_many_pairs_and_index_types(gpu, index_dtype):
+def test_gather_qmm_many_pairs_and_index_types(oracle, gpu, index_dtype):
     """More than 16384 pairs take the three-kernel grouping (fewer take the
-    one-workgroup form); both must give what a plain matmul per expert gives.
-    Index tensors of every integer width are accepted: 32-bit ones are used as
-    they are, others are converted."""
+    one-workgroup form); every pair is held to the fp64 product of the exact
+    affine weights and to the CPU oracle's loop over the pairs
+    (cpu/quantized.cpp:700-747).  Index tensors of every integer width are
+    accepted: 32-bit ones are used as they are, others are converted."""
     E, N, K, X = 4, 96, 128, 50
     dtype = torch.bfloat16
-    w = normal_weights((E, N, K), dtype, std=0.5).to(gpu)
-    wq, s, b = mlx_amd.quantize(w, 64, 4)
-    w_hat = mlx_amd.dequantize(wq, s, b, 64, 4).float()          # [E, N, K]
-    x = activations((X, 1, K), dtype).to(gpu)
+    w = normal_weights((E, N, K), dtype, std=0.5)
+    wq, s, b = oracle.quantize(w, 64, 4)
+    w_hat = exact_affine_weights(wq, s, b, 64, 4)                 # [E, N, K] fp64
+    x = activations((X, 1, K), dtype)
+    gx, gwq, gs_, gb = _to(gpu, x, wq, s, b)
     for T in (3000, 20000):
         g = torch.Generator().manual_seed(T)
         rhs = torch.randint(0, E, (T,), generator=g)
         lhs = torch.randint(0, X, (T,), generator=g)
-        got = mlx_amd.gather_qmm(x, wq, s, b, lhs.to(index_dtype).to(gpu),
-                                 rhs.to(index_dtype).to(gpu), True, 64, 4)
+        got = mlx_amd.gather_qmm(gx, gwq, gs_, gb, lhs.to(index_dtype).to(gpu),
+                                 rhs.to(index_dtype).to(gpu), True, 64, 4).cpu()
         assert got.shape == (T, 1, N)
-        want = torch.einsum("tk,tnk->tn", x.reshape(X, K).float()[lhs.to(gpu)],
-                            w_hat[rhs.to(gpu)])
-        err = float((got.reshape(T, N).float() - want).abs().max())
-        assert err <= 2 ** -7 * float(want.abs().max()), (T, err)
+        exact = torch.einsum("tk,tnk->tn", x.reshape(X, K).double()[lhs], w_hat[rhs])
+        err = float((got.reshape(T, N).double() - exact).abs().max())
+        assert err <= exact_tolerance(dtype, K, x, w_hat, exact), (T, err)
+        ref = oracle.gather_qmm(x, wq, s, b, lhs, rhs, True, 64, 4).reshape(T, N).double()
+        tol = matmul_tolerance(dtype, K, x, w_hat) + float((ref - exact).abs().max())
+        assert float((got.reshape(T, N).double() - ref).abs().max()) <= tol, T
 
 
 def test_gather_qmm_grouped_matches_ungrouped(gpu):
@@ -270,45 +274,6 @@ def test_gather_qmm_grouped_matches_ungrouped(gpu):
     diff = (grouped.float() - single.float()).abs().max()
     scale = single.float().abs().max()
     assert float(diff) <= 2 ** -7 * float(scale)
-
-
-def test_gather_qmm_full_size_moe_permutation_invariant(oracle, gpu):
-    """8 experts of [14336, 4096], 4-bit group 64, T = 2048 tokens routed top-2
-    (seeded): the grouped GEMM gives, for every index pair, a row that depends on
-    that pair only -- so the run on expert-sorted pairs must reproduce the
-    unsorted run bit for bit after un-permuting -- and sampled rows agree with
-    the CPU oracle."""
-    E, N, K, T = 8, 14336, 4096, 2048
-    g = torch.Generator().manual_seed(0)
-    w = (torch.randn((E, N, K), generator=g) * 0.02).to(torch.bfloat16)
-    wq, s, b = mlx_amd.quantize(w.to(gpu), 64, 4)
-    del w
-    x = torch.randn((T, 1, 1, K), generator=g).to(torch.bfloat16)
-    idx = torch.randint(0, E, (T, 2), generator=torch.Generator().manual_seed(0))
-    gx, gidx = x.to(gpu), idx.to(gpu)
-    unsorted = mlx_amd.gather_qmm(gx, wq, s, b, rhs_indices=gidx, transpose=True,
-                                  group_size=64, bits=4)
-    assert unsorted.shape == (T, 2, 1, N)
-    flat = gidx.reshape(-1)
-    order = torch.argsort(flat, stable=True)
-    xs = gx.reshape(T, 1, K)[order // 2].contiguous()
-    ys = mlx_amd.gather_qmm(xs, wq, s, b, rhs_indices=flat[order].contiguous(),
-                            transpose=True, group_size=64, bits=4, sorted_indices=True)
-    resorted = ys[torch.argsort(order)].reshape(T, 2, 1, N)
-    assert torch.equal(unsorted.view(torch.int16), resorted.view(torch.int16))
-    # oracle on a few pairs
-    cq = [t.cpu() for t in (wq, s, b)]
-    for t, j in ((0, 0), (777, 1), (2047, 1)):
-        e = int(idx[t, j])
-        ref = oracle.qmm(x[t].reshape(1, K), cq[0][e], cq[1][e], cq[2][e], True, 64, 4)
-        w_hat = exact_affine_weights(cq[0][e], cq[1][e], cq[2][e], 64, 4)
-        exact = x[t].reshape(1, K).double() @ w_hat.T
-        got = unsorted[t, j].cpu().double()
-        tol = matmul_tolerance(torch.bfloat16, K, x[t], w_hat) + float(
-            (ref.double() - exact).abs().max())
-        assert float((got - ref.double()).abs().max()) <= tol
-        assert float((got - exact).abs().max()) <= exact_tolerance(
-            torch.bfloat16, K, x[t], w_hat, exact)
 
 
 @pytest.mark.parametrize("bits,gs", ((4, 64), (5, 32), (8, 128)))
@@ -398,6 +363,59 @@ def test_gather_qmm_full_size_moe_few_tokens(oracle, gpu, mixtral_stack, T):
     cq = [t.cpu() for t in (wq, s, b)]
     for p in sorted({0, (2 * T) // 3, 2 * T - 1}):
         t, j = p // 2, p % 2
+        e = int(idx[t, j])
+        xr = x[t].reshape(1, K)
+        ref = oracle.qmm(xr, cq[0][e], cq[1][e], cq[2][e], True, 64, 4).double()
+        exact = (xr.to(gpu).double() @ w_hat[e].T).cpu()
+        tol = 2e-2 * (K ** 0.5) * x_absmax * float(w_hat[e].abs().max()) + float(
+            (ref - exact).abs().max())
+        assert float((unsorted[t, j].cpu().double() - ref).abs().max()) <= tol
+
+
+def test_gather_qmm_full_size_moe_prefill(oracle, gpu, mixtral_stack):
+    """T = 2048 tokens routed top-2 over the 8 full-size experts (seeded): the
+    grouped GEMM.  Every one of the 4096 index pairs against the fp64 product,
+    expert by expert; the run on expert-sorted pairs reproduces the unsorted
+    run bit for bit after un-permuting (a row depends on its own pair only);
+    a few pairs against the CPU oracle."""
+    wq, s, b, w_hat = mixtral_stack
+    E, N, K, T = 8, 14336, 4096, 2048
+    x = activations((T, 1, 1, K), torch.bfloat16, seed=T)
+    idx = torch.randint(0, E, (T, 2), generator=torch.Generator().manual_seed(0))
+    gx, gidx = x.to(gpu), idx.to(gpu)
+    unsorted = mlx_amd.gather_qmm(gx, wq, s, b, rhs_indices=gidx, transpose=True,
+                                  group_size=64, bits=4)
+    assert unsorted.shape == (T, 2, 1, N)
+    flat = gidx.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    xs = gx.reshape(T, 1, K)[order // 2].contiguous()
+    ys = mlx_amd.gather_qmm(xs, wq, s, b, rhs_indices=flat[order].contiguous(),
+                            transpose=True, group_size=64, bits=4, sorted_indices=True)
+    torch.cuda.synchronize()
+    resorted = ys[torch.argsort(order)].reshape(T, 2, 1, N)
+    assert torch.equal(unsorted.view(torch.int16), resorted.view(torch.int16))
+    del ys, resorted, xs
+    # every pair against fp64, expert by expert
+    got = unsorted.reshape(2 * T, N)
+    xd = gx.reshape(T, K).double()
+    tok = torch.arange(2 * T, device=gpu) // 2
+    x_absmax = float(x.abs().max())
+    checked = 0
+    for e in range(E):
+        pairs = torch.nonzero(flat == e).reshape(-1)
+        if pairs.numel() == 0:
+            continue
+        exact = xd[tok[pairs]] @ w_hat[e].T
+        err = float((got[pairs].double() - exact).abs().max())
+        tol = exact_tolerance_from(torch.bfloat16, K, x_absmax, float(w_hat[e].abs().max()),
+                                   float(exact.abs().max()))
+        assert err <= tol, f"expert {e}: {err} > {tol}"
+        checked += int(pairs.numel())
+        del exact
+    assert checked == 2 * T
+    # the oracle on a few pairs
+    cq = [t.cpu() for t in (wq, s, b)]
+    for t, j in ((0, 0), (777, 1), (2047, 1)):
         e = int(idx[t, j])
         xr = x[t].reshape(1, K)
         ref = oracle.qmm(xr, cq[0][e], cq[1][e], cq[2][e], True, 64, 4).double()

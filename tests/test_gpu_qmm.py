@@ -136,6 +136,27 @@ def test_odd_width_stress_matmul(oracle, gpu, dtype, bits, tails):
         _check_qmm(oracle, gpu, x, None, 32, bits, rows=_spread_rows(1024), quantized=q)
 
 
+@pytest.mark.parametrize("bits", (2, 3, 5, 6))
+@pytest.mark.parametrize("dtype", (torch.float32, torch.bfloat16))
+@pytest.mark.parametrize("tails", ("normal", "student_t"))
+def test_odd_width_stress_matmul_weight_as_k_by_n(oracle, gpu, dtype, bits, tails):
+    """The other reading of the [4096, 11008] stress weight: x of width 4096
+    only fits it with transpose=False, i.e. W is [K = 4096, N = 11008] with
+    the groups of 32 along n (`_qmm`, cpu/quantized.cpp:96-152).  Full size,
+    x [1, 4096] and [1024, 4096], every row against the fp64 product, spread
+    rows against the scalar oracle."""
+    make = normal_weights if tails == "normal" else student_t_weights
+    K, N = 4096, 11008
+    w = make((K, N), dtype, seed=bits)
+    q = oracle.quantize(w, 32, bits)
+    assert q[0].shape == (K, N * bits // 32) and q[1].shape == (K, N // 32)
+    _check_qmm(oracle, gpu, activations((1, K), dtype), None, 32, bits, transpose=False,
+               quantized=q)
+    x = activations((1024, K), dtype)
+    _check_qmm(oracle, gpu, x, None, 32, bits, transpose=False, rows=_spread_rows(1024),
+               quantized=q)
+
+
 def test_qmm_batched_shapes(oracle, gpu):
     # python/tests/test_quantized.py:540-563
     gs, bits = 64, 4

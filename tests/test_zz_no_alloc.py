@@ -48,6 +48,46 @@ CASES = (
 )
 
 
+def _memory_state(lib):
+    """(bytes the library's allocator holds, its peak, its cache, free device
+    memory as the driver reports it)."""
+    free, total = torch.cuda.mem_get_info()
+    return (lib.mlxrocm_get_active_memory(), lib.mlxrocm_get_peak_memory(),
+            lib.mlxrocm_get_cache_memory(), free)
+
+
+def test_static_entry_point_allocates_nothing(gpu):
+    """The property in the entry point's name: around calls of every kind of
+    shape that uses scratch, the library's allocator counters (active, peak,
+    cache) and the driver's free-memory figure do not move.  The array's
+    address is resolved by an empty call first, as documented."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.mlxrocm_qmm_static(None, None, None, None, None, 0, 32, 128, 1, 0, 0, 0,
+                                  64, 4, 2, 1, stream) == 0
+    prepared = []
+    for dtype, bits, gs, transpose, first, second in CASES:
+        for M, N, K in (first, second):
+            w = normal_weights((N, K) if transpose else (K, N), dtype, seed=M + N).to(gpu)
+            wq, s, b = mlx_amd.quantize(w, gs, bits)
+            x = activations((M, K), dtype, seed=K).to(gpu)
+            out = torch.empty((M, N), dtype=dtype, device=gpu)
+            prepared.append((x, wq, s, b, out, (M, N, K, 1, M * K, 0, 0, gs, bits, CODE[dtype],
+                                                int(transpose))))
+            del w
+    def run_all():
+        for x, wq, s, b, out, args in prepared:
+            _lib.check(lib.mlxrocm_qmm_static(x.data_ptr(), wq.data_ptr(), s.data_ptr(),
+                                              b.data_ptr(), out.data_ptr(), *args, stream))
+        torch.cuda.synchronize()
+
+    run_all()  # the runtime loads each kernel's code on its first launch
+    before = _memory_state(lib)
+    run_all()
+    after = _memory_state(lib)
+    assert after == before, (before, after)
+
+
 @pytest.mark.parametrize("dtype,bits,gs,transpose,first,second", CASES)
 def test_static_scratch_matches_workspace_call(gpu, dtype, bits, gs, transpose, first, second):
     lib = _lib.load()
