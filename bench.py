@@ -262,7 +262,17 @@ def sweep(torch, mlx_amd, dev) -> list:
         launcher = Launcher(torch, step, len(ring), small)
         launcher.run(len(ring))
         torch.cuda.synchronize()
-        ms = hip_event_ms(lib, launcher, max(len(ring) * (20 if small else 1), 10))
+        if small:
+            ms = hip_event_ms(lib, launcher, max(len(ring) * 20, 10))
+        else:
+            # launches of 40 us to 1 ms: warm up until the clocks have settled, then
+            # the median of five regions of at least 5 ms each (a single region of
+            # ten cold launches read 15-20 % slow at 8192 rows)
+            launcher.run(10)
+            torch.cuda.synchronize()
+            first = hip_event_ms(lib, launcher, 10)
+            per_region = max(10, int(5.0 / max(first, 1e-3)))
+            ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
         wshape = f"[{n},{k}]" if transpose else f"[{k},{n}] transpose=False"
         name = f"x {str(dtype)[6:]} [{M},{k}] W {wshape} b{bits} g{gs}"
         if small:

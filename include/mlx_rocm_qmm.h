@@ -106,6 +106,121 @@ int mlxrocm_affine_dequantize(
     mlxrocm_stream_t stream);
 
 /*
+ * The floating-point quantization modes (mlx/primitives.h QuantizationMode,
+ * mlx/ops.cpp:4675-4707 for the group size and bits each mode fixes):
+ *   mxfp4: e2m1 codes, groups of 32, one e8m0 scale byte per group
+ *   mxfp8: e4m3 codes, groups of 32, one e8m0 scale byte per group
+ *   nvfp4: e2m1 codes, groups of 16, one e4m3 scale byte per group
+ * No biases.  Codes are packed little-end first into uint32 words exactly as
+ * the affine codes are (eight 4-bit or four 8-bit codes per word).
+ */
+typedef enum {
+  MLXROCM_MXFP4 = 0,
+  MLXROCM_MXFP8 = 1,
+  MLXROCM_NVFP4 = 2
+} mlxrocm_fp_mode;
+
+/*
+ * Replaces fp_quantize (mlx/ops.cpp:5101-5205, the CPU op graph it builds when
+ * the stream is not on a GPU) and the GPU primitive behind it
+ * (mlx/backend/cuda/quantized/fp_quantize.cu).  w: n_elems elements of dtype,
+ * n_elems a multiple of the mode's group size; wq: n_elems * bits / 32 words;
+ * scales: n_elems / group_size bytes.  Scale of a group: mxfp*: e8m0 of
+ * round(log2(amax / max_code_value)) evaluated in double; nvfp4: e4m3 of
+ * amax / 6.  Elements are divided by the decoded scale in dtype and rounded to
+ * the nearest code (e2m1: first nearest of the value table, as argmin does;
+ * e4m3: round to nearest even with saturation at 448).
+ */
+int mlxrocm_fp_quantize(
+    const void* w,
+    uint32_t* wq,
+    uint8_t* scales,
+    size_t n_elems,
+    int mode,
+    int dtype,
+    mlxrocm_stream_t stream);
+
+/* Replaces fp_dequantize (mlx/ops.cpp:5342-5440; CPU kernel
+ * mlx/backend/cpu/quantized.cpp:49-62 dequantize_scale, :1322-1356):
+ * out[i] = dtype(value(code i) * scale(group of i)). */
+int mlxrocm_fp_dequantize(
+    const uint32_t* wq,
+    const uint8_t* scales,
+    void* out,
+    size_t n_elems,
+    int mode,
+    int dtype,
+    mlxrocm_stream_t stream);
+
+/* Quantize and dequantize in one pass without materialising the codes: what
+ * qqmm applies to its activation operand (mlx/ops.cpp:4926-4990; CPU:
+ * fp_quantize_dequantize, mlx/backend/cpu/quantized.cpp:1049-1128, called from
+ * QQMatmul::eval_cpu :1322-1356).  It follows that function's fp32 rules -- the
+ * scale from float log2 rounded half away from zero, e2m1 codes by its
+ * threshold table (ties to the even code) -- which are not the rules of
+ * mlxrocm_fp_quantize on ties, as in the reference. */
+int mlxrocm_fp_quantize_dequantize(
+    const void* x,
+    void* out,
+    size_t n_elems,
+    int mode,
+    int dtype,
+    mlxrocm_stream_t stream);
+
+/*
+ * quantized_matmul for the floating-point modes (mlx/ops.cpp:4784-4834 with
+ * mode != "affine"; CPU kernels mlx/backend/cpu/quantized.cpp:449-698
+ * fp_qmm / fp_qmm_t and their dispatch).  Shapes as mlxrocm_qmm: x [L, M, K],
+ * transpose: w [L, N, K bits / 32], scales [L, N, K / group_size] bytes;
+ * otherwise w [L, K, N bits / 32], scales [L, K, N / group_size]; out
+ * [L, M, N].  Batch strides in elements (x), words (w) and bytes (scales); a
+ * stride of 0 broadcasts.  Products and sums are evaluated in fp32 and rounded
+ * once to dtype.
+ */
+int mlxrocm_fp_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t scales_batch_stride,
+    int mode,
+    int dtype,
+    int transpose,
+    mlxrocm_stream_t stream);
+
+/* gather_qmm for the floating-point modes (mlx/ops.cpp:5553-5629 with
+ * mode != "affine"; CPU: mlx/backend/cpu/quantized.cpp:806-900 fp_bs_qmm_dispatch_mode).
+ * Arguments as mlxrocm_gather_qmm without biases; pair i multiplies
+ * x[lhs_indices[i]] by w[rhs_indices[i]]; a pair with an index out of range
+ * writes zeros. */
+int mlxrocm_fp_gather_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const uint32_t* lhs_indices,
+    const uint32_t* rhs_indices,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int64_t x_batch_stride,
+    int64_t w_expert_stride,
+    int64_t scales_expert_stride,
+    int mode,
+    int dtype,
+    int transpose,
+    mlxrocm_stream_t stream);
+
+/*
  * GGML tensor types the GGUF loader keeps quantized (ids as in the GGUF file
  * format; every other quantized type is dequantized to fp16 by MLX's loader,
  * mlx/io/gguf.cpp, and is not handled here).
@@ -204,8 +319,9 @@ int mlxrocm_qmm(
 
 /*
  * Prefill calls (16-bit types, transpose != 0, M >= 512) first transpose scales
- * and biases to [K / group_size][N] so that consecutive rows of W read
- * consecutive values (a few MB, about 5 us per call).  Weights do not change
+ * and biases to [K / group_size][N] (scale, bias) pairs so that consecutive rows
+ * of W read consecutive values, both with one load (a few MB, about 5 us per
+ * call).  Weights do not change
  * between calls: a caller that keeps that image beside a weight skips the
  * pre-pass.  The reference has no such cache -- its GPU backends read scales in
  * the caller's layout (mlx/backend/cuda/quantized/qmm/qmm.cu:143-146,

@@ -17,6 +17,7 @@ HIP_ERROR = -3
 OUT_OF_MEMORY = -4
 
 FLOAT32, FLOAT16, BFLOAT16 = 0, 1, 2
+MXFP4, MXFP8, NVFP4 = 0, 1, 2  # mlxrocm_fp_mode
 
 _i = ctypes.c_int
 _i64 = ctypes.c_int64
@@ -52,6 +53,11 @@ SIGNATURES = {
         [_p] * 7 + [_i] * 6 + [_i64] * 3 + [_i] * 5 + [_p, _sz, _p],
     ),
     "mlxrocm_gather_qmm_workspace_size": (_sz, [_i] * 10),
+    "mlxrocm_fp_quantize": (_i, [_p, _p, _p, _sz, _i, _i, _p]),
+    "mlxrocm_fp_dequantize": (_i, [_p, _p, _p, _sz, _i, _i, _p]),
+    "mlxrocm_fp_quantize_dequantize": (_i, [_p, _p, _sz, _i, _i, _p]),
+    "mlxrocm_fp_qmm": (_i, [_p] * 4 + [_i] * 4 + [_i64] * 3 + [_i] * 3 + [_p]),
+    "mlxrocm_fp_gather_qmm": (_i, [_p] * 6 + [_i] * 6 + [_i64] * 3 + [_i] * 3 + [_p]),
     "mlxrocm_qmm_kernel_name": (ctypes.c_char_p, [_i] * 8),
     "mlxrocm_qmm_plan": (_i, [_i] * 9 + [_sz, ctypes.c_char_p, _sz]),
     "mlxrocm_gather_qmm_plan": (_i, [_i] * 10 + [_sz, ctypes.c_char_p, _sz]),

@@ -302,25 +302,25 @@ int run_qmm_t_transposed_sb(
   const void* sb = sc.sb_image;
   if (!prepacked) {
     // rows of the source are the N rows of W, columns its G groups
-    rc = transpose_sb_for_qmm_n(
-        a.scales, a.biases, region, a.N, G, batches, a.sb_batch_stride, dtype, s);
+    rc = interleave_sb_for_qmm_t(
+        a.scales, a.biases, region, a.N, G, batches, a.sb_batch_stride, s);
     if (rc != MLXROCM_OK) {
       return rc;
     }
     sb = region;
   }
-  const size_t image = static_cast<size_t>(a.N) * G;
+  const size_t image = static_cast<size_t>(a.N) * G; // pairs of one weight matrix
   QmmArgs part = a;
   part.scales = sb;
-  part.biases = static_cast<const char*>(sb) + image * dtype_size(dtype);
+  part.biases = sb; // (unused: a pair holds both)
   part.sb_batch_stride = batches == 1 ? 0 : static_cast<int64_t>(2 * image);
-  part.sb_transposed = 1;
+  part.sb_transposed = 2;
   if (k_splits <= 1) {
-    return launch_qmm_mfma(part, gs, bits, dtype, s);
+    return launch_qmm_mfma_pairs(part, gs, bits, dtype, s);
   }
   void* partial = static_cast<char*>(region) + sb_bytes;
   part.out = partial;
-  rc = launch_qmm_mfma_ksplit(part, gs, bits, dtype, k_splits, s);
+  rc = launch_qmm_mfma_ksplit_pairs(part, gs, bits, dtype, k_splits, s);
   if (rc != MLXROCM_OK) {
     return rc;
   }
@@ -1171,6 +1171,12 @@ extern "C" int mlxrocm_qmm_sb_image(
   }
   if (!scales || !biases || !image) {
     return fail(MLXROCM_INVALID_ARGUMENT, "[qmm_sb_image] null device pointer");
+  }
+  if (dtype != MLXROCM_FLOAT32) {
+    // what the 16-bit prefill path reads: (scale, bias) pairs, [K / group][N]
+    return interleave_sb_for_qmm_t(
+        scales, biases, image, N, K / group_size, batches, sb_batch_stride,
+        static_cast<hipStream_t>(stream));
   }
   return transpose_sb_for_qmm_n(
       scales, biases, image, N, K / group_size, batches, sb_batch_stride, dtype,

@@ -35,9 +35,12 @@ struct QmmArgs {
   const int32_t* group_ntiles;
   int group_tile_rows;
   // Prefill tile kernel only: scales / biases point at a transposed image
-  // [K / group][N] (made by transpose_sb_for_qmm_n with the roles of K and N
-  // swapped), so that the lanes of a wavefront, which own consecutive rows of
-  // W, read consecutive values.  0: the caller's [N][K / group] arrays.
+  // [K / group][N], so that the lanes of a wavefront, which own consecutive rows
+  // of W, read consecutive values.  0: the caller's [N][K / group] arrays.
+  // 1: two images, scales and biases (transpose_sb_for_qmm_n with the roles of K
+  // and N swapped; float32 operands).  2: one image of (scale, bias) pairs, a.scales
+  // pointing at it (interleave_sb_for_qmm_t; 16-bit types): one load per thread
+  // and K-step fetches both.
   int sb_transposed;
   // Two weight matrices sharing one x (the gate and up projections of a gated
   // MLP): with L == 2 and these set, problem 1 reads them instead of w / scales /
@@ -106,6 +109,12 @@ bool qmv_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype);
 int launch_qmv_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 bool qmm_mfma_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmm_mfma(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+// The same reading the (scale, bias) pair image (a.sb_transposed == 2, a.scales
+// pointing at it; interleave_sb_for_qmm_t), whole K and split K.
+int launch_qmm_mfma_pairs(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
+int launch_qmm_mfma_ksplit_pairs(
+    const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
+
 bool qmv_wide_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmv_wide(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 bool qmm_skinny_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
@@ -159,6 +168,18 @@ int qmm_mfma_k_splits(int M, int N, int K, int L);
 // `a.scales` / `a.biases` must point at [group][k] images (transpose_sb_for_qmm_n).
 int launch_qmm_mfma_n(const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
 size_t qmm_n_sb_bytes(int K, int G, int batches, int dtype);
+// scales / biases [N][G] (16-bit types) -> per batch entry [G][N] pairs
+// (scale in the low half of a dword, bias in the high half); same size as the
+// two separate images.
+int interleave_sb_for_qmm_t(
+    const void* scales,
+    const void* biases,
+    void* out,
+    int N,
+    int G,
+    int batches,
+    int64_t src_stride,
+    hipStream_t s);
 int transpose_sb_for_qmm_n(
     const void* scales,
     const void* biases,

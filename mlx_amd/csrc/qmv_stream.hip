@@ -179,7 +179,12 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 // no lane ever falls outside a row and the loads carry no predicate.
 template <typename T, int BITS, int GS, int M, int RW, int KW, bool FULL, int RM = 1, bool MD = false,
           bool GLU = false>
-__global__ __launch_bounds__(RW * KW * 64) void qmv_stream_kernel(const QmmArgs a) {
+// (At least two waves per SIMD: the kernel needs under 80 registers, and with a
+// budget of 256 the compiler keeps the 4x4x4 results in vector registers; with
+// the 512 that a workgroup of 256 threads may claim it puts them in accumulation
+// registers and reads each one back with v_accvgpr_read.)
+__global__ __launch_bounds__(RW * KW * 64) __attribute__((amdgpu_waves_per_eu(2))) void
+qmv_stream_kernel(const QmmArgs a) {
   using S = StreamShape<BITS, GS>;
   constexpr int CPW = S::kChunksPerWave;
   constexpr int kRowsPerWave = S::kRowsPerWave * RM;
@@ -580,10 +585,14 @@ StreamPlan stream_plan(int K, int N, int M) {
     }
     pl.rm = rm;
   }
-  // One k-wave, one row of x, 4-bit: workgroups of four waves when that lowers
-  // the number of rows the busiest compute unit ends up with (14336 rows on 256
-  // units: 7 x 8 rows instead of 4 x 16); measured 3-6 % faster when it does
-  // and slower when it does not, and slower for 8-bit codes either way.
+  // One k-wave, one row of x, 4-bit: workgroups of seven or four waves when that
+  // does not raise the number of rows the busiest compute unit ends up with
+  // (14336 rows on 256 units: 4 x 14 or 7 x 8 rows instead of 4 x 16).  Seven
+  // waves put exactly seven on every SIMD with a quarter fewer workgroups staging
+  // x than four do: 14336 x 4096, 8.04 us with eight or four waves, 7.84 with seven;
+  // where the shape does not balance the smaller workgroup is slower (measured for
+  // four waves: 3-6 % faster when it lowers the busiest unit's rows, slower when
+  // not), and 8-bit codes are slower either way.
   if (pl.kw == 1 && M == 1 && BITS == 4) {
     const long cus = compute_units();
     auto busiest = [&](int rw) {
@@ -591,7 +600,9 @@ StreamPlan stream_plan(int K, int N, int M) {
       const long wgs = (N + rows - 1) / rows;
       return (wgs + cus - 1) / cus * rows;
     };
-    if (busiest(4) < busiest(8)) {
+    if (busiest(7) <= busiest(4) && busiest(7) < busiest(8)) {
+      pl.rw = 7;
+    } else if (busiest(4) < busiest(8)) {
       pl.rw = 4;
     }
   }
@@ -692,7 +703,10 @@ int launch_qmv_stream_glu(const QmmArgs& a, int gs, int bits, int dtype, hipStre
     if constexpr (RM == 0) {
       return fail(MLXROCM_UNSUPPORTED, "[qmv] shape not covered by the gated GEMV");
     } else {
-      const StreamPlan pl = stream_plan<B, G>(a.K, 2 * a.N, 1);
+      StreamPlan pl = stream_plan<B, G>(a.K, 2 * a.N, 1);
+      if (pl.rw == 7) {
+        pl.rw = 8; // the gated form has four- and eight-wave workgroups
+      }
       const size_t smem = stream_smem_bytes<B, G>(1, a.K, pl.rw, pl.kw, RM);
       const bool full = a.K == pl.kw * S::kChunksPerWave * S::kChunkCodes;
       const dim3 grid((a.N + pl.rw - 1) / pl.rw, 1);
@@ -791,6 +805,11 @@ int launch_qmv_stream(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t
         case 1:
           if (pl.rw == 4) {
             return by_rm(mval, IntC<4>{}, IntC<1>{});
+          }
+          if constexpr (B == 4 && decltype(mval)::value == 1) {
+            if (pl.rw == 7) {
+              return by_rm(mval, IntC<7>{}, IntC<1>{});
+            }
           }
           return by_rm(mval, IntC<8>{}, IntC<1>{});
         case 2:

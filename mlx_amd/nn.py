@@ -6,7 +6,9 @@ operators.
 The host module system is ``torch.nn`` (torch is the device-memory plumbing of
 this package): a quantized layer keeps ``weight`` (uint32 codes), ``scales`` and
 ``biases`` as buffers -- frozen, as in MLX -- and an optional trainable-free
-``bias``.  Only ``mode="affine"`` exists here.
+``bias``.  In the floating-point modes (``mxfp4``, ``mxfp8``, ``nvfp4``) there
+are no ``biases`` and ``scales`` are bytes; ``QQLinear`` (:310-432) quantizes its
+input as well.
 """
 from __future__ import annotations
 
@@ -17,17 +19,19 @@ import torch
 
 from . import ops
 
-__all__ = ["QuantizedLinear", "QuantizedEmbedding", "QuantizedSwitchLinear", "SwitchGLU",
+__all__ = ["QuantizedLinear", "QQLinear", "QuantizedEmbedding", "QuantizedSwitchLinear", "SwitchGLU",
            "quantize", "save_weights", "load_weights"]
 
 
 def _defaults_for_mode(mode: str, group_size: Optional[int], bits: Optional[int]):
     # python/mlx/nn/layers/quantized.py:12-24
-    if mode != "affine":
+    mode_defaults = {"affine": (64, 4), "mxfp4": (32, 4), "nvfp4": (16, 4), "mxfp8": (32, 8)}
+    if mode not in mode_defaults:
         raise ValueError(
-            f"[quantize] quantization mode '{mode}' is not available; only 'affine' is"
+            f"Invalid quantization mode '{mode}'. Valid modes are: {', '.join(mode_defaults)}."
         )
-    return (64 if group_size is None else group_size, 4 if bits is None else bits)
+    default_group_size, default_bits = mode_defaults[mode]
+    return group_size or default_group_size, bits or default_bits
 
 
 class QuantizedLinear(torch.nn.Module):
@@ -47,7 +51,8 @@ class QuantizedLinear(torch.nn.Module):
             "bias", torch.zeros((output_dims,), device=device, dtype=dtype) if bias else None)
 
     def _set_quantized(self, weight: torch.Tensor) -> None:
-        wq, scales, biases = ops.quantize(weight, self.group_size, self.bits, self.mode)
+        wq, scales, *biases = ops.quantize(weight, self.group_size, self.bits, self.mode)
+        biases = biases[0] if biases else None  # none in the floating-point modes
         for name, t in (("weight", wq), ("scales", scales), ("biases", biases)):
             if name in self._buffers:
                 self._buffers[name] = t
@@ -64,6 +69,8 @@ class QuantizedLinear(torch.nn.Module):
         """Keeps the transposed image of scales and biases that prefill calls
         (512 rows of x and more) would otherwise rebuild on every call.  Not in
         the reference; call again after changing the weights."""
+        if self.mode != "affine":
+            return self  # no biases, nothing to transpose
         self._sb_image = ops.quantized_matmul_sb_image(self.scales, self.biases, self.group_size)
         self._sb_image_of = (self.scales.data_ptr(), self.biases.data_ptr())
         return self
@@ -71,7 +78,8 @@ class QuantizedLinear(torch.nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         image = getattr(self, "_sb_image", None)
         if image is not None and (
-                self._sb_image_of != (self.scales.data_ptr(), self.biases.data_ptr())
+                self.biases is None
+                or self._sb_image_of != (self.scales.data_ptr(), self.biases.data_ptr())
                 or torch.promote_types(x.dtype, self.scales.dtype) != image.dtype):
             image = None  # weights replaced, or a product in another type
         y = ops.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
@@ -91,6 +99,73 @@ class QuantizedLinear(torch.nn.Module):
         ql._set_quantized(w)
         if getattr(linear_layer, "bias", None) is not None:
             ql._buffers["bias"] = linear_layer.bias.detach()
+        return ql
+
+
+class QQLinear(torch.nn.Module):
+    """``y = qqmm(x, weight, scales)``: the input is quantized on the fly as well
+    (python/mlx/nn/layers/quantized.py:310-432).  In eval mode the weight is kept
+    quantized with its scales; in training mode it is kept in its floating-point
+    type and quantized inside every call.  Modes ``nvfp4`` (default) and
+    ``mxfp8``; no bias term."""
+
+    def __init__(self, input_dims: int, output_dims: int, group_size: Optional[int] = None,
+                 bits: Optional[int] = None, mode: str = "nvfp4", device=None,
+                 dtype=torch.float32):
+        super().__init__()
+        self.group_size, self.bits = _defaults_for_mode(mode, group_size, bits)
+        self.mode = mode
+        device = torch.device("cuda:0") if device is None else torch.device(device)
+        scale = math.sqrt(1.0 / input_dims)
+        weight = (torch.rand((output_dims, input_dims), device=device) * 2 - 1) * scale
+        self.register_buffer("weight", weight.to(dtype))
+        self.register_buffer("scales", None)
+        self._quantized = False
+
+    def extra_repr(self) -> str:
+        out_dims, in_dims = self.weight.shape
+        if self.weight.dtype == torch.uint32:
+            in_dims = (in_dims * 32) // self.bits
+        return (f"input_dims={in_dims}, output_dims={out_dims}, "
+                f"group_size={self.group_size}, bits={self.bits}, mode={self.mode}")
+
+    def quantize(self) -> None:
+        if not self._quantized:
+            self._float_dtype = self.weight.dtype
+            wq, scales = ops.quantize(self.weight, self.group_size, self.bits, self.mode)
+            self._buffers["weight"], self._buffers["scales"] = wq, scales
+            self._quantized = True
+
+    def dequantize(self) -> None:
+        if self._quantized:
+            self._buffers["weight"] = ops.dequantize(
+                self.weight, self.scales, group_size=self.group_size, bits=self.bits,
+                mode=self.mode, dtype=getattr(self, "_float_dtype", None))
+            self._buffers["scales"] = None
+            self._quantized = False
+
+    def train(self, mode: bool = True):
+        super().train(mode)
+        if mode:
+            self.dequantize()
+        else:
+            self.quantize()
+        return self
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.qqmm(x, self.weight, self.scales, group_size=self.group_size,
+                        bits=self.bits, mode=self.mode)
+
+    @classmethod
+    def from_linear(cls, linear_layer, group_size: Optional[int] = None,
+                    bits: Optional[int] = None, mode: str = "nvfp4") -> "QQLinear":
+        output_dims, input_dims = linear_layer.weight.shape
+        if getattr(linear_layer, "bias", None) is not None:
+            raise NotImplementedError("QQLinear does not support bias yet.")
+        w = linear_layer.weight.detach()
+        ql = cls(input_dims, output_dims, group_size, bits, mode, device=w.device, dtype=w.dtype)
+        ql._buffers["weight"] = w
+        ql.train(linear_layer.training)
         return ql
 
 
@@ -114,7 +189,7 @@ class QuantizedEmbedding(torch.nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         # torch cannot index uint32 tensors: gather the rows through an int32 view
         rows = self.weight.view(torch.int32)[x].view(torch.uint32)
-        return ops.dequantize(rows, self.scales[x], self.biases[x],
+        return ops.dequantize(rows, self.scales[x], None if self.biases is None else self.biases[x],
                               group_size=self.group_size, bits=self.bits, mode=self.mode)
 
     def as_linear(self, x: torch.Tensor) -> torch.Tensor:
@@ -249,7 +324,17 @@ class SwitchGLU(torch.nn.Module):
 
 def _to_quantized(m, **kwargs):
     if isinstance(m, torch.nn.Linear):
+        # Linear.to_quantized, python/mlx/nn/layers/linear.py:72-107
+        if kwargs.pop("quantize_input", False):
+            mode = kwargs.get("mode", "affine")
+            if mode not in ("nvfp4", "mxfp8"):
+                raise ValueError(
+                    "Quantized activations are only supported for 'nvfp4' and 'mxfp8' "
+                    f"modes, got {mode}."
+                )
+            return QQLinear.from_linear(m, **kwargs)
         return QuantizedLinear.from_linear(m, **kwargs)
+    kwargs.pop("quantize_input", None)
     if isinstance(m, torch.nn.Embedding):
         return QuantizedEmbedding.from_embedding(m, **kwargs)
     return None
@@ -263,8 +348,6 @@ def quantize(model: torch.nn.Module, group_size: Optional[int] = None,
     the predicate accepts by their quantized counterparts (``nn.quantize``).
     ``class_predicate(path, module)`` returns a bool or a dict of parameters for
     the conversion."""
-    if quantize_input:
-        raise ValueError("[quantize] quantize_input needs an fp quantization mode")
     _defaults_for_mode(mode, group_size, bits)
     quantizable = lambda m: isinstance(m, (torch.nn.Linear, torch.nn.Embedding))  # noqa: E731
     class_predicate = class_predicate or (lambda _, m: quantizable(m))
@@ -280,6 +363,8 @@ def quantize(model: torch.nn.Module, group_size: Optional[int] = None,
                 raise ValueError(f"Unable to quantize model of type {type(child)}")
             if isinstance(decision, bool):
                 kwargs = {"group_size": group_size, "bits": bits, "mode": mode}
+                if quantize_input:
+                    kwargs["quantize_input"] = True
             elif isinstance(decision, dict):
                 kwargs = dict(decision)
             else:

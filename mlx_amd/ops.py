@@ -60,11 +60,42 @@ def _params_from_mode(mode: str, group_size, bits) -> Tuple[int, int]:
             db if bits is None else int(bits))
 
 
-def _affine_only(tag: str, mode: str) -> None:
-    if mode != "affine":
+_MODE_CODE = {"mxfp4": _lib.MXFP4, "mxfp8": _lib.MXFP8, "nvfp4": _lib.NVFP4}
+
+
+def _check_fp_params(tag: str, mode: str, group_size: int, bits: int) -> None:
+    # fp_quantize / fp_dequantize, mlx/ops.cpp:5108-5123, 5351-5366
+    want_gs = 16 if mode == "nvfp4" else 32
+    want_bits = 8 if mode == "mxfp8" else 4
+    if group_size != want_gs:
+        raise ValueError(
+            f"[{tag}] {mode} quantization requires group size {want_gs} but got {group_size}."
+        )
+    if bits != want_bits:
+        raise ValueError(
+            f"[{tag}] {mode} quantization requires bits to be {want_bits} but got {bits}."
+        )
+
+
+def _no_global_scale(tag: str, mode: str, *global_scales) -> None:
+    # validate_global_scale, mlx/ops.cpp:4756-4782
+    for g in global_scales:
+        if g is None:
+            continue
+        if mode != "nvfp4":
+            raise ValueError(
+                f"[{tag}] Global scale is only supported for 'nvfp4' quantization mode."
+            )
+        if g.numel() != 1:
+            raise ValueError(
+                f"[{tag}] Global scale must be a scalar but got shape {tuple(g.shape)}."
+            )
+        if g.dtype != torch.float32:
+            raise ValueError(
+                f"[{tag}] Global scale must have dtype float32 but got {g.dtype}."
+            )
         raise RuntimeError(
-            f"[{tag}] quantization mode '{mode}' has no ROCm implementation; "
-            "only 'affine' is supported."
+            f"[{tag}] nvfp4 with a global scale has no ROCm implementation."
         )
 
 
@@ -75,16 +106,25 @@ def _validate_mode_with_type(tag, scales, biases, out_type, mode):
         raise ValueError(
             f"[{tag}] Only real floating types are supported but output dtype == {out_type}."
         )
-    _affine_only(tag, mode)
-    if biases is None:
-        raise ValueError(f"[{tag}] Biases must be provided for affine quantization.")
-    dtype = torch.promote_types(scales.dtype, biases.dtype)
-    if dtype not in _FLOATING:
+    if mode == "affine":
+        if biases is None:
+            raise ValueError(f"[{tag}] Biases must be provided for affine quantization.")
+        dtype = torch.promote_types(scales.dtype, biases.dtype)
+        if dtype not in _FLOATING:
+            raise ValueError(
+                f"[{tag}] Only real floating types are supported but scales.dtype() == "
+                f"{scales.dtype} and biases.dtype() == {biases.dtype}."
+            )
+        return (out_type if out_type is not None else dtype), mode
+    if scales.dtype != torch.uint8:
         raise ValueError(
-            f"[{tag}] Only real floating types are supported but scales.dtype() == "
-            f"{scales.dtype} and biases.dtype() == {biases.dtype}."
+            f"[{tag}] Scale type must be uint8 but received type {scales.dtype}."
         )
-    return (out_type if out_type is not None else dtype), mode
+    if biases is not None:
+        raise ValueError(
+            f"[{tag}] Biases must be null for quantization mode '{mode}'."
+        )
+    return (out_type if out_type is not None else torch.bfloat16), mode
 
 
 def _validate_quantized_input(tag, w, scales, group_size, bits, biases):
@@ -157,9 +197,12 @@ def quantize(
     group_size: Optional[int] = None,
     bits: Optional[int] = None,
     mode: str = "affine",
+    global_scale: Optional[torch.Tensor] = None,
 ):
-    """``mx.quantize``: returns ``(w_q uint32, scales, biases)``
-    (mlx/ops.cpp:5208-5246 -> affine_quantize :5035-5099)."""
+    """``mx.quantize``: returns ``(w_q uint32, scales, biases)`` for
+    ``mode="affine"`` (mlx/ops.cpp:5208-5246 -> affine_quantize :5035-5099) and
+    ``(w_q uint32, scales uint8)`` for the floating-point modes (fp_quantize
+    :5101-5205)."""
     mode = _mode("quantize", mode)
     group_size, bits = _params_from_mode(mode, group_size, bits)
     if w.dtype not in _FLOATING:
@@ -177,14 +220,27 @@ def quantize(
             f"quantization group size {group_size}. However the provided  matrix has "
             f"shape {tuple(w.shape)}"
         )
-    _affine_only("quantize", mode)
-    _check_affine_params("quantize", group_size, bits)
+    _no_global_scale("quantize", mode, global_scale)
+    if mode == "affine":
+        _check_affine_params("quantize", group_size, bits)
+    else:
+        _check_fp_params("quantize", mode, group_size, bits)
     _require_gpu("quantize", w)
     lib = _lib.load()
     w = _contiguous(w)  # ensure_row_contiguous, cpu/quantized.cpp:1233
     lead = tuple(w.shape[:-1])
     K = w.shape[-1]
     wq = torch.empty(lead + (K * bits // 32,), dtype=torch.uint32, device=w.device)
+    if mode != "affine":
+        # fp_quantize, mlx/ops.cpp:5101-5205: two outputs, one scale byte per group
+        scales = torch.empty(lead + (K // group_size,), dtype=torch.uint8, device=w.device)
+        _lib.check(
+            lib.mlxrocm_fp_quantize(
+                w.data_ptr(), wq.data_ptr(), scales.data_ptr(), w.numel(),
+                _MODE_CODE[mode], _DTYPE_CODE[w.dtype], _stream_ptr(w),
+            )
+        )
+        return wq, scales
     scales = torch.empty(lead + (K // group_size,), dtype=w.dtype, device=w.device)
     biases = torch.empty_like(scales)
     _lib.check(
@@ -203,11 +259,16 @@ def dequantize(
     group_size: Optional[int] = None,
     bits: Optional[int] = None,
     mode: str = "affine",
+    global_scale: Optional[torch.Tensor] = None,
     dtype: Optional[torch.dtype] = None,
 ):
-    """``mx.dequantize`` (mlx/ops.cpp:5465-5517 -> affine_dequantize :5248-5340)."""
+    """``mx.dequantize`` (mlx/ops.cpp:5465-5517 -> affine_dequantize :5248-5340,
+    fp_dequantize :5342-5462)."""
     out_type, mode = _validate_mode_with_type("dequantize", scales, biases, dtype, mode)
     group_size, bits = _params_from_mode(mode, group_size, bits)
+    _no_global_scale("dequantize", mode, global_scale)
+    if mode != "affine":
+        return _fp_dequantize(w, scales, group_size, bits, mode, out_type)
     if bits <= 0:
         raise ValueError(f"[dequantize] Invalid value for bits: {bits}")
     if group_size <= 0:
@@ -253,6 +314,43 @@ def dequantize(
         )
     )
     return _astype(out, out_type)  # astype, :5502-5505
+
+
+def _fp_dequantize(w, scales, group_size, bits, mode, out_type):
+    # fp_dequantize, mlx/ops.cpp:5342-5462
+    if bits <= 0:
+        raise ValueError(f"[dequantize] Invalid value for bits: {bits}")
+    if group_size <= 0:
+        raise ValueError(f"[dequantize] Invalid value for group_size: {group_size}")
+    if w.dtype != torch.uint32:
+        raise ValueError("[dequantize] The matrix should be given as a uint32")
+    if w.dim() < 2:
+        raise ValueError(
+            "[dequantize] The matrix to be dequantized must have at least 2 dimension "
+            f"but it has only {w.dim()}."
+        )
+    _check_fp_params("dequantize", mode, group_size, bits)
+    if w.dim() != scales.dim() or tuple(w.shape[:-1]) != tuple(scales.shape[:-1]):
+        raise ValueError("[dequantize] Shape of scales does not match the matrix")
+    out_size = w.shape[-1] * 32 // bits
+    if out_size != scales.shape[-1] * group_size:
+        raise ValueError(
+            "[dequantize] Shape of scales does not match the matrix given the "
+            f"quantization parameters. Provided matrix of shape {tuple(w.shape)} and "
+            f"scales of shape {tuple(scales.shape)}."
+        )
+    _require_gpu("dequantize", w, scales)
+    lib = _lib.load()
+    w = _contiguous(w)
+    scales = _contiguous(scales)
+    out = torch.empty(tuple(w.shape[:-1]) + (out_size,), dtype=out_type, device=w.device)
+    _lib.check(
+        lib.mlxrocm_fp_dequantize(
+            w.data_ptr(), scales.data_ptr(), out.data_ptr(), out.numel(),
+            _MODE_CODE[mode], _DTYPE_CODE[out_type], _stream_ptr(w),
+        )
+    )
+    return out
 
 
 def _dense_batches(t: torch.Tensor, batch_shape: Tuple[int, ...]):
@@ -339,19 +437,27 @@ def quantized_matmul(
     _, w_outer = _extract_dims(
         "quantized_matmul", x, w, scales, biases, transpose, group_size, bits
     )
-    dtype = torch.promote_types(x.dtype, dtype)
+    affine = mode == "affine"
+    dtype = torch.promote_types(x.dtype, dtype) if affine else x.dtype  # :4803-4807
     if dtype not in _FLOATING:
         raise ValueError(
             "[quantized_matmul] Only real floating types are supported but "
             f"x.dtype() == {x.dtype}."
         )
-    _check_affine_params("quantized_matmul", group_size, bits)
-    _require_gpu("quantized_matmul", x, w, scales, biases)
+    if affine:
+        _check_affine_params("quantized_matmul", group_size, bits)
+        _require_gpu("quantized_matmul", x, w, scales, biases)
+    else:
+        _check_fp_params("quantized_matmul", mode, group_size, bits)
+        _require_gpu("quantized_matmul", x, w, scales)
+        if sb_image is not None:
+            raise ValueError("[quantized_matmul] sb_image belongs to mode='affine'")
     lib = _lib.load()
 
-    x = _astype(x, dtype)
-    scales = _astype(scales, dtype)
-    biases = _astype(biases, dtype)
+    if affine:
+        x = _astype(x, dtype)
+        scales = _astype(scales, dtype)
+        biases = _astype(biases, dtype)
     K = x.shape[-1]
     M = x.shape[-2] if x.dim() > 1 else 1
     x_batch = tuple(x.shape[:-2]) if x.dim() > 2 else ()
@@ -377,9 +483,18 @@ def quantized_matmul(
         M, L = M * L, 1
     wb, w_stride = _dense_batches(w, batch_shape)
     sb, sb_stride = _dense_batches(scales, batch_shape)
-    bb, _ = _dense_batches(biases, batch_shape)
     out = torch.empty(out_shape, dtype=dtype, device=x.device)
     code = _DTYPE_CODE[dtype]
+    if not affine:
+        _lib.check(
+            lib.mlxrocm_fp_qmm(
+                xb.data_ptr(), wb.data_ptr(), sb.data_ptr(), out.data_ptr(),
+                M, w_outer, K, L, M * K, w_stride, sb_stride, _MODE_CODE[mode], code,
+                int(bool(transpose)), _stream_ptr(x),
+            )
+        )
+        return out
+    bb, _ = _dense_batches(biases, batch_shape)
     ws_bytes = lib.mlxrocm_qmm_workspace_size(
         M, w_outer, K, L, int(w_stride != 0), group_size, bits, code, int(bool(transpose))
     )
@@ -526,7 +641,8 @@ def gather_qmm(
     _, w_outer = _extract_dims(
         "gather_qmm", x, w, scales, biases, transpose, group_size, bits
     )
-    out_type = torch.promote_types(x.dtype, out_type)
+    affine = mode == "affine"
+    out_type = torch.promote_types(x.dtype, out_type) if affine else x.dtype
     if out_type not in _FLOATING:
         raise ValueError(
             f"[gather_qmm] Only real floating types are supported but x.dtype() == {x.dtype}."
@@ -542,8 +658,12 @@ def gather_qmm(
                 f"shape {tuple(x.shape)}."
             )
         lhs_shape = _broadcast_shape(tuple(x.shape[:-2]), tuple(rhs.shape))
-    _check_affine_params("gather_qmm", group_size, bits)
-    _require_gpu("gather_qmm", x, w, scales, biases, rhs, *(() if lhs is None else (lhs,)))
+    if affine:
+        _check_affine_params("gather_qmm", group_size, bits)
+    else:
+        _check_fp_params("gather_qmm", mode, group_size, bits)
+    _require_gpu("gather_qmm", x, w, scales, rhs, *(() if biases is None else (biases,)),
+                 *(() if lhs is None else (lhs,)))
     lib = _lib.load()
     if lhs is None:
         if tuple(rhs.shape) != lhs_shape:
@@ -552,9 +672,10 @@ def gather_qmm(
         lhs, rhs = torch.broadcast_tensors(lhs, rhs)
     right_sorted = bool(sorted_indices) and lhs_indices is None
 
-    x = _astype(x, out_type)
-    scales = _astype(scales, out_type)
-    biases = _astype(biases, out_type)
+    if affine:
+        x = _astype(x, out_type)
+        scales = _astype(scales, out_type)
+        biases = _astype(biases, out_type)
     M, K = x.shape[-2], x.shape[-1]
     xb = _contiguous(x).reshape(-1, M, K)
     # Only the trailing matrices must be dense; a sliced expert stack keeps its
@@ -566,6 +687,24 @@ def gather_qmm(
         return t, t.shape[-1] * t.shape[-2]
     wb, w_stride = experts(w)
     sb, sb_stride = experts(scales)
+    if not affine:
+        n_idx = rhs.numel()
+        if lhs is None:
+            lhs_u = _default_lhs_uint32(tuple(x.shape[:-2]), tuple(rhs.shape), x.device)
+        else:
+            lhs_u = _as_uint32(lhs) if n_idx else lhs.reshape(-1)
+        rhs_u = _as_uint32(rhs) if n_idx else rhs.reshape(-1)
+        out = torch.empty(tuple(rhs.shape) + (M, w_outer), dtype=out_type, device=x.device)
+        _lib.check(
+            lib.mlxrocm_fp_gather_qmm(
+                xb.data_ptr(), wb.data_ptr(), sb.data_ptr(),
+                lhs_u.data_ptr() if n_idx else None, rhs_u.data_ptr() if n_idx else None,
+                out.data_ptr(), M, w_outer, K, n_idx, xb.shape[0], wb.shape[0],
+                M * K, w_stride, sb_stride, _MODE_CODE[mode], _DTYPE_CODE[out_type],
+                int(bool(transpose)), _stream_ptr(x),
+            )
+        )
+        return out
     bb, bb_stride = experts(biases)
     if bb_stride != sb_stride:
         bb = _contiguous(bb)
@@ -596,4 +735,87 @@ def gather_qmm(
             ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x),
         )
     )
+    return out
+
+
+def qqmm(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    scales: Optional[torch.Tensor] = None,
+    group_size: Optional[int] = None,
+    bits: Optional[int] = None,
+    mode: str = "nvfp4",
+    global_scale_x: Optional[torch.Tensor] = None,
+    global_scale_w: Optional[torch.Tensor] = None,
+):
+    """``mx.qqmm`` (mlx/ops.cpp:4926-4990): x is quantized and dequantized on
+    the fly, then multiplied by the transposed quantized w.  Like the CPU backend
+    (QQMatmul::eval_cpu, mlx/backend/cpu/quantized.cpp:1322-1360) this takes a
+    quantized w; unlike it, any number of rows of x.  A floating-point w, which
+    the CPU backend does not take either, is quantized first as the CUDA backend
+    does (mlx/backend/cuda/quantized/qqmm.cpp)."""
+    mode = _mode("qqmm", mode)
+    group_size, bits = _params_from_mode(mode, group_size, bits)
+    in_shape = tuple(x.shape)
+    if x.dim() == 1:
+        x = x.unsqueeze(0)
+    elif w.dim() == 2 and x.dim() > 2:
+        x = x.reshape(-1, x.shape[-1])
+    # validate_qqmm_inputs, mlx/ops.cpp:4836-4894
+    if x.dim() > 2 or w.dim() > 2:
+        raise ValueError(
+            f"[qqmm] Only 2D inputs are supported but x.ndim() == {x.dim()} and "
+            f"w.ndim() == {w.dim()}."
+        )
+    if w.dtype == torch.uint32:
+        if scales is None:
+            raise ValueError("[qqmm] Scales must be provided if second argument is quantized.")
+        _validate_quantized_input("qqmm", w, scales, group_size, bits, None)
+    elif w.dtype not in _FLOATING:
+        raise ValueError(
+            "[qqmm] Only real floating types except float64 are supported but "
+            f"second argument dtype == {w.dtype}."
+        )
+    if x.dtype not in _FLOATING:
+        raise ValueError(
+            "[qqmm] Only real floating types except float64 are supported but "
+            f"first argument dtype == {x.dtype}."
+        )
+    if mode == "affine":
+        raise ValueError("[qqmm] Affine quantization is not supported for qqmm.")
+    if mode == "nvfp4" and (global_scale_x is None) != (global_scale_w is None):
+        raise ValueError(
+            "[qqmm] For nvfp4 mode, either both global_scale_x and global_scale_w "
+            "must be provided, or neither."
+        )
+    _no_global_scale("qqmm", mode, global_scale_x, global_scale_w)
+    _check_fp_params("qqmm", mode, group_size, bits)
+    if w.dtype != torch.uint32:
+        # extract_qqmm_dims, :4896-4924
+        if x.shape[-1] != w.shape[-1]:
+            raise ValueError(
+                f"[qqmm] Last dimension of first input with shape {tuple(x.shape)} must "
+                f"match last dimension of second input with shape {tuple(w.shape)}."
+            )
+        w, scales = quantize(_astype(w, x.dtype), group_size, bits, mode)
+    else:
+        _extract_dims("qqmm", x, w, scales, None, True, group_size, bits)
+    if scales.dtype != torch.uint8:
+        raise ValueError(f"[qqmm] Scale type must be uint8 but received type {scales.dtype}.")
+    _require_gpu("qqmm", x, w, scales)
+    lib = _lib.load()
+    xc = _contiguous(x)
+    xhat = torch.empty_like(xc)
+    if xc.numel():
+        _lib.check(
+            lib.mlxrocm_fp_quantize_dequantize(
+                xc.data_ptr(), xhat.data_ptr(), xc.numel(), _MODE_CODE[mode],
+                _DTYPE_CODE[xc.dtype], _stream_ptr(xc),
+            )
+        )
+    out = quantized_matmul(xhat, w, scales, None, True, group_size, bits, mode)
+    if len(in_shape) > 2:
+        return out.reshape(in_shape[:-1] + (out.shape[-1],))
+    if len(in_shape) == 1:
+        return out.squeeze(0)
     return out

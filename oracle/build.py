@@ -3,7 +3,8 @@
   python oracle/build.py          # both targets (the second only if possible)
 
 * ``oracle/libaffine_qref.so``  -- this repository's C restatement
-  (``affine_qref.c``), always buildable with gcc.
+  (``affine_qref.c`` and, for the floating-point modes, ``fp_qref.c``), always
+  buildable with gcc.
 * ``oracle/_ref/libmlx_cpu_qref.so`` -- the reference's own
   ``mlx/backend/cpu/quantized.cpp`` compiled as a single translation unit from
   where it lies in the reference checkout (``ref_harness.cpp`` includes it).
@@ -40,7 +41,8 @@ def build_qref() -> str:
         [
             "gcc", "-std=c11", "-O3", "-fPIC", "-shared", "-ffp-contract=off",
             "-fno-fast-math", "-Wall", "-Wextra",
-            os.path.join(HERE, "affine_qref.c"), "-lm", "-o", QREF_SO,
+            os.path.join(HERE, "affine_qref.c"), os.path.join(HERE, "fp_qref.c"),
+            "-lm", "-o", QREF_SO,
         ]
     )
     return QREF_SO

@@ -11,6 +11,9 @@
 //   ref_quantize -> mlx::core::quantize<T,U>          cpu/quantized.cpp:1148
 //   ref_qmm      -> _qmm_dispatch_typed<T> (pointers) cpu/quantized.cpp:340
 //   ref_*16_*    -> _MLX_Float16 / _MLX_BFloat16      mlx/types/{fp16,bf16}.h
+//   ref_to_fp8 / ref_from_fp8 -> detail::ToFP8 / FromFP8  cpu/unary_ops.h:120-174
+//   ref_e8m0 / ref_e2m1 -> to_fp8_e8m0 / to_fp4_e2m1   cpu/quantized.cpp:1049-1091
+//   ref_fp_qmm   -> fp_qmm_dispatch_transpose<T, gs, bits> cpu/quantized.cpp:603
 #include "mlx/backend/cpu/quantized.cpp"
 
 #define REF_EXPORT extern "C" __attribute__((visibility("default")))
@@ -128,5 +131,62 @@ REF_EXPORT int ref_qmm(
     }
   } catch (const std::exception&) {
     return -1;
+  }
+}
+
+REF_EXPORT uint8_t ref_to_fp8(float x) {
+  return detail::ToFP8{}(x);
+}
+REF_EXPORT float ref_from_fp8(uint8_t x) {
+  return detail::FromFP8{}(x);
+}
+REF_EXPORT uint8_t ref_e8m0(float x) {
+  return to_fp8_e8m0(x);
+}
+REF_EXPORT uint8_t ref_e2m1(float x) {
+  return to_fp4_e2m1(x);
+}
+
+template <typename T>
+static void fp_qmm_any(
+    void* result, const void* x, const uint32_t* w, const uint8_t* scales, int M, int N, int K,
+    int mode, bool transposed_w) {
+  // the three instantiations of fp_qmm_dispatch_typed (cpu/quantized.cpp:648-662)
+  if (mode == 1) {
+    fp_qmm_dispatch_transpose<T, 32, 8>((T*)result, (const T*)x, w, scales, M, N, K, transposed_w);
+  } else if (mode == 0) {
+    fp_qmm_dispatch_transpose<T, 32, 4>((T*)result, (const T*)x, w, scales, M, N, K, transposed_w);
+  } else {
+    fp_qmm_dispatch_transpose<T, 16, 4>((T*)result, (const T*)x, w, scales, M, N, K, transposed_w);
+  }
+}
+
+// mode: 0 mxfp4, 1 mxfp8, 2 nvfp4
+REF_EXPORT int ref_fp_qmm(
+    void* result,
+    const void* x,
+    const uint32_t* w,
+    const uint8_t* scales,
+    int M,
+    int N,
+    int K,
+    int mode,
+    int transposed_w,
+    int dtype) {
+  if (mode < 0 || mode > 2) {
+    return -1;
+  }
+  switch (dtype) {
+    case 0:
+      fp_qmm_any<float>(result, x, w, scales, M, N, K, mode, transposed_w);
+      return 0;
+    case 1:
+      fp_qmm_any<float16_t>(result, x, w, scales, M, N, K, mode, transposed_w);
+      return 0;
+    case 2:
+      fp_qmm_any<bfloat16_t>(result, x, w, scales, M, N, K, mode, transposed_w);
+      return 0;
+    default:
+      return -1;
   }
 }

@@ -60,7 +60,7 @@ BASELINE = (
     # Cfg1: float32 4096 x 4096, 4-bit group 64, one row
     (dict(M=1, N=4096, K=4096, dtype=F32), ["qmv_f32"], "qmv_f32"),
     # Cfg2: decode, gate/up and down projection, B in {1, 4, 8}
-    (dict(M=1, N=14336, K=4096), ["qmv_stream"], "qmv_stream(rw=4,kw=1,rm=1)"),
+    (dict(M=1, N=14336, K=4096), ["qmv_stream"], "qmv_stream(rw=7,kw=1,rm=1)"),
     (dict(M=4, N=14336, K=4096), ["qmv_quad"], "qmv_quad(kw=4,sets=1)"),
     (dict(M=8, N=14336, K=4096), ["qmm_rows8"], "qmm_rows8(kw=4,slots=2)"),
     (dict(M=1, N=4096, K=14336), ["qmv_quad"], None),
@@ -73,10 +73,10 @@ BASELINE = (
     (dict(M=8, N=4096, K=14336, bits=8, group_size=128), ["qmv_wide"], None),
     # Cfg3: prefill
     (dict(M=2048, N=14336, K=4096), ["qmm_t_tile_sb_transposed"],
-     "transpose_sb+qmm_t_tile(nt=7)"),
+     "interleave_sb+qmm_t_tile(nt=7,pairs)"),
     (dict(M=8192, N=14336, K=4096, bits=8, group_size=128), ["qmm_t_tile_sb_transposed"],
-     "transpose_sb+qmm_t_tile(nt=7)"),
-    (dict(M=2048, N=4096, K=4096), ["qmm_t_tile_sb_transposed"], "transpose_sb+qmm_t_tile(nt=4)"),
+     "interleave_sb+qmm_t_tile(nt=7,pairs)"),
+    (dict(M=2048, N=4096, K=4096), ["qmm_t_tile_sb_transposed"], "interleave_sb+qmm_t_tile(nt=5,pairs)"),
     (dict(M=512, N=4096, K=14336), ["qmm_t_tile_sb_transposed"], None),
     # Cfg5: odd widths, group 32, both readings of the [4096, 11008] weight
     (dict(M=1, N=11008, K=4096, bits=3, group_size=32), ["qmv_f32"], "qmv_f32"),
@@ -103,7 +103,7 @@ def test_benchmark_shapes_take_the_documented_rule(shape, rules, launches):
 
 
 @pytest.mark.parametrize("tokens,expect", (
-    (1, "[qmv_stream]+qmv_stream(rw=4,kw=1,rm=1)"),
+    (1, "[qmv_stream]+qmv_stream(rw=7,kw=1,rm=1)"),
     (8, "qmm_slab_grouped(plans,tile=16,ranges=4)"),
     (64, "qmm_slab_grouped(plans,tile=32,ranges=4)"),
     (2048, "gather_group(fused)+qmm_t_tile_grouped"),

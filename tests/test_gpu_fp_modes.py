@@ -1,0 +1,318 @@
+"""GPU parity of the floating-point quantization modes (mxfp4 / mxfp8 / nvfp4)
+through the operators of mlx_amd (and so through the C ABI): quantize,
+dequantize and the on-the-fly quantize-dequantize bit for bit against the CPU
+oracle; quantized_matmul / gather_qmm / qqmm against the oracle (the
+reference's translation unit where it was built) within the stated tolerance
+and against an fp64 product of the exactly decoded weights.  Cases follow
+python/tests/test_quantized.py:41-181 (quantize / dequantize per mode),
+:183-237 (qqmm), :300-360 (fp_qmm shapes), :1180-1266 (gather)."""
+import os
+
+import pytest
+import torch
+
+import mlx_amd
+from oracle import build as obuild
+from oracle import fp_qref, qref
+
+pytestmark = pytest.mark.gpu
+
+MODES = ("mxfp4", "mxfp8", "nvfp4")
+DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+# fp32 accumulation on the GPU against an fp64 product: relative to the sum of
+# absolute products.  The final rounding to the element type adds half an ulp.
+ACC_TOL = {torch.float32: 2e-6, torch.float16: 1e-3, torch.bfloat16: 8e-3}
+# The CPU reference rounds every product and partial sum to the element type,
+# so it is the looser side: bound on |gpu - reference| relative to sum |x w|.
+REF_TOL = {torch.float32: 5e-6, torch.float16: 4e-3, torch.bfloat16: 3e-2}
+
+
+@pytest.fixture(scope="module")
+def fp_oracle():
+    if not os.path.isfile(qref.QREF_SO):
+        obuild.build_qref()
+    return fp_qref.FpOracle("reference" if qref.reference_built() else "port")
+
+
+def _weights(shape, dtype, seed, spread=True):
+    """Rows of very different magnitude, exact zeros, whole zero groups and
+    values that sit exactly between two codes after scaling."""
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(shape, generator=g)
+    if spread:
+        rows = w.reshape(-1, shape[-1])
+        rows *= torch.exp(torch.randn(rows.shape[0], 1, generator=g) * 2.0)
+        rows[0, :64] = 0.0
+        rows[1, ::3] = 0.0
+        if rows.shape[0] > 2:
+            # a group whose maximum is 6: the rest are multiples of 0.25
+            rows[2, :32] = torch.randint(-24, 25, (32,), generator=g).float() * 0.25
+            rows[2, 0] = 6.0
+    return w.to(dtype)
+
+
+def _equal_bits(a: torch.Tensor, b: torch.Tensor) -> bool:
+    view = {4: torch.int32, 2: torch.int16, 1: torch.uint8}[a.element_size()]
+    return torch.equal(a.contiguous().view(view), b.contiguous().view(view))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_quantize_matches_oracle_bit_for_bit(fp_oracle, gpu, mode, dtype):
+    for shape, seed in (((64, 512), 1), ((3, 17, 64), 2), ((2, 4096), 3)):
+        w = _weights(shape, dtype, seed)
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+        want_q, want_s = fp_oracle.quantize(w, mode)
+        assert wq.dtype == torch.uint32 and scales.dtype == torch.uint8
+        assert wq.shape == want_q.shape and scales.shape == want_s.shape
+        assert torch.equal(scales.cpu(), want_s), (mode, dtype, shape)
+        bad = (wq.cpu().view(torch.int32) != want_q.view(torch.int32)).sum().item()
+        assert bad == 0, (mode, dtype, shape, bad)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_dequantize_matches_oracle_bit_for_bit(fp_oracle, gpu, mode, dtype):
+    g = torch.Generator().manual_seed(11)
+    bits, gs = fp_qref.BITS[mode], fp_qref.GROUP_SIZE[mode]
+    K = 1024
+    wq = torch.randint(0, 2 ** 31, (32, K * bits // 32), generator=g, dtype=torch.int64)
+    wq = (wq * 2 + torch.randint(0, 2, wq.shape, generator=g)).to(torch.int32).view(torch.uint32)
+    if mode == "nvfp4":
+        # every e4m3 scale code (the reference's decoder has no NaN codes)
+        scales = torch.arange(32 * K // gs, dtype=torch.int64).reshape(32, -1) % 256
+    else:
+        # every e8m0 exponent but 255, which decodes to NaN
+        scales = torch.arange(32 * K // gs, dtype=torch.int64).reshape(32, -1) % 255
+    scales = scales.to(torch.uint8)
+    got = mlx_amd.dequantize(wq.to(gpu), scales.to(gpu), mode=mode, dtype=dtype)
+    want = fp_oracle.dequantize(wq, scales, mode, dtype)
+    assert got.dtype == dtype and got.shape == want.shape
+    if mode == "mxfp8":
+        # e4m3 codes 0x7f / 0xff decode to 480: finite, so still comparable
+        pass
+    assert _equal_bits(got.cpu(), want), (mode, dtype)
+    # default output type of the fp modes is bfloat16 (mlx/ops.cpp:4749-4753)
+    assert mlx_amd.dequantize(wq.to(gpu), scales.to(gpu), mode=mode).dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_values_on_the_code_grid_round_trip(gpu, mode):
+    """python/tests/test_quantized.py:41-181: values that are representable
+    (code value times a power-of-two scale) come back exactly."""
+    g = torch.Generator().manual_seed(5)
+    if mode == "mxfp8":
+        table = fp_qref._e4m3_values()[:127].float()  # positive codes below 448
+        table = table[table <= 448]
+    else:
+        table = torch.tensor(fp_qref.FP4_VALUES[:8])
+    top = table.max()
+    gs = fp_qref.GROUP_SIZE[mode]
+    idx = torch.randint(0, table.numel(), (16, 256), generator=g)
+    w = table[idx] * torch.where(torch.rand(16, 256, generator=g) < 0.5, -1.0, 1.0)
+    w.reshape(-1, gs)[:, 0] = top  # every group's maximum is the top code: scale 1
+    w = w * torch.exp2(torch.randint(-3, 4, (16, 1), generator=g).float())
+    for dtype in DTYPES:
+        wq, scales = mlx_amd.quantize(w.to(dtype).to(gpu), mode=mode)
+        back = mlx_amd.dequantize(wq, scales, mode=mode, dtype=dtype)
+        assert torch.equal(back.cpu().float(), w.to(dtype).float()), (mode, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_quantize_dequantize_matches_oracle_bit_for_bit(fp_oracle, gpu, mode, dtype):
+    from mlx_amd import _lib
+    from mlx_amd.ops import _DTYPE_CODE, _MODE_CODE
+
+    lib = _lib.load()
+    x = _weights((48, 512), dtype, 21)
+    xg = x.to(gpu)
+    out = torch.empty_like(xg)
+    _lib.check(lib.mlxrocm_fp_quantize_dequantize(
+        xg.data_ptr(), out.data_ptr(), xg.numel(), _MODE_CODE[mode], _DTYPE_CODE[dtype],
+        torch.cuda.current_stream().cuda_stream))
+    want = fp_oracle.quantize_dequantize(x, mode)
+    assert _equal_bits(out.cpu(), want), (mode, dtype)
+
+
+def _check_product(got, x, wq, scales, mode, transpose, ref, dtype):
+    """got [M, N] against fp64 of the exactly decoded weights and against the
+    CPU reference's own result."""
+    w = fp_qref.exact_fp_weights(wq, scales, mode)  # [N, K] or [K, N]
+    xd = x.double()
+    wd = w.T if transpose else w
+    exact = xd @ wd
+    mag = xd.abs() @ wd.abs() + 1e-30
+    err = ((got.double() - exact).abs() / mag).max().item()
+    half_ulp = {torch.float32: 2.0 ** -24, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    assert err <= ACC_TOL[dtype] + half_ulp, (mode, dtype, transpose, err)
+    if ref is not None:
+        rerr = ((got.double() - ref.double()).abs() / mag).max().item()
+        assert rerr <= REF_TOL[dtype], (mode, dtype, transpose, rerr)
+        # and the GPU result is the closer of the two to the exact product
+        ours = (got.double() - exact).abs().mean().item()
+        theirs = (ref.double() - exact).abs().mean().item()
+        assert ours <= theirs * 1.05 + 1e-12, (mode, dtype, ours, theirs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("transpose", (True, False))
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_quantized_matmul(fp_oracle, gpu, mode, transpose, dtype):
+    # python/tests/test_quantized.py:300-360: M in 8, 32, 33, 64 and gemv rows
+    for M, N, K, seed in ((1, 256, 512, 1), (8, 128, 256, 2), (33, 256, 128, 3), (64, 96, 2048, 4),
+                          (5, 64, 48 if mode == "nvfp4" else 96, 5)):
+        g = torch.Generator().manual_seed(seed)
+        w = torch.randn((N, K) if transpose else (K, N), generator=g).to(dtype)
+        x = torch.randn((M, K), generator=g).to(dtype)
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+        got = mlx_amd.quantized_matmul(x.to(gpu), wq, scales, transpose=transpose, mode=mode)
+        assert got.dtype == dtype and got.shape == (M, N)
+        ref = fp_oracle.qmm(x, wq.cpu(), scales.cpu(), mode, transpose)
+        _check_product(got.cpu(), x, wq.cpu(), scales.cpu(), mode, transpose, ref, dtype)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_quantized_matmul_full_size_decode(gpu, mode):
+    """The decode shape of the affine headline, x [1, 4096] @ W [14336, 4096]^T,
+    every output against fp64."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(7)
+    w = torch.randn((14336, 4096), generator=g).to(dtype)
+    for M in (1, 4, 6):
+        x = torch.randn((M, 4096), generator=g).to(dtype)
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+        got = mlx_amd.quantized_matmul(x.to(gpu), wq, scales, mode=mode)
+        _check_product(got.cpu(), x, wq.cpu(), scales.cpu(), mode, True, None, dtype)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_quantized_matmul_batched(fp_oracle, gpu, mode):
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(9)
+    w = torch.randn((3, 64, 128), generator=g).to(dtype)
+    x = torch.randn((2, 3, 5, 128), generator=g).to(dtype)
+    wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq, scales, mode=mode)
+    assert got.shape == (2, 3, 5, 64)
+    for b in range(2):
+        for e in range(3):
+            ref = fp_oracle.qmm(x[b, e], wq[e].cpu(), scales[e].cpu(), mode, True)
+            _check_product(got[b, e].cpu(), x[b, e], wq[e].cpu(), scales[e].cpu(), mode, True,
+                           ref, dtype)
+    # one weight for a batch of x: the batch folds into the rows
+    got2 = mlx_amd.quantized_matmul(x.to(gpu), wq[1], scales[1], mode=mode)
+    assert got2.shape == (2, 3, 5, 64)
+    assert torch.equal(got2[:, 1], got[:, 1])
+    # empty reduction and empty outputs
+    z = mlx_amd.quantized_matmul(torch.zeros((0, 128), dtype=dtype, device=gpu), wq[0], scales[0],
+                                 mode=mode)
+    assert z.shape == (0, 64)
+
+
+@pytest.mark.parametrize("transpose", (True, False))
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_gather_qmm(fp_oracle, gpu, mode, transpose):
+    # python/tests/test_quantized.py:1180-1266 with mode != "affine"
+    dtype = torch.float32
+    g = torch.Generator().manual_seed(13)
+    E, M, N, K = 6, 3, 64, 128
+    w = torch.randn((E, N, K) if transpose else (E, K, N), generator=g).to(dtype)
+    x = torch.randn((4, M, K), generator=g).to(dtype)
+    wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+    lhs = torch.tensor([[0, 3, 1], [2, 2, 0]], dtype=torch.int32)
+    rhs = torch.tensor([[5, 0, 2], [1, 1, 4]], dtype=torch.int32)
+    got = mlx_amd.gather_qmm(x.to(gpu), wq, scales, None, lhs.to(gpu), rhs.to(gpu),
+                             transpose=transpose, mode=mode)
+    assert got.shape == (2, 3, M, N)
+    for i in range(2):
+        for j in range(3):
+            e, b = rhs[i, j].item(), lhs[i, j].item()
+            ref = fp_oracle.qmm(x[b], wq[e].cpu(), scales[e].cpu(), mode, transpose)
+            _check_product(got[i, j].cpu(), x[b], wq[e].cpu(), scales[e].cpu(), mode, transpose,
+                           ref, dtype)
+    # rhs only: x broadcasts against the index shape
+    x1 = x[:1]
+    got = mlx_amd.gather_qmm(x1.to(gpu), wq, scales, None, rhs_indices=rhs.reshape(-1).to(gpu),
+                             transpose=transpose, mode=mode)
+    assert got.shape == (6, M, N)
+    for j, e in enumerate(rhs.reshape(-1).tolist()):
+        ref = fp_oracle.qmm(x1[0], wq[e].cpu(), scales[e].cpu(), mode, transpose)
+        _check_product(got[j].cpu(), x1[0], wq[e].cpu(), scales[e].cpu(), mode, transpose, ref, dtype)
+
+
+@pytest.mark.parametrize("mode", ("nvfp4", "mxfp8", "mxfp4"))
+def test_qqmm(fp_oracle, gpu, mode):
+    """python/tests/test_quantized.py:183-290: qqmm(x, w_q, scales) against
+    dequantize(quantize(x)) @ dequantize(w_q).T, and -- for one row of x, the
+    case the CPU backend implements -- against its result."""
+    for M, N, K in ((1, 128, 256), (8, 128, 128), (33, 256, 256), (64, 128, 256)):
+        g = torch.Generator().manual_seed(M + N)
+        x = torch.randn((M, K), generator=g)
+        w = torch.randn((N, K), generator=g)
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+        got = mlx_amd.qqmm(x.to(gpu), wq, scales, mode=mode)
+        assert got.shape == (M, N) and got.dtype == torch.float32
+        x_hat = fp_oracle.quantize_dequantize(x, mode)
+        w_hat = fp_qref.exact_fp_weights(wq.cpu(), scales.cpu(), mode)
+        want = x_hat.double() @ w_hat.T
+        assert (got.cpu().double() - want).abs().max().item() < 1e-3
+        if M == 1:
+            ref = fp_oracle.qqmm(x, wq.cpu(), scales.cpu(), mode)
+            assert (got.cpu() - ref).abs().max().item() < 1e-4
+        # a floating-point w is quantized inside the call
+        got_w = mlx_amd.qqmm(x.to(gpu), w.to(gpu), mode=mode)
+        assert torch.equal(got_w, got)
+    # gemv input and batched input keep their shapes
+    assert mlx_amd.qqmm(x[0].to(gpu), wq, scales, mode=mode).shape == (N,)
+    assert mlx_amd.qqmm(x.reshape(8, 8, K).to(gpu), wq, scales, mode=mode).shape == (8, 8, N)
+
+
+def test_fp_mode_layers(gpu):
+    import mlx_amd.nn as qnn
+
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(256, 128, bias=True, device=gpu)
+    x = torch.randn((5, 256), device=gpu)
+    for mode in MODES:
+        q = qnn.QuantizedLinear.from_linear(lin, mode=mode)
+        assert q.biases is None and q.scales.dtype == torch.uint8
+        w_hat = mlx_amd.dequantize(q.weight, q.scales, mode=mode, dtype=torch.float32)
+        want = x @ w_hat.T + lin.bias
+        assert (q(x) - want).abs().max().item() < 1e-3
+        emb = qnn.QuantizedEmbedding.from_embedding(torch.nn.Embedding(16, 64, device=gpu), mode=mode)
+        tok = torch.tensor([[1, 5], [0, 15]], device=gpu)
+        assert emb(tok).shape == (2, 2, 64)
+    plain = torch.nn.Linear(256, 128, bias=False, device=gpu)
+    qq = qnn.QQLinear.from_linear(plain)  # training mode: float weight
+    assert qq.weight.dtype == torch.float32 and qq.scales is None
+    y_train = qq(x)
+    qq.eval()
+    assert qq.weight.dtype == torch.uint32 and qq.scales.dtype == torch.uint8
+    assert torch.equal(qq(x), y_train)
+    qq.train()
+    assert qq.weight.dtype == torch.float32
+    with pytest.raises(NotImplementedError):
+        qnn.QQLinear.from_linear(lin)
+    model = torch.nn.Sequential(torch.nn.Linear(64, 64, bias=False, device=gpu))
+    qnn.quantize(model, mode="mxfp8", quantize_input=True)
+    assert isinstance(model[0], qnn.QQLinear)
+
+
+def test_fp_abi_rejects_bad_arguments(gpu):
+    from mlx_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(4096, dtype=torch.uint8, device=gpu)
+    p = buf.data_ptr()
+    assert lib.mlxrocm_fp_quantize(p, p, p, 64, 3, 0, None) == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_fp_quantize(p, p, p, 48, _lib.MXFP4, 0, None) == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_fp_quantize(p, p, p, 64, _lib.MXFP4, 7, None) == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_fp_dequantize(p, p, p, 40, _lib.NVFP4, 0, None) == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_fp_qmm(p, p, p, p, 1, 8, 40, 1, 0, 0, 0, _lib.MXFP8, 0, 1, None) \
+        == _lib.INVALID_ARGUMENT
+    assert "multiple of group_size" in _lib.last_error()
+    assert lib.mlxrocm_fp_qmm(None, p, p, p, 1, 8, 64, 1, 0, 0, 0, _lib.MXFP8, 0, 1, None) \
+        == _lib.INVALID_ARGUMENT
+    # nothing to do
+    assert lib.mlxrocm_fp_quantize(None, None, None, 0, _lib.MXFP4, 0, None) == _lib.OK

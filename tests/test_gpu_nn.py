@@ -29,7 +29,7 @@ def test_quantize_swaps_linear_and_embedding(gpu):
     assert isinstance(m[0], torch.nn.Embedding)
     assert (m[2].group_size, m[2].bits) == (32, 8)
     with pytest.raises(ValueError):
-        qnn.quantize(_model(gpu), group_size=32, mode="mxfp4")
+        qnn.quantize(_model(gpu), group_size=64, mode="mxfp4")
     with pytest.raises(ValueError):
         qnn.quantize(_model(gpu), quantize_input=True)
 

@@ -622,7 +622,7 @@ def test_prefill_call_replays_from_a_hip_graph(oracle, gpu):
 
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
 def test_qmm_prepacked_scale_image(gpu, dtype):
-    """A prefill call that is handed the transposed scale / bias image of its
+    """A prefill call that is handed the transposed (scale, bias) pair image of its
     weight skips the pre-pass and returns the bits of the plain call; shapes that
     read no image ignore it; an image of another weight shape is refused."""
     N, K, gs = 1024, 2048, 64
@@ -630,9 +630,10 @@ def test_qmm_prepacked_scale_image(gpu, dtype):
     wq, s, b = mlx_amd.quantize(w, gs, 4)
     image = mlx_amd.quantized_matmul_sb_image(s, b, gs)
     assert image.numel() == 2 * N * (K // gs) and image.dtype == dtype
-    # the image is the two arrays transposed, scales first
-    assert torch.equal(image[: N * (K // gs)].reshape(K // gs, N), s.T.contiguous())
-    assert torch.equal(image[N * (K // gs):].reshape(K // gs, N), b.T.contiguous())
+    # the image is [K / gs][N] pairs: a row's scale, then its bias
+    pairs = image.reshape(K // gs, N, 2)
+    assert torch.equal(pairs[..., 0], s.T.contiguous())
+    assert torch.equal(pairs[..., 1], b.T.contiguous())
     for M in (1, 8, 600, 2048):
         x = activations((M, K), dtype).to(gpu)
         plain = mlx_amd.quantized_matmul(x, wq, s, b, True, gs, 4)

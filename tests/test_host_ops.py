@@ -27,8 +27,8 @@ def test_quantize_errors():
         mlx_amd.quantize(torch.zeros((4, 64)), bits=7)
     with pytest.raises(ValueError, match="mode"):
         mlx_amd.quantize(torch.zeros((4, 64)), mode="bogus")
-    with pytest.raises(RuntimeError, match="ROCm"):
-        mlx_amd.quantize(torch.zeros((4, 64)), mode="mxfp4")
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.quantize(torch.zeros((4, 64)), mode="mxfp4")  # valid, but not on the device
     with pytest.raises(RuntimeError, match="GPU"):
         mlx_amd.quantize(torch.zeros((4, 64)))  # valid, but not on the device
 
@@ -99,3 +99,68 @@ def test_broadcast_shape_matches_numpy():
                 _broadcast_shape(a, b)
             continue
         assert _broadcast_shape(a, b) == want, (a, b)
+
+
+def test_fp_mode_errors():
+    """Argument checks of the floating-point modes (mlx/ops.cpp:4704-4782,
+    5108-5123, 5351-5390; python/tests/test_quantized.py:41-181) run before any
+    device work."""
+    w = torch.zeros((8, 64))
+    for mode, gs, bits in (("mxfp4", 32, 4), ("mxfp8", 32, 8), ("nvfp4", 16, 4)):
+        with pytest.raises(ValueError, match="requires group size"):
+            mlx_amd.quantize(w, group_size=64, mode=mode)
+        with pytest.raises(ValueError, match="requires bits"):
+            mlx_amd.quantize(w, bits=2 if bits != 2 else 4, mode=mode)
+        with pytest.raises(RuntimeError, match="GPU"):
+            mlx_amd.quantize(w, mode=mode)
+        wq = torch.zeros((8, 64 * bits // 32), dtype=torch.uint32)
+        sc = torch.zeros((8, 64 // gs), dtype=torch.uint8)
+        with pytest.raises(ValueError, match="Scale type must be uint8"):
+            mlx_amd.dequantize(wq, sc.to(torch.float32), mode=mode)
+        with pytest.raises(ValueError, match="Biases must be null"):
+            mlx_amd.dequantize(wq, sc, sc, mode=mode)
+        with pytest.raises(ValueError, match="does not match"):
+            mlx_amd.dequantize(wq, sc[:, :1], mode=mode)
+        with pytest.raises(ValueError, match="output dtype"):
+            mlx_amd.dequantize(wq, sc, mode=mode, dtype=torch.int32)
+        with pytest.raises(ValueError, match="requires group size"):
+            mlx_amd.dequantize(wq, sc, group_size=64, mode=mode)
+        x = torch.zeros((2, 64))
+        with pytest.raises(ValueError, match="Biases must be null"):
+            mlx_amd.quantized_matmul(x, wq, sc, sc, mode=mode)
+        with pytest.raises(ValueError, match="does not match"):
+            mlx_amd.quantized_matmul(x[:, :32], wq, sc, mode=mode)
+        with pytest.raises(ValueError, match="real floating"):
+            mlx_amd.quantized_matmul(x.to(torch.int32), wq, sc, mode=mode)
+        with pytest.raises(RuntimeError, match="GPU"):
+            mlx_amd.quantized_matmul(x, wq, sc, mode=mode)
+        with pytest.raises(RuntimeError, match="GPU"):
+            mlx_amd.gather_qmm(x, wq[None], sc[None], rhs_indices=torch.zeros(1, dtype=torch.int32),
+                               mode=mode)
+    with pytest.raises(ValueError, match="only supported for 'nvfp4'"):
+        mlx_amd.quantize(w, mode="mxfp8", global_scale=torch.ones(()))
+    with pytest.raises(ValueError, match="scalar"):
+        mlx_amd.quantize(w, mode="nvfp4", global_scale=torch.ones(2))
+    with pytest.raises(RuntimeError, match="global scale"):
+        mlx_amd.quantize(w, mode="nvfp4", global_scale=torch.ones(()))
+
+
+def test_qqmm_errors():
+    # validate_qqmm_inputs, mlx/ops.cpp:4836-4894
+    x = torch.zeros((2, 64))
+    wq = torch.zeros((8, 8), dtype=torch.uint32)
+    sc = torch.zeros((8, 4), dtype=torch.uint8)
+    with pytest.raises(ValueError, match="Only 2D"):
+        mlx_amd.qqmm(x, wq[None], sc[None])
+    with pytest.raises(ValueError, match="Scales must be provided"):
+        mlx_amd.qqmm(x, wq)
+    with pytest.raises(ValueError, match="second argument dtype"):
+        mlx_amd.qqmm(x, wq.view(torch.int32), sc)
+    with pytest.raises(ValueError, match="first argument dtype"):
+        mlx_amd.qqmm(x.to(torch.float64), wq, sc)
+    with pytest.raises(ValueError, match="either both"):
+        mlx_amd.qqmm(x, wq, sc, global_scale_x=torch.ones(()))
+    with pytest.raises(ValueError, match="must match last dimension"):
+        mlx_amd.qqmm(x, torch.zeros((8, 32)))
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.qqmm(x, wq, sc)
