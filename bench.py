@@ -441,6 +441,53 @@ def sweep(torch, mlx_amd, dev) -> list:
             matmul_case("cfg5", 1024, 11008, 4096, bits, 32, dtype)
             matmul_case("cfg5", 1, 4096, 11008, bits, 32, dtype)
 
+    # floating-point modes: quantize / dequantize and the matmul at the headline shape
+    def fp_case(mode, M, n, k):
+        from mlx_amd import _lib
+        lib = _lib.load()
+        mcode = {"mxfp4": _lib.MXFP4, "mxfp8": _lib.MXFP8, "nvfp4": _lib.NVFP4}[mode]
+        bits = 8 if mode == "mxfp8" else 4
+        gs = 16 if mode == "nvfp4" else 32
+        q = mlx_amd.quantize(weights(n, k, bf16, std=1.0), mode=mode)
+        wbytes = n * k * bits // 8 + n * (k // gs)
+        small = M <= 64
+        ring = ring_of(q, wbytes) if small else [q]
+        x = torch.randn((M, k), generator=g, dtype=torch.float32).to(bf16).to(dev)
+        out = torch.empty((M, n), dtype=bf16, device=dev)
+        ws_bytes = lib.mlxrocm_fp_qmm_workspace_size(M, n, k, 1, 0, mcode, 2, 1)
+        ws = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=dev)
+
+        def step(i, stream):
+            wq_, s_ = ring[i % len(ring)]
+            rc = lib.mlxrocm_fp_qmm(x.data_ptr(), wq_.data_ptr(), s_.data_ptr(), out.data_ptr(),
+                                    M, n, k, 1, M * k, 0, 0, mcode, 2, 1, ws.data_ptr(), ws_bytes,
+                                    stream)
+            if rc != 0:
+                raise RuntimeError(_lib.last_error())
+
+        launcher = Launcher(torch, step, len(ring), small)
+        launcher.run(len(ring))
+        torch.cuda.synchronize()
+        ms = hip_event_ms(lib, launcher, max(len(ring) * 20, 10) if small else 10)
+        name = f"{mode}: x bfloat16 [{M},{k}] W [{n},{k}]"
+        if small:
+            add("f4", name, ms, nbytes=wbytes + M * k * 2 + M * n * 2)
+        else:
+            add("f4", name, ms, flops=2.0 * M * n * k)
+
+    for mode in ("mxfp4", "mxfp8", "nvfp4"):
+        bits = 8 if mode == "mxfp8" else 4
+        gs = 16 if mode == "nvfp4" else 32
+        w = weights(14336, 4096, bf16, std=1.0)
+        nb = 14336 * 4096 * 2 + 14336 * 4096 * bits // 8 + 14336 * 4096 // gs
+        ms = timed(lambda i: mlx_amd.quantize(w, mode=mode))
+        add("f4", f"quantize bfloat16 [14336,4096] {mode}", ms, nbytes=nb)
+        q = mlx_amd.quantize(w, mode=mode)
+        ms = timed(lambda i: mlx_amd.dequantize(*q, mode=mode))
+        add("f4", f"dequantize bfloat16 [14336,4096] {mode}", ms, nbytes=nb)
+        for M in (1, 4, 512):
+            fp_case(mode, M, 14336, 4096)
+
     # GGUF blocks -> affine triplet (load-time conversion of a [14336, 4096] tensor)
     from mlx_amd import gguf
     for name, type_id, block_bytes, out_bytes in (("Q4_0", 2, 18, 20), ("Q4_1", 3, 20, 20), ("Q8_0", 8, 34, 36)):

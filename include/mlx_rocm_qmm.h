@@ -175,8 +175,20 @@ int mlxrocm_fp_quantize_dequantize(
  * otherwise w [L, K, N bits / 32], scales [L, K, N / group_size]; out
  * [L, M, N].  Batch strides in elements (x), words (w) and bytes (scales); a
  * stride of 0 broadcasts.  Products and sums are evaluated in fp32 and rounded
- * once to dtype.
+ * once to dtype.  workspace: mlxrocm_fp_qmm_workspace_size bytes of device
+ * scratch, 16-byte aligned, used only during the call (prefill shapes decode
+ * the scales into an image first; 0 bytes for decode shapes, float32 and
+ * transpose == 0, and then it may be NULL).
  */
+size_t mlxrocm_fp_qmm_workspace_size(
+    int M,
+    int N,
+    int K,
+    int L,
+    int batched_weights, /* scales_batch_stride != 0 */
+    int mode,
+    int dtype,
+    int transpose);
 int mlxrocm_fp_qmm(
     const void* x,
     const uint32_t* wq,
@@ -192,6 +204,8 @@ int mlxrocm_fp_qmm(
     int mode,
     int dtype,
     int transpose,
+    void* workspace,
+    size_t workspace_bytes,
     mlxrocm_stream_t stream);
 
 /* gather_qmm for the floating-point modes (mlx/ops.cpp:5553-5629 with

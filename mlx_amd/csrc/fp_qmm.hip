@@ -12,8 +12,14 @@
 // owns 16 bytes of a packed row per step -- whole 1 KiB pieces of one row per
 // wavefront instruction, as in the affine decode kernels -- and up to four rows
 // of x per pass; more rows of x repeat the pass (the weights are re-read once
-// per four rows: a functional floor for prefill, not a tile GEMM).
+// per four rows: a functional floor for prefill, not a tile GEMM).  For the
+// 16-bit element types the codes are widened two at a time by the hardware's
+// fp4 / fp8 converts (v_cvt_scalef32_pk_{bf16,f16}_{fp4,fp8} with scale 1: both
+// formats are exact in bf16 and f16) and multiplied with v_dot2_f32_{bf16,f16};
+// the group's scale is applied to the partial sum, once per group.
 // transpose=false: one thread per eight output columns, k ascending.
+#include <type_traits>
+
 #include "qmm_args.h"
 
 namespace mlxrocm {
@@ -173,6 +179,196 @@ __global__ __launch_bounds__(64 * kFpWaves) void fp_qmv_kernel(const QmmArgs a) 
   }
 }
 
+typedef __bf16 fp_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 fp_f16x2 __attribute__((ext_vector_type(2)));
+
+// Codes -> pairs of T, packed in a dword (first code in the low half), and the
+// two-element dot product with fp32 accumulation.
+template <typename T>
+struct FpWiden;
+
+template <>
+struct FpWiden<bf16_t> {
+  // the eight e2m1 codes of a word: byte b holds codes 2 b (low nibble), 2 b + 1
+  static __device__ __forceinline__ void fp4(uint32_t w, uint32_t (&p)[4]) {
+    p[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 0));
+    p[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 1));
+    p[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 2));
+    p[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 3));
+  }
+  // the four e4m3 codes of a word
+  static __device__ __forceinline__ void fp8(uint32_t w, uint32_t (&p)[2]) {
+    p[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+    p[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true));
+  }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(
+        __builtin_bit_cast(fp_bf16x2, a), __builtin_bit_cast(fp_bf16x2, b), c, false);
+  }
+};
+
+template <>
+struct FpWiden<f16_t> {
+  static __device__ __forceinline__ void fp4(uint32_t w, uint32_t (&p)[4]) {
+    p[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 0));
+    p[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 1));
+    p[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 2));
+    p[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 3));
+  }
+  static __device__ __forceinline__ void fp8(uint32_t w, uint32_t (&p)[2]) {
+    p[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+    p[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
+  }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(
+        __builtin_bit_cast(fp_f16x2, a), __builtin_bit_cast(fp_f16x2, b), c, false);
+  }
+};
+
+// An e4m3 byte whose low seven bits are all ones: NaN to the hardware convert,
+// +-480 to the reference's decoder (mlx/backend/cpu/quantized.cpp FromFP8, which
+// has no special codes).  The quantizer never writes it (it saturates at 448).
+__device__ __forceinline__ bool has_e4m3_top_code(uint32_t w) {
+  return (((w & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u) != 0;
+}
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  const T a = from_f32<T>(lo);
+  const T b = from_f32<T>(hi);
+  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, a)) |
+      (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, b)) << 16);
+}
+
+// 16-byte load of data that is read exactly once: nontemporal, so the stream
+// does not displace x and the scales from the caches.
+__device__ __forceinline__ uint4 load_once(const uint8_t* p) {
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+constexpr int kFp16Waves = 4;
+
+// 16-bit element types, K % (128 / BITS) == 0.  MB rows of x per pass (1, 2 or
+// 4), RPW rows of w per wavefront.
+template <typename T, int GS, int BITS, int MB, int RPW>
+__global__ __launch_bounds__(64 * kFp16Waves) void fp_qmv16_kernel(const QmmArgs a) {
+  constexpr int kCodes = 128 / BITS; // codes per lane and step: 32 or 16
+  constexpr int kPairs = kCodes / 2;
+  constexpr int kGroups = kCodes / GS > 0 ? kCodes / GS : 1;
+  constexpr int kPairsPerGroup = kPairs / kGroups;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const FpProblem p = fp_resolve(a, blockIdx.z, sizeof(T));
+  const int K = a.K;
+  const int N = a.N;
+  const int m0 = blockIdx.y * MB;
+  const int n0 = (blockIdx.x * kFp16Waves + wave) * RPW;
+  if (n0 >= N) {
+    return;
+  }
+  const size_t row_bytes = static_cast<size_t>(K) * BITS / 8;
+  const int groups = K / GS;
+  const T* x = reinterpret_cast<const T*>(p.x);
+
+  float acc[RPW][MB];
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      acc[r][m] = 0.0f;
+    }
+  }
+  const uint8_t* wrow[RPW];
+  const uint8_t* srow[RPW];
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    const int n = n0 + r < N ? n0 + r : N - 1; // clamp: stay in bounds
+    wrow[r] = p.w + static_cast<size_t>(n) * row_bytes;
+    srow[r] = p.scales + static_cast<size_t>(n) * groups;
+  }
+  for (int k0 = lane * kCodes; k0 < K; k0 += 64 * kCodes) {
+    uint4 wv[RPW];
+    uint32_t sb[RPW][kGroups];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      wv[r] = load_once(wrow[r] + static_cast<size_t>(k0) * BITS / 8);
+#pragma unroll
+      for (int g = 0; g < kGroups; ++g) {
+        sb[r][g] = srow[r][k0 / GS + g];
+      }
+    }
+    // this lane's slice of the rows of x, as pairs
+    uint32_t xr[MB][kPairs];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const int row = m0 + m < a.M ? m0 + m : a.M - 1;
+      const uint4* src = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row) * K + k0);
+#pragma unroll
+      for (int j = 0; j < kPairs / 4; ++j) {
+        const uint4 v = src[j];
+        xr[m][4 * j + 0] = v.x;
+        xr[m][4 * j + 1] = v.y;
+        xr[m][4 * j + 2] = v.z;
+        xr[m][4 * j + 3] = v.w;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      const uint32_t words[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+      uint32_t pr[kPairs];
+      if constexpr (BITS == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          uint32_t q[4];
+          FpWiden<T>::fp4(words[i], q);
+          pr[4 * i + 0] = q[0];
+          pr[4 * i + 1] = q[1];
+          pr[4 * i + 2] = q[2];
+          pr[4 * i + 3] = q[3];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          uint32_t q[2];
+          FpWiden<T>::fp8(words[i], q);
+          if (has_e4m3_top_code(words[i])) {
+            q[0] = pack_pair<T>(e4m3_value(words[i] & 0xffu), e4m3_value((words[i] >> 8) & 0xffu));
+            q[1] = pack_pair<T>(e4m3_value((words[i] >> 16) & 0xffu), e4m3_value(words[i] >> 24));
+          }
+          pr[2 * i + 0] = q[0];
+          pr[2 * i + 1] = q[1];
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < kGroups; ++g) {
+        const float s = scale_value<GS>(sb[r][g]);
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+          float part = 0.0f;
+#pragma unroll
+          for (int j = 0; j < kPairsPerGroup; ++j) {
+            part = FpWiden<T>::dot2(xr[m][g * kPairsPerGroup + j], pr[g * kPairsPerGroup + j], part);
+          }
+          acc[r][m] = fmaf(s, part, acc[r][m]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const float y = wave_sum(acc[r][m]);
+      if (lane == 0 && m0 + m < a.M && n0 + r < N) {
+        reinterpret_cast<T*>(p.out)[static_cast<size_t>(m0 + m) * N + n0 + r] =
+            from_f32<T>(p.valid ? y : 0.0f);
+      }
+    }
+  }
+}
+
 // transpose=true, any K that is a multiple of the group size: one thread per
 // output element (nvfp4 rows whose length is an odd multiple of 16).
 template <typename T, int GS, int BITS>
@@ -283,6 +479,39 @@ int fp_check(const char* who, int M, int N, int K, int L, int mode, int dtype, i
   return MLXROCM_OK;
 }
 
+// From this many rows of x on, 16-bit problems with transpose=true run on the
+// matrix-core tile kernel (one pass over W, K split into ranges while the tiles
+// do not fill the chip) instead of one streaming pass per four rows.  bf16
+// [M, 4096] x [14336, 4096], mxfp4 / mxfp8 / nvfp4: streaming 43 / 36 / 36 us at
+// 8 rows (two passes); the tile kernel with its scale pre-pass 37 / 39 / 40 us at
+// 9 rows, 39 / 41 / 43 at 64, 70 / 73 / 75 at 512.
+constexpr int kFpTileMinM = 9;
+
+// The tile kernel addresses its operands with 32-bit byte offsets.
+bool fp_tile_applies(int M, int N, int K, int L, int mode, int dtype, bool transpose) {
+  const int bits = mode == MLXROCM_MXFP8 ? 8 : 4;
+  const uint64_t limit = uint64_t{1} << 32;
+  return transpose && dtype != MLXROCM_FLOAT32 && M >= kFpTileMinM && K % 64 == 0 && K >= 64 &&
+      L >= 1 && static_cast<uint64_t>(N) * K * bits / 8 < limit &&
+      static_cast<uint64_t>(M) * K * 2 < limit && static_cast<uint64_t>(M) * N * 2 < limit &&
+      static_cast<uint64_t>(N) * (K / 32) * 4 < limit;
+}
+
+size_t fp_image_bytes(int N, int K, int batches) {
+  return (static_cast<size_t>(batches) * N * (K / 32) * 4 + 255) / 256 * 256;
+}
+
+// ranges of K for a launch whose tiles do not fill the compute units
+int fp_k_splits(int M, int N, int K, int L) {
+  return (static_cast<int64_t>(M) * N) % 4 == 0 ? qmm_mfma_k_splits(M, N, K, L) : 1;
+}
+
+size_t fp_tile_workspace(int M, int N, int K, int L, int batches) {
+  const int splits = fp_k_splits(M, N, K, L);
+  const size_t planes = splits > 1 ? static_cast<size_t>(M) * N * splits * sizeof(float) : 0;
+  return fp_image_bytes(N, K, batches) + planes;
+}
+
 // L problems (batch entries or index pairs), at most 65535 per launch.
 int fp_launch(const QmmArgs& a, int mode, int dtype, bool transpose, hipStream_t s) {
   if (a.L > 65535 || a.M > 65535 * kFpRowBlock) {
@@ -297,6 +526,21 @@ int fp_launch(const QmmArgs& a, int mode, int dtype, bool transpose, hipStream_t
         MLXROCM_REHEARSE("fp_qmm_n");
         const dim3 grid((a.N / 8 + 255) / 256, a.M, a.L);
         fp_qmm_n_kernel<T, G, B><<<grid, 256, 0, s>>>(a);
+      } else if (a.K % (128 / B) == 0 && !std::is_same_v<T, float>) {
+        if constexpr (!std::is_same_v<T, float>) {
+          constexpr int kRows = 2; // rows of w per wavefront
+          const int mb = a.M == 1 ? 1 : (a.M == 2 ? 2 : 4);
+          MLXROCM_REHEARSE("fp_qmv16(mb=%d)", mb);
+          const int rows_per_wg = kFp16Waves * kRows;
+          const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, (a.M + mb - 1) / mb, a.L);
+          if (mb == 1) {
+            fp_qmv16_kernel<T, G, B, 1, kRows><<<grid, 64 * kFp16Waves, 0, s>>>(a);
+          } else if (mb == 2) {
+            fp_qmv16_kernel<T, G, B, 2, kRows><<<grid, 64 * kFp16Waves, 0, s>>>(a);
+          } else {
+            fp_qmv16_kernel<T, G, B, 4, kRows><<<grid, 64 * kFp16Waves, 0, s>>>(a);
+          }
+        }
       } else if (a.K % (128 / B) == 0) {
         MLXROCM_REHEARSE("fp_qmv");
         const int rows_per_wg = kFpWaves * kFpRowsPerWave;
@@ -339,6 +583,8 @@ extern "C" int mlxrocm_fp_qmm(
     int mode,
     int dtype,
     int transpose,
+    void* workspace,
+    size_t workspace_bytes,
     mlxrocm_stream_t stream) {
   mlxrocm::ApiRange api_range("mlxrocm_fp_qmm");
   int rc = fp_check("quantized_matmul", M, N, K, L, mode, dtype, transpose);
@@ -378,7 +624,52 @@ extern "C" int mlxrocm_fp_qmm(
   a.sb_batch_stride = scales_batch_stride;
   a.x_batches = L;
   a.n_experts = L;
+  if (fp_tile_applies(M, N, K, L, mode, dtype, transpose != 0)) {
+    const int batches = scales_batch_stride != 0 ? L : 1;
+    const size_t need = fp_tile_workspace(M, N, K, L, batches);
+    if (workspace == nullptr || workspace_bytes < need ||
+        (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
+      return fail(
+          MLXROCM_INVALID_ARGUMENT,
+          "[quantized_matmul] this shape needs a 16-byte aligned workspace of %zu bytes "
+          "(mlxrocm_fp_qmm_workspace_size); got %zu",
+          need, workspace_bytes);
+    }
+    rc = fp_scale_image_for_qmm_t(
+        scales, workspace, N, K, batches, scales_batch_stride, mode, dtype, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    a.scales = workspace;
+    a.biases = workspace;
+    a.sb_transposed = 2;
+    // elements of T between the images of two batch entries
+    a.sb_batch_stride = batches > 1 ? static_cast<int64_t>(N) * (K / 32) * 2 : 0;
+    const int splits = fp_k_splits(M, N, K, L);
+    if (splits <= 1) {
+      return launch_qmm_mfma_fp(a, mode, dtype, 1, s);
+    }
+    void* partial = static_cast<char*>(workspace) + fp_image_bytes(N, K, batches);
+    a.out = partial;
+    rc = launch_qmm_mfma_fp(a, mode, dtype, splits, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    return reduce_k_splits(partial, out, static_cast<size_t>(M) * N, splits, dtype, s);
+  }
   return fp_launch(a, mode, dtype, transpose != 0, s);
+}
+
+extern "C" size_t mlxrocm_fp_qmm_workspace_size(
+    int M, int N, int K, int L, int batched_weights, int mode, int dtype, int transpose) {
+  if (fp_check("quantized_matmul", M, N, K, L, mode, dtype, transpose) != MLXROCM_OK ||
+      static_cast<int64_t>(M) * N * L == 0 || K == 0) {
+    return 0;
+  }
+  if (!fp_tile_applies(M, N, K, L, mode, dtype, transpose != 0)) {
+    return 0;
+  }
+  return fp_tile_workspace(M, N, K, L, batched_weights ? L : 1);
 }
 
 extern "C" int mlxrocm_fp_gather_qmm(

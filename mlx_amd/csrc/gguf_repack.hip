@@ -88,18 +88,27 @@ __global__ __launch_bounds__(kRepackBlock) void gguf_repack_kernel(
     }
   } else {
     // byte j holds element j (low nibble) and element j + 16 (high nibble);
-    // the packed stream wants element e at bit 4 e
+    // the packed stream wants element e at bit 4 e.  The quants start 2 bytes
+    // into an 18-byte block (Q4_0), so they are read as halfwords; byte reads
+    // (what the compiler makes of an indexed byte loop) ran this format at a
+    // quarter of the rate of the other two.
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t lo = *reinterpret_cast<const uint16_t*>(q + 4 * i);
+      const uint32_t hi = *reinterpret_cast<const uint16_t*>(q + 4 * i + 2);
+      w[i] = lo | (hi << 16);
+    }
+    // the four low nibbles of a word's bytes, packed into 16 bits
+    auto squeeze = [](uint32_t v) {
+      v &= 0x0f0f0f0fu;
+      v = (v | (v >> 4)) & 0x00ff00ffu;
+      return (v | (v >> 8)) & 0xffffu;
+    };
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      uint32_t lo = 0, hi = 0;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t byte = q[8 * i + j];
-        lo |= (byte & 0xfu) << (4 * j);
-        hi |= (byte >> 4) << (4 * j);
-      }
-      out[i] = lo;
-      out[2 + i] = hi;
+      out[i] = squeeze(w[2 * i]) | (squeeze(w[2 * i + 1]) << 16);
+      out[2 + i] = squeeze(w[2 * i] >> 4) | (squeeze(w[2 * i + 1] >> 4) << 16);
     }
   }
   const size_t b = b0 + tid;

@@ -107,6 +107,71 @@ struct PairDequant {
   }
 };
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// The floating-point modes in the same shape: 32 codes of one row of W in four
+// (e2m1) or eight (e4m3) consecutive dwords, pair<Q>() returns elements 2Q and
+// 2Q+1 times their group's scale, packed as T.  Every such product is exact in
+// bf16 and f16 (at most 4 significant bits times a power of two, or 2 times 4).
+//   FP == 1: e2m1 codes, one power-of-two scale `s` for all 32 (mxfp4)
+//   FP == 2: e4m3 codes, one power-of-two scale `s` for all 32 (mxfp8)
+//   FP == 3: e2m1 codes, scale `s` for codes 0..15 and `b` for 16..31 (nvfp4)
+// With a power-of-two scale the hardware convert applies it: one instruction
+// per pair.  The e4m3 bytes 0x7f / 0xff, which the quantizer never writes, are
+// NaN to that convert.
+template <typename T, int FP>
+struct FpPairDequant {
+  static constexpr float kCodeScale = 1.0f;
+  static constexpr int kWords = FP == 2 ? 8 : 4;
+
+  template <int Q>
+  __device__ __forceinline__ uint32_t
+  pair(const uint32_t (&w)[kWords], float s, float b, bool = false) {
+    if constexpr (FP == 1) {
+      if constexpr (std::is_same<T, bf16_t>::value) {
+        return __builtin_bit_cast(
+            uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[Q / 4], s, Q % 4));
+      } else {
+        return __builtin_bit_cast(
+            uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[Q / 4], s, Q % 4));
+      }
+    } else if constexpr (FP == 2) {
+      if constexpr (std::is_same<T, bf16_t>::value) {
+        return __builtin_bit_cast(
+            uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[Q / 2], s, Q % 2 == 1));
+      } else {
+        return __builtin_bit_cast(
+            uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[Q / 2], s, Q % 2 == 1));
+      }
+    } else {
+      const floatx2 v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[Q / 4], 1.0f, Q % 4);
+      const float sc = Q < 8 ? s : b;
+      return pack2<T>(v[0] * sc, v[1] * sc);
+    }
+  }
+};
+
+template <typename T, int FP, int... Q>
+__device__ __forceinline__ void dequant32_fp_impl(
+    const uint32_t (&w)[FpPairDequant<T, FP>::kWords],
+    float s,
+    float b,
+    uint32_t (&out)[16],
+    std::integer_sequence<int, Q...>) {
+  FpPairDequant<T, FP> dq;
+  ((out[Q] = dq.template pair<Q>(w, s, b)), ...);
+}
+
+template <typename T, int FP>
+__device__ __forceinline__ void dequant32_fp(
+    const uint32_t (&w)[FpPairDequant<T, FP>::kWords],
+    float s,
+    float b,
+    uint32_t (&out)[16]) {
+  dequant32_fp_impl<T, FP>(w, s, b, out, std::make_integer_sequence<int, 16>{});
+}
+
 // Dequantization of a 4 (k) x 8 (n) block of a [K, N] weight matrix whose codes
 // run along n: w holds, row by row, the BITS / 4 words with the 8 codes of each
 // of the 4 rows, s / b the rows' scale and bias.  pair<Q>() returns column

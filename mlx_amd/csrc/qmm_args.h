@@ -115,6 +115,22 @@ int launch_qmm_mfma_pairs(const QmmArgs& a, int gs, int bits, int dtype, hipStre
 int launch_qmm_mfma_ksplit_pairs(
     const QmmArgs& a, int gs, int bits, int dtype, int k_splits, hipStream_t s);
 
+// The tile kernel for the floating-point modes (qmm_mfma_fp.hip): `mode` is a
+// mlxrocm_fp_mode, a.scales the scale image that fp_scale_image_for_qmm_t builds
+// from the caller's byte scales (batches * (K / 32) * N dwords), K % 64 == 0,
+// 16-bit dtype.
+int fp_scale_image_for_qmm_t(
+    const uint8_t* scales,
+    void* out,
+    int N,
+    int K,
+    int batches,
+    int64_t src_stride,
+    int mode,
+    int dtype,
+    hipStream_t s);
+int launch_qmm_mfma_fp(const QmmArgs& a, int mode, int dtype, int k_splits, hipStream_t s);
+
 bool qmv_wide_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmv_wide(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 bool qmm_skinny_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);

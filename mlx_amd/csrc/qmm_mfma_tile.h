@@ -100,8 +100,11 @@ constexpr int wstore_at(int m, int ns) {
 // stores it to the same [n][k] LDS tile as eight 8-byte column pieces.
 // SBI: a.scales points at the image of (scale, bias) pairs (QmmArgs::sb_transposed
 // == 2): one dword load per thread and K-step instead of two 16-bit loads.
+// FP != 0: the codes are e2m1 / e4m3 numbers (FpPairDequant's modes) instead of
+// affine integers; the pair image then holds, per 32 codes, the scale of the
+// first 16 in the low half and of the last 16 in the high half (gs_shift == 5).
 template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED, bool WN = false,
-          bool SBI = false>
+          bool SBI = false, int FP = 0>
 __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     const QmmArgs a,
     const int gs_shift,
@@ -111,6 +114,8 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   static_assert(!(WN && kSplit), "[K, N] weights: 16-bit problems only");
   static_assert(!WN || BITS == 4 || BITS == 8, "[K, N] weights: 4- and 8-bit codes");
   static_assert(!SBI || (!WN && !GROUPED && !kSplit && sizeof(TS) == 2), "pair image: plain 16-bit launches");
+  static_assert(FP == 0 || (SBI && BITS == (FP == 2 ? 8 : 4)), "fp codes: pair image, 4 or 8 bits");
+  using DQ = std::conditional_t<FP != 0, FpPairDequant<T, (FP != 0 ? FP : 1)>, PairDequant<T, BITS>>;
   constexpr int kBN = 32 * NT;
   constexpr int kNS = 8 * NT; // MFMAs per wavefront per K-step
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -376,7 +381,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
             make_uint2(dq__[2 * i__], dq__[2 * i__ + 1]);                        \
       }                                                                          \
     } else {                                                                     \
-      dequant32<T, BITS>(wreg, raw_value<TS>(sreg), raw_value<TS>(breg), dq__);  \
+      if constexpr (FP != 0) {                                                   \
+        dequant32_fp<T, (FP != 0 ? FP : 1)>(                                     \
+            wreg, raw_value<TS>(sreg), raw_value<TS>(breg), dq__);               \
+      } else {                                                                   \
+        dequant32<T, BITS>(wreg, raw_value<TS>(sreg), raw_value<TS>(breg), dq__); \
+      }                                                                          \
       _Pragma("unroll") for (int j__ = 0; j__ < 4; ++j__) {                      \
         *reinterpret_cast<uint4*>(ws__ + wrow_off[j__]) = make_uint4(            \
             dq__[4 * j__], dq__[4 * j__ + 1], dq__[4 * j__ + 2], dq__[4 * j__ + 3]); \
@@ -567,13 +577,13 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     float sf[kSB], bf[kSB];                                                      \
     _Pragma("unroll") for (int j__ = 0; j__ < kSB; ++j__) {                      \
       sf[j__] = WN ? wn_value(swn, j__)                                          \
-                   : raw_value<TS>(sreg) * PairDequant<T, BITS>::kCodeScale;     \
+                   : raw_value<TS>(sreg) * DQ::kCodeScale;                       \
       bf[j__] = WN ? wn_value(bwn, j__) : raw_value<TS>(breg);                   \
     }                                                                            \
     /* the tile prepared in step tt is tile tt + 1: block (tt + 1) % 3 of its   \
        group of three takes the weights' low parts */                           \
     const bool low_part = kSplit && ((tt) + 1) % 3 == 2;                         \
-    PairDequant<T, BITS> dq;                                                     \
+    DQ dq;                                                                       \
     ColDequant<T, (WN ? BITS : 4)> cdq;                                          \
     uint32_t dqv[16];                                                            \
     __builtin_amdgcn_sched_barrier(0);                                           \
@@ -718,13 +728,13 @@ int choose_nt(int M, int N, int L, int min_nt = 5) {
 }
 
 template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED, bool WN = false,
-          bool SBI = false>
+          bool SBI = false, int FP = 0>
 int launch_variant(const QmmArgs& a, int gs_shift, dim3 grid, hipStream_t s, int k_splits = 1) {
   constexpr size_t smem = qmm_smem_bytes<NT>();
   if (grid.y > 65535u || grid.z > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qmm] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
-  auto kern = qmm_t_mfma_kernel<T, TS, TO, BITS, NT, GROUPED, WN, SBI>;
+  auto kern = qmm_t_mfma_kernel<T, TS, TO, BITS, NT, GROUPED, WN, SBI, FP>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(

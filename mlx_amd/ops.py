@@ -486,11 +486,15 @@ def quantized_matmul(
     out = torch.empty(out_shape, dtype=dtype, device=x.device)
     code = _DTYPE_CODE[dtype]
     if not affine:
+        ws_bytes = lib.mlxrocm_fp_qmm_workspace_size(
+            M, w_outer, K, L, int(sb_stride != 0), _MODE_CODE[mode], code, int(bool(transpose)))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
         _lib.check(
             lib.mlxrocm_fp_qmm(
                 xb.data_ptr(), wb.data_ptr(), sb.data_ptr(), out.data_ptr(),
                 M, w_outer, K, L, M * K, w_stride, sb_stride, _MODE_CODE[mode], code,
-                int(bool(transpose)), _stream_ptr(x),
+                int(bool(transpose)), ws.data_ptr() if ws is not None else None, ws_bytes,
+                _stream_ptr(x),
             )
         )
         return out

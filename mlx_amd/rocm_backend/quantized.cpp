@@ -1,6 +1,7 @@
-// quantized.cpp -- eval_gpu of the affine quantization primitives for the ROCm
-// backend: QuantizedMatmul, GatherQMM and fast::Quantize
-// (mlx/primitives.h:1616-1717, mlx/fast_primitives.h:337-371).
+// quantized.cpp -- eval_gpu of the quantization primitives for the ROCm
+// backend: QuantizedMatmul, QQMatmul, GatherQMM and fast::Quantize
+// (mlx/primitives.h:1616-1717, mlx/fast_primitives.h:337-371), in the affine
+// mode and the floating-point modes mxfp4 / mxfp8 / nvfp4.
 //
 // Each body does what the CUDA backend's does around its kernels
 // (mlx/backend/cuda/quantized/quantized.cpp:15-324): make operands dense where
@@ -42,12 +43,23 @@ int dtype_code(Dtype t, const char* who) {
   }
 }
 
-void require_affine(QuantizationMode mode, const char* who) {
-  if (mode != QuantizationMode::Affine) {
+int fp_mode_code(QuantizationMode mode) {
+  switch (mode) {
+    case QuantizationMode::Mxfp4:
+      return MLXROCM_MXFP4;
+    case QuantizationMode::Mxfp8:
+      return MLXROCM_MXFP8;
+    default:
+      return MLXROCM_NVFP4;
+  }
+}
+
+// nvfp4 takes an optional tensor-wide scale as a trailing input
+// (mlx/ops.cpp:5124-5128, 5393-5397): not implemented by these kernels.
+void no_global_scale(bool present, const char* who) {
+  if (present) {
     std::ostringstream msg;
-    msg << "[" << who << "] quantization mode '"
-        << quantization_mode_to_string(mode)
-        << "' has no ROCm implementation; only 'affine' is supported.";
+    msg << "[" << who << "] nvfp4 with a global scale has no ROCm implementation.";
     throw std::runtime_error(msg.str());
   }
 }
@@ -118,14 +130,13 @@ bool single_batch_stride(const array& a) {
 } // namespace
 
 void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
-  require_affine(mode_, "quantized_matmul");
   auto& s = stream();
   auto& enc = rocm::get_command_encoder(s);
+  const bool affine = mode_ == QuantizationMode::Affine;
 
   array x = ensure_row_contiguous(inputs[0], enc, s);
   array w = ensure_row_contiguous(inputs[1], enc, s);
   array scales = ensure_row_contiguous(inputs[2], enc, s);
-  array biases = ensure_row_contiguous(inputs[3], enc, s);
 
   out.set_data(allocator::malloc(out.nbytes()));
 
@@ -148,6 +159,39 @@ void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
     L = 1;
   }
   const int dt = dtype_code(x.dtype(), "quantized_matmul");
+
+  if (!affine) {
+    // inputs are {x, w, scales}: no biases (mlx/ops.cpp:4816-4821)
+    const int mode = fp_mode_code(mode_);
+    const size_t ws_bytes = mlxrocm_fp_qmm_workspace_size(
+        M, N, K, L, w.ndim() > 2, mode, dt, transpose_ ? 1 : 0);
+    void* ws_ptr = nullptr;
+    if (ws_bytes > 0) {
+      array ws = workspace_array(ws_bytes);
+      enc.add_temporary(ws);
+      ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
+    }
+    rocm::check(mlxrocm_fp_qmm(
+        rocm::gpu_ptr<void>(x, enc.stream()),
+        rocm::gpu_ptr<uint32_t>(w, enc.stream()),
+        rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+        rocm::gpu_ptr<void>(out, enc.stream()),
+        M,
+        N,
+        K,
+        L,
+        int64_t(M) * K,
+        w_stride,
+        sb_stride,
+        mode,
+        dt,
+        transpose_ ? 1 : 0,
+        ws_ptr,
+        ws_bytes,
+        enc.stream()));
+    return;
+  }
+  array biases = ensure_row_contiguous(inputs[3], enc, s);
 
   // device scratch of the call: a temporary like any other
   const size_t ws_bytes = mlxrocm_qmm_workspace_size(
@@ -181,15 +225,104 @@ void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
       enc.stream()));
 }
 
-void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
-  require_affine(mode_, "gather_qmm");
+// x is quantized and dequantized on the fly in its own type, then multiplied by
+// the transposed quantized w: what QQMatmul::eval_cpu does for one row of x
+// (mlx/backend/cpu/quantized.cpp:1322-1360), here for any number of rows.  A
+// floating-point w (inputs {x, w}) is quantized into temporaries first, as the
+// CUDA backend does (mlx/backend/cuda/quantized/qqmm.cpp).
+void QQMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
   auto& s = stream();
   auto& enc = rocm::get_command_encoder(s);
+  if (mode_ == QuantizationMode::Affine) {
+    throw std::runtime_error("[qqmm] Affine quantization is not supported.");
+  }
+  const bool w_quantized = inputs[1].dtype() == uint32;
+  no_global_scale(inputs.size() > (w_quantized ? 3u : 2u), "qqmm");
+  const int mode = fp_mode_code(mode_);
+
+  array x = ensure_row_contiguous(inputs[0], enc, s);
+  array w = ensure_row_contiguous(inputs[1], enc, s);
+  const int K = x.shape(-1);
+  const int N = out.shape(-1);
+  const int64_t rows = K == 0 ? 0 : static_cast<int64_t>(x.size() / size_t(K));
+  if (rows > std::numeric_limits<int>::max()) {
+    throw std::runtime_error("[qqmm] more than 2^31 - 1 rows of x");
+  }
+  const int dt = dtype_code(x.dtype(), "qqmm");
+
+  array scales = w_quantized ? ensure_row_contiguous(inputs[2], enc, s)
+                             : array({N, K / group_size_}, uint8, nullptr, {});
+  if (!w_quantized) {
+    if (w.dtype() != x.dtype()) {
+      throw std::runtime_error("[qqmm] x and a floating-point w must share one type");
+    }
+    array wq({N, K * bits_ / 32}, uint32, nullptr, {});
+    wq.set_data(allocator::malloc(wq.nbytes()));
+    scales.set_data(allocator::malloc(scales.nbytes()));
+    enc.add_temporary(wq);
+    enc.add_temporary(scales);
+    rocm::check(mlxrocm_fp_quantize(
+        rocm::gpu_ptr<void>(w, enc.stream()),
+        rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+        rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+        w.size(),
+        mode,
+        dt,
+        enc.stream()));
+    w = wq;
+  }
+
+  out.set_data(allocator::malloc(out.nbytes()));
+  array xhat(x.shape(), x.dtype(), nullptr, {});
+  xhat.set_data(allocator::malloc(xhat.nbytes()));
+  enc.add_temporary(xhat);
+  rocm::check(mlxrocm_fp_quantize_dequantize(
+      rocm::gpu_ptr<void>(x, enc.stream()),
+      rocm::gpu_ptr<void>(xhat, enc.stream()),
+      x.size(),
+      mode,
+      dt,
+      enc.stream()));
+  const size_t ws_bytes =
+      mlxrocm_fp_qmm_workspace_size(static_cast<int>(rows), N, K, 1, 0, mode, dt, 1);
+  void* ws_ptr = nullptr;
+  if (ws_bytes > 0) {
+    array ws = workspace_array(ws_bytes);
+    enc.add_temporary(ws);
+    ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
+  }
+  rocm::check(mlxrocm_fp_qmm(
+      rocm::gpu_ptr<void>(xhat, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(w, enc.stream()),
+      rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+      rocm::gpu_ptr<void>(out, enc.stream()),
+      static_cast<int>(rows),
+      N,
+      K,
+      1,
+      0,
+      0,
+      0,
+      mode,
+      dt,
+      1,
+      ws_ptr,
+      ws_bytes,
+      enc.stream()));
+}
+
+void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
+  auto& s = stream();
+  auto& enc = rocm::get_command_encoder(s);
+  const bool affine = mode_ == QuantizationMode::Affine;
+  // inputs: {x, w, scales, biases, lhs, rhs}; without biases in the
+  // floating-point modes (mlx/ops.cpp:5601-5618)
+  const int first_index = affine ? 4 : 3;
 
   array x = ensure_row_contiguous(inputs[0], enc, s);
   array w = ensure_dense_matrices(inputs[1], enc, s);
   array scales = ensure_dense_matrices(inputs[2], enc, s);
-  array biases = ensure_dense_matrices(inputs[3], enc, s);
+  array biases = affine ? ensure_dense_matrices(inputs[3], enc, s) : scales;
   // A stack the kernels can address as base + e * stride keeps its layout
   // (sliced expert stacks); anything more exotic is made dense.
   if (!single_batch_stride(w) || !single_batch_stride(scales) ||
@@ -197,10 +330,10 @@ void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
       matrix_stride(scales) != matrix_stride(biases)) {
     w = ensure_row_contiguous(w, enc, s);
     scales = ensure_row_contiguous(scales, enc, s);
-    biases = ensure_row_contiguous(biases, enc, s);
+    biases = affine ? ensure_row_contiguous(biases, enc, s) : scales;
   }
-  array lhs = ensure_row_contiguous(inputs[4], enc, s);
-  array rhs = ensure_row_contiguous(inputs[5], enc, s);
+  array lhs = ensure_row_contiguous(inputs[first_index], enc, s);
+  array rhs = ensure_row_contiguous(inputs[first_index + 1], enc, s);
 
   out.set_data(allocator::malloc(out.nbytes()));
 
@@ -212,6 +345,30 @@ void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
   const int n_experts =
       static_cast<int>(w.size() / (size_t(w.shape(-1)) * w.shape(-2)));
   const int dt = dtype_code(x.dtype(), "gather_qmm");
+
+  if (!affine) {
+    rocm::check(mlxrocm_fp_gather_qmm(
+        rocm::gpu_ptr<void>(x, enc.stream()),
+        rocm::gpu_ptr<uint32_t>(w, enc.stream()),
+        rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+        rocm::gpu_ptr<uint32_t>(lhs, enc.stream()),
+        rocm::gpu_ptr<uint32_t>(rhs, enc.stream()),
+        rocm::gpu_ptr<void>(out, enc.stream()),
+        M,
+        N,
+        K,
+        n_idx,
+        x_batches,
+        n_experts,
+        int64_t(M) * K,
+        w.ndim() > 2 ? matrix_stride(w) : 0,
+        scales.ndim() > 2 ? matrix_stride(scales) : 0,
+        fp_mode_code(mode_),
+        dt,
+        transpose_ ? 1 : 0,
+        enc.stream()));
+    return;
+  }
 
   const size_t ws_bytes = mlxrocm_gather_qmm_workspace_size(
       M, N, K, n_idx, n_experts, group_size_, bits_, dt, transpose_, right_sorted_);
@@ -252,9 +409,45 @@ void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
 void fast::Quantize::eval_gpu(
     const std::vector<array>& inputs,
     std::vector<array>& outputs) {
-  require_affine(mode_, "quantize");
   auto& s = stream();
   auto& enc = rocm::get_command_encoder(s);
+
+  if (mode_ != QuantizationMode::Affine) {
+    // fp_quantize: {w [, global_scale]} -> {wq, scales}; fp_dequantize:
+    // {wq, scales [, global_scale]} -> {w} (mlx/ops.cpp:5124-5128, 5393-5397)
+    const int mode = fp_mode_code(mode_);
+    if (dequantize_) {
+      no_global_scale(inputs.size() > 2, "dequantize");
+      array wq = ensure_row_contiguous(inputs[0], enc, s);
+      array scales = ensure_row_contiguous(inputs[1], enc, s);
+      array& w = outputs[0];
+      w.set_data(allocator::malloc(w.nbytes()));
+      rocm::check(mlxrocm_fp_dequantize(
+          rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+          rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+          rocm::gpu_ptr<void>(w, enc.stream()),
+          w.size(),
+          mode,
+          dtype_code(w.dtype(), "dequantize"),
+          enc.stream()));
+    } else {
+      no_global_scale(inputs.size() > 1, "quantize");
+      array w = ensure_row_contiguous(inputs[0], enc, s);
+      array& wq = outputs[0];
+      array& scales = outputs[1];
+      wq.set_data(allocator::malloc(wq.nbytes()));
+      scales.set_data(allocator::malloc(scales.nbytes()));
+      rocm::check(mlxrocm_fp_quantize(
+          rocm::gpu_ptr<void>(w, enc.stream()),
+          rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+          rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+          w.size(),
+          mode,
+          dtype_code(w.dtype(), "quantize"),
+          enc.stream()));
+    }
+    return;
+  }
 
   if (dequantize_) {
     array wq = ensure_row_contiguous(inputs[0], enc, s);

@@ -52,6 +52,13 @@ def _weights(shape, dtype, seed, spread=True):
 
 
 def _equal_bits(a: torch.Tensor, b: torch.Tensor) -> bool:
+    """Bit for bit, signed zeros and infinities included; a NaN (0 * inf where a
+    scale overflows float16) matches any NaN."""
+    nan_a, nan_b = torch.isnan(a), torch.isnan(b)
+    if not torch.equal(nan_a, nan_b):
+        return False
+    a = torch.where(nan_a, torch.zeros_like(a), a)
+    b = torch.where(nan_b, torch.zeros_like(b), b)
     view = {4: torch.int32, 2: torch.int16, 1: torch.uint8}[a.element_size()]
     return torch.equal(a.contiguous().view(view), b.contiguous().view(view))
 
@@ -88,9 +95,6 @@ def test_fp_dequantize_matches_oracle_bit_for_bit(fp_oracle, gpu, mode, dtype):
     got = mlx_amd.dequantize(wq.to(gpu), scales.to(gpu), mode=mode, dtype=dtype)
     want = fp_oracle.dequantize(wq, scales, mode, dtype)
     assert got.dtype == dtype and got.shape == want.shape
-    if mode == "mxfp8":
-        # e4m3 codes 0x7f / 0xff decode to 480: finite, so still comparable
-        pass
     assert _equal_bits(got.cpu(), want), (mode, dtype)
     # default output type of the fp modes is bfloat16 (mlx/ops.cpp:4749-4753)
     assert mlx_amd.dequantize(wq.to(gpu), scales.to(gpu), mode=mode).dtype == torch.bfloat16
@@ -149,7 +153,9 @@ def _check_product(got, x, wq, scales, mode, transpose, ref, dtype):
     if ref is not None:
         rerr = ((got.double() - ref.double()).abs() / mag).max().item()
         assert rerr <= REF_TOL[dtype], (mode, dtype, transpose, rerr)
-        # and the GPU result is the closer of the two to the exact product
+        if dtype == torch.float32:
+            return
+        # 16-bit types: the GPU result is the closer of the two to the exact product
         ours = (got.double() - exact).abs().mean().item()
         theirs = (ref.double() - exact).abs().mean().item()
         assert ours <= theirs * 1.05 + 1e-12, (mode, dtype, ours, theirs)
@@ -170,6 +176,46 @@ def test_fp_quantized_matmul(fp_oracle, gpu, mode, transpose, dtype):
         assert got.dtype == dtype and got.shape == (M, N)
         ref = fp_oracle.qmm(x, wq.cpu(), scales.cpu(), mode, transpose)
         _check_product(got.cpu(), x, wq.cpu(), scales.cpu(), mode, transpose, ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16), ids=str)
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_quantized_matmul_prefill_tiles(fp_oracle, gpu, mode, dtype):
+    """Rows of x from the cut-over to the matrix-core tile kernel on: ragged M
+    and N (partial tiles), several tile widths, every output against fp64 and a
+    band of rows against the CPU reference."""
+    for M, N, K, seed in ((12, 224, 64, 1), (77, 1000, 256, 2), (300, 96, 512, 3), (513, 2240, 1024, 4)):
+        g = torch.Generator().manual_seed(seed)
+        w = torch.randn((N, K), generator=g).to(dtype)
+        w[:, :32] *= 37.0  # groups of very different scale
+        x = torch.randn((M, K), generator=g).to(dtype)
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+        got = mlx_amd.quantized_matmul(x.to(gpu), wq, scales, mode=mode)
+        assert got.dtype == dtype and got.shape == (M, N)
+        _check_product(got.cpu(), x, wq.cpu(), scales.cpu(), mode, True, None, dtype)
+        rows = slice(max(0, M - 5), M)
+        ref = fp_oracle.qmm(x[rows], wq.cpu(), scales.cpu(), mode, True)
+        _check_product(got[rows].cpu(), x[rows], wq.cpu(), scales.cpu(), mode, True, ref, dtype)
+        # the streaming kernel (rows taken four at a time) agrees to fp32 rounding
+        few = mlx_amd.quantized_matmul(x[:4].to(gpu), wq, scales, mode=mode)
+        assert (few.float() - got[:4].float()).abs().max().item() <= \
+            2.0 ** -7 * got[:4].float().abs().max().item()
+
+
+def test_fp_qmm_workspace_contract(gpu):
+    from mlx_amd import _lib
+
+    lib = _lib.load()
+    need = lib.mlxrocm_fp_qmm_workspace_size(512, 1024, 256, 1, 0, _lib.MXFP4, _lib.BFLOAT16, 1)
+    assert need >= 1024 * (256 // 32) * 4
+    assert lib.mlxrocm_fp_qmm_workspace_size(1, 1024, 256, 1, 0, _lib.MXFP4, _lib.BFLOAT16, 1) == 0
+    assert lib.mlxrocm_fp_qmm_workspace_size(512, 1024, 256, 1, 0, _lib.MXFP4, _lib.FLOAT32, 1) == 0
+    assert lib.mlxrocm_fp_qmm_workspace_size(512, 1024, 256, 1, 0, _lib.MXFP4, _lib.BFLOAT16, 0) == 0
+    buf = torch.zeros(1 << 20, dtype=torch.uint8, device=gpu)
+    p = buf.data_ptr()
+    rc = lib.mlxrocm_fp_qmm(p, p, p, p, 512, 1024, 256, 1, 0, 0, 0, _lib.MXFP4, _lib.BFLOAT16, 1,
+                            None, 0, None)
+    assert rc == _lib.INVALID_ARGUMENT and "workspace" in _lib.last_error()
 
 
 @pytest.mark.parametrize("mode", MODES)
@@ -309,10 +355,10 @@ def test_fp_abi_rejects_bad_arguments(gpu):
     assert lib.mlxrocm_fp_quantize(p, p, p, 48, _lib.MXFP4, 0, None) == _lib.INVALID_ARGUMENT
     assert lib.mlxrocm_fp_quantize(p, p, p, 64, _lib.MXFP4, 7, None) == _lib.INVALID_ARGUMENT
     assert lib.mlxrocm_fp_dequantize(p, p, p, 40, _lib.NVFP4, 0, None) == _lib.INVALID_ARGUMENT
-    assert lib.mlxrocm_fp_qmm(p, p, p, p, 1, 8, 40, 1, 0, 0, 0, _lib.MXFP8, 0, 1, None) \
+    assert lib.mlxrocm_fp_qmm(p, p, p, p, 1, 8, 40, 1, 0, 0, 0, _lib.MXFP8, 0, 1, None, 0, None) \
         == _lib.INVALID_ARGUMENT
     assert "multiple of group_size" in _lib.last_error()
-    assert lib.mlxrocm_fp_qmm(None, p, p, p, 1, 8, 64, 1, 0, 0, 0, _lib.MXFP8, 0, 1, None) \
+    assert lib.mlxrocm_fp_qmm(None, p, p, p, 1, 8, 64, 1, 0, 0, 0, _lib.MXFP8, 0, 1, None, 0, None) \
         == _lib.INVALID_ARGUMENT
     # nothing to do
     assert lib.mlxrocm_fp_quantize(None, None, None, 0, _lib.MXFP4, 0, None) == _lib.OK
