@@ -475,6 +475,37 @@ def sweep(torch, mlx_amd, dev) -> list:
         else:
             add("f4", name, ms, flops=2.0 * M * n * k)
 
+    def qq_case(mode, M, n, k):
+        """qqmm: x quantized inside the call, then the product (MX modes from 16
+        rows on: both operands' codes on the block-scaled matrix instruction)."""
+        from mlx_amd import _lib
+        lib = _lib.load()
+        mcode = {"mxfp4": _lib.MXFP4, "mxfp8": _lib.MXFP8, "nvfp4": _lib.NVFP4}[mode]
+        q = mlx_amd.quantize(weights(n, k, bf16, std=1.0), mode=mode)
+        x = torch.randn((M, k), generator=g, dtype=torch.float32).to(bf16).to(dev)
+        out = torch.empty((M, n), dtype=bf16, device=dev)
+        ws_bytes = lib.mlxrocm_fp_qqmm_workspace_size(M, n, k, mcode, 2)
+        ws = torch.empty(max(int(ws_bytes), 256), dtype=torch.uint8, device=dev)
+
+        def step(i, stream):
+            rc = lib.mlxrocm_fp_qqmm(x.data_ptr(), q[0].data_ptr(), q[1].data_ptr(), out.data_ptr(),
+                                     M, n, k, mcode, 2, ws.data_ptr(), ws_bytes, stream)
+            if rc != 0:
+                raise RuntimeError(_lib.last_error())
+
+        launcher = Launcher(torch, step, 1, False)
+        launcher.run(10)
+        torch.cuda.synchronize()
+        first = hip_event_ms(lib, launcher, 10)
+        per_region = max(10, int(5.0 / max(first, 1e-3)))
+        ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
+        add("f4", f"qqmm {mode}: x bfloat16 [{M},{k}] W [{n},{k}] (x quantized in the call)", ms,
+            flops=2.0 * M * n * k)
+
+    for mode in ("mxfp8", "mxfp4", "nvfp4"):
+        for M in (512, 2048, 8192):
+            qq_case(mode, M, 14336, 4096)
+
     for mode in ("mxfp4", "mxfp8", "nvfp4"):
         bits = 8 if mode == "mxfp8" else 4
         gs = 16 if mode == "nvfp4" else 32
@@ -485,7 +516,7 @@ def sweep(torch, mlx_amd, dev) -> list:
         q = mlx_amd.quantize(w, mode=mode)
         ms = timed(lambda i: mlx_amd.dequantize(*q, mode=mode))
         add("f4", f"dequantize bfloat16 [14336,4096] {mode}", ms, nbytes=nb)
-        for M in (1, 4, 512):
+        for M in (1, 4, 512, 2048):
             fp_case(mode, M, 14336, 4096)
 
     # GGUF blocks -> affine triplet (load-time conversion of a [14336, 4096] tensor)

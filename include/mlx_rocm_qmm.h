@@ -208,6 +208,35 @@ int mlxrocm_fp_qmm(
     size_t workspace_bytes,
     mlxrocm_stream_t stream);
 
+/*
+ * qqmm with a quantized second operand (mlx/ops.cpp:4926-4990; CPU:
+ * QQMatmul::eval_cpu, mlx/backend/cpu/quantized.cpp:1322-1360, which takes one
+ * row of x): y = quantize_dequantize(x) . dequantize(w)^T.  x [M, K] and out
+ * [M, N] in dtype, w [N, K bits / 32], scales [N, K / group_size] bytes.  In the
+ * MX modes (mxfp4; mxfp8 for the 16-bit dtypes) with K a multiple of 128 and 16
+ * rows of x or more, x is quantized to codes by the rules of
+ * mlxrocm_fp_quantize_dequantize and both operands' codes are multiplied on the
+ * block-scaled matrix instruction (v_mfma_scale_f32_16x16x128_f8f6f4) -- the
+ * same real products, summed exactly for e2m1 codes and with about 17 bits
+ * below the largest product of a 128-code step for e4m3 codes; otherwise x is
+ * quantized and dequantized in dtype and takes the kernels of mlxrocm_fp_qmm.  workspace: mlxrocm_fp_qqmm_workspace_size bytes,
+ * 256-byte aligned, used only during the call.
+ */
+size_t mlxrocm_fp_qqmm_workspace_size(int M, int N, int K, int mode, int dtype);
+int mlxrocm_fp_qqmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int mode,
+    int dtype,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream);
+
 /* gather_qmm for the floating-point modes (mlx/ops.cpp:5553-5629 with
  * mode != "affine"; CPU: mlx/backend/cpu/quantized.cpp:806-900 fp_bs_qmm_dispatch_mode).
  * Arguments as mlxrocm_gather_qmm without biases; pair i multiplies

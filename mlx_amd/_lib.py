@@ -58,6 +58,8 @@ SIGNATURES = {
     "mlxrocm_fp_quantize_dequantize": (_i, [_p, _p, _sz, _i, _i, _p]),
     "mlxrocm_fp_qmm_workspace_size": (_sz, [_i] * 8),
     "mlxrocm_fp_qmm": (_i, [_p] * 4 + [_i] * 4 + [_i64] * 3 + [_i] * 3 + [_p, _sz, _p]),
+    "mlxrocm_fp_qqmm_workspace_size": (_sz, [_i] * 5),
+    "mlxrocm_fp_qqmm": (_i, [_p] * 4 + [_i] * 5 + [_p, _sz, _p]),
     "mlxrocm_fp_gather_qmm": (_i, [_p] * 6 + [_i] * 6 + [_i64] * 3 + [_i] * 3 + [_p]),
     "mlxrocm_qmm_kernel_name": (ctypes.c_char_p, [_i] * 8),
     "mlxrocm_qmm_plan": (_i, [_i] * 9 + [_sz, ctypes.c_char_p, _sz]),

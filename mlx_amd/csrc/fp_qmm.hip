@@ -568,7 +568,9 @@ bool aligned16(const void* p) {
 
 using namespace mlxrocm;
 
-extern "C" int mlxrocm_fp_qmm(
+namespace {
+
+int fp_qmm_entry(
     const void* x,
     const uint32_t* wq,
     const uint8_t* scales,
@@ -586,7 +588,6 @@ extern "C" int mlxrocm_fp_qmm(
     void* workspace,
     size_t workspace_bytes,
     mlxrocm_stream_t stream) {
-  mlxrocm::ApiRange api_range("mlxrocm_fp_qmm");
   int rc = fp_check("quantized_matmul", M, N, K, L, mode, dtype, transpose);
   if (rc != MLXROCM_OK) {
     return rc;
@@ -658,6 +659,128 @@ extern "C" int mlxrocm_fp_qmm(
     return reduce_k_splits(partial, out, static_cast<size_t>(M) * N, splits, dtype, s);
   }
   return fp_launch(a, mode, dtype, transpose != 0, s);
+}
+
+// From this many rows of x on, qqmm in the MX modes multiplies the codes of both
+// operands on the block-scaled matrix instruction; below, x is quantized and
+// dequantized in its own type and takes the kernels of quantized_matmul.
+constexpr int kQqNativeMinM = 16;
+
+// 4-bit codes: the instruction's sums are exact (products of two e2m1 numbers
+// have few bits), results equal the fp32-accumulated ones bit for bit on the
+// test shapes.  8-bit codes: inside a 128-code step the hardware aligns the
+// products to the largest and keeps about 17 bits below it (measured: errors of
+// 8e-6 of sum |x w|, against 1e-7 for fp32 accumulation) -- far below the
+// rounding of a 16-bit result, but visible in a float32 one, so float32 problems
+// stay on the fp32-accumulating kernels.
+bool qq_native(int M, int N, int K, int mode, int dtype) {
+  return M >= kQqNativeMinM && qq_mfma_supported(M, N, K, mode) &&
+      (mode == MLXROCM_MXFP4 || dtype != MLXROCM_FLOAT32);
+}
+
+size_t round256(size_t n) {
+  return (n + 255) / 256 * 256;
+}
+
+} // namespace
+
+extern "C" int mlxrocm_fp_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int L,
+    int64_t x_batch_stride,
+    int64_t w_batch_stride,
+    int64_t scales_batch_stride,
+    int mode,
+    int dtype,
+    int transpose,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_fp_qmm");
+  return fp_qmm_entry(
+      x, wq, scales, out, M, N, K, L, x_batch_stride, w_batch_stride, scales_batch_stride, mode,
+      dtype, transpose, workspace, workspace_bytes, stream);
+}
+
+extern "C" size_t mlxrocm_fp_qqmm_workspace_size(int M, int N, int K, int mode, int dtype) {
+  if (fp_check("qqmm", M, N, K, 1, mode, dtype, 1) != MLXROCM_OK ||
+      static_cast<int64_t>(M) * N == 0 || K == 0) {
+    return 0;
+  }
+  if (qq_native(M, N, K, mode, dtype)) {
+    const int bits = mode == MLXROCM_MXFP8 ? 8 : 4;
+    return round256(static_cast<size_t>(M) * K * bits / 8) + round256(static_cast<size_t>(M) * K / 32);
+  }
+  return round256(static_cast<size_t>(M) * K * dtype_size(dtype)) +
+      mlxrocm_fp_qmm_workspace_size(M, N, K, 1, 0, mode, dtype, 1);
+}
+
+extern "C" int mlxrocm_fp_qqmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int mode,
+    int dtype,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_fp_qqmm");
+  int rc = fp_check("qqmm", M, N, K, 1, mode, dtype, 1);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (static_cast<int64_t>(M) * N == 0) {
+    return MLXROCM_OK;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (K == 0) {
+    return launch_zero_fill(out, static_cast<size_t>(M) * N * dtype_size(dtype), s);
+  }
+  if (!x || !wq || !scales || !out) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[qqmm] null device pointer");
+  }
+  const size_t need = mlxrocm_fp_qqmm_workspace_size(M, N, K, mode, dtype);
+  if (workspace == nullptr || workspace_bytes < need ||
+      (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[qqmm] needs a 256-byte aligned workspace of %zu bytes (mlxrocm_fp_qqmm_workspace_size); "
+        "got %zu",
+        need, workspace_bytes);
+  }
+  if (!aligned16(x) || !aligned16(wq) || !aligned16(out)) {
+    return fail(MLXROCM_UNSUPPORTED, "[qqmm] operands must keep 16-byte alignment");
+  }
+  const size_t n_elems = static_cast<size_t>(M) * K;
+  if (qq_native(M, N, K, mode, dtype)) {
+    const int bits = mode == MLXROCM_MXFP8 ? 8 : 4;
+    void* codes = workspace;
+    uint8_t* xs = static_cast<uint8_t*>(workspace) + round256(n_elems * bits / 8);
+    rc = fp_quantize_activations(x, codes, xs, n_elems, mode, dtype, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    return launch_qq_mfma(codes, xs, wq, scales, out, M, N, K, mode, dtype, s);
+  }
+  // x_hat in the element type, then the product with the quantized w
+  rc = mlxrocm_fp_quantize_dequantize(x, workspace, n_elems, mode, dtype, stream);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  const size_t xhat_bytes = round256(n_elems * dtype_size(dtype));
+  return fp_qmm_entry(
+      workspace, wq, scales, out, M, N, K, 1, 0, 0, 0, mode, dtype, 1,
+      static_cast<char*>(workspace) + xhat_bytes, workspace_bytes - xhat_bytes, stream);
 }
 
 extern "C" size_t mlxrocm_fp_qmm_workspace_size(

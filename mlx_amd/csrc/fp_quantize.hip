@@ -221,9 +221,12 @@ __global__ __launch_bounds__(kFpBlock) void fp_dequantize_kernel(
 }
 
 // mlx/backend/cpu/quantized.cpp:1094-1128, fp32 arithmetic throughout.
-template <typename T, int GS, int BITS>
+// CODES: write the codes and the scale byte (wq, scales) instead of the
+// dequantized elements (out): the operand the block-scaled matrix instruction
+// multiplies as it is.
+template <typename T, int GS, int BITS, bool CODES = false>
 __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
-    const T* w, T* out, size_t n_units) {
+    const T* w, T* out, size_t n_units, uint8_t* wq = nullptr, uint8_t* scales = nullptr) {
   const size_t u = static_cast<size_t>(blockIdx.x) * kFpBlock + threadIdx.x;
   constexpr int kLanes = GS / 8;
   float v[8];
@@ -243,8 +246,10 @@ __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
   }
   m = group_max(m, kLanes);
   float scale = m / (BITS == 4 ? 6.0f : 448.0f);
+  uint32_t scale_byte;
   if constexpr (GS == 16) {
-    scale = from_fp8_bits(to_fp8_bits(scale));
+    scale_byte = to_fp8_bits(scale);
+    scale = from_fp8_bits(scale_byte);
   } else {
     // to_fp8_e8m0 (:1049-1061): round(log2(scale)) half away from zero, clamped;
     // log2(0) = -inf clamps to -127, which decodes to 2^-127
@@ -259,19 +264,46 @@ __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
     }
     const uint32_t s8 = static_cast<uint32_t>(n + 127);
     scale = __uint_as_float((s8 == 0 ? 0x40u : (s8 << 7)) << 16);
+    scale_byte = s8;
   }
   if (!live) {
     return;
   }
-  float o[8];
+  if constexpr (CODES) {
+    uint32_t lo = 0, hi = 0;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float w_el = scale == 0.0f ? 0.0f : v[i] / scale;
-    const float val = BITS == 8 ? from_fp8_bits(to_fp8_bits(w_el))
-                                : fp4_value(fp4_nearest_even(w_el));
-    o[i] = scale * val;
+    for (int i = 0; i < 8; ++i) {
+      const float w_el = scale == 0.0f ? 0.0f : v[i] / scale;
+      if constexpr (BITS == 8) {
+        const uint32_t c = to_fp8_bits(w_el);
+        if (i < 4) {
+          lo |= c << (8 * i);
+        } else {
+          hi |= c << (8 * (i - 4));
+        }
+      } else {
+        lo |= fp4_nearest_even(w_el) << (4 * i);
+      }
+    }
+    if constexpr (BITS == 8) {
+      reinterpret_cast<uint2*>(wq)[u] = make_uint2(lo, hi);
+    } else {
+      reinterpret_cast<uint32_t*>(wq)[u] = lo;
+    }
+    if (u % kLanes == 0) {
+      scales[u / kLanes] = static_cast<uint8_t>(scale_byte);
+    }
+  } else {
+    float o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float w_el = scale == 0.0f ? 0.0f : v[i] / scale;
+      const float val = BITS == 8 ? from_fp8_bits(to_fp8_bits(w_el))
+                                  : fp4_value(fp4_nearest_even(w_el));
+      o[i] = scale * val;
+    }
+    store8<T>(out + u * 8, o);
   }
-  store8<T>(out + u * 8, o);
 }
 
 int check_mode(const char* who, int mode, int dtype, size_t n_elems) {
@@ -383,6 +415,33 @@ extern "C" int mlxrocm_fp_dequantize(
     });
   });
 }
+
+namespace mlxrocm {
+
+// x -> codes and scale bytes by the rules of fp_quantize_dequantize (what qqmm
+// applies to its first operand).  n_elems a multiple of the group size.
+int fp_quantize_activations(
+    const void* x, void* codes, uint8_t* scales, size_t n_elems, int mode, int dtype, hipStream_t s) {
+  const size_t n_units = n_elems / 8;
+  const size_t blocks = (n_units + kFpBlock - 1) / kFpBlock;
+  if (blocks > 0x7fffffffull) {
+    return fail(MLXROCM_UNSUPPORTED, "[qqmm] %zu elements exceed the grid", n_elems);
+  }
+  MLXROCM_REHEARSE("fp_quantize_activations");
+  return dispatch_dtype(dtype, [&](auto tval) {
+    using T = decltype(tval);
+    return dispatch_mode(mode, [&](auto gval, auto bval) {
+      constexpr int G = decltype(gval)::value;
+      constexpr int B = decltype(bval)::value;
+      fp_quantize_dequantize_kernel<T, G, B, true><<<static_cast<unsigned>(blocks), kFpBlock, 0, s>>>(
+          static_cast<const T*>(x), nullptr, n_units, static_cast<uint8_t*>(codes), scales);
+      MLXROCM_HIP_TRY(hipGetLastError());
+      return static_cast<int>(MLXROCM_OK);
+    });
+  });
+}
+
+} // namespace mlxrocm
 
 extern "C" int mlxrocm_fp_quantize_dequantize(
     const void* x,

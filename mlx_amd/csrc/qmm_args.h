@@ -131,6 +131,25 @@ int fp_scale_image_for_qmm_t(
     hipStream_t s);
 int launch_qmm_mfma_fp(const QmmArgs& a, int mode, int dtype, int k_splits, hipStream_t s);
 
+// qqmm in the MX modes on the block-scaled matrix instruction (qq_mfma.hip):
+// x as codes and scale bytes (fp_quantize_activations, fp_quantize.hip) times
+// the quantized w, both [rows][K]; K % 128 == 0.
+bool qq_mfma_supported(int M, int N, int K, int mode);
+int launch_qq_mfma(
+    const void* xq,
+    const uint8_t* xs,
+    const uint32_t* wq,
+    const uint8_t* ws,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int mode,
+    int dtype,
+    hipStream_t s);
+int fp_quantize_activations(
+    const void* x, void* codes, uint8_t* scales, size_t n_elems, int mode, int dtype, hipStream_t s);
+
 bool qmv_wide_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);
 int launch_qmv_wide(const QmmArgs& a, int gs, int bits, int dtype, hipStream_t s);
 bool qmm_skinny_supported(const QmmArgs& a, int gs, int bits, int dtype, bool transpose);

@@ -492,28 +492,35 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
 
   // One slot: MFMA number m of a step of parity P and the side work assigned
   // to it.  `t` is the step, cur/nxt its LDS stages.
-#define QMM_SLOT(m, P)                                                           \
+// MM: the wavefront's 64 rows of the tile hold rows of x (below M).  A
+// wavefront whose rows all lie past M (a tile with fewer than 193 rows) takes
+// the slots without their matrix instruction and fragment reads: it still loads,
+// dequantizes and stores its share of W and joins the barriers, and leaves its
+// SIMD's matrix pipe to the wavefront beside it.
+#define QMM_SLOT(m, P, MM)                                                       \
   if constexpr ((m) < kNS) {                                                     \
     constexpr int s__ = (m) / (4 * NT);                                          \
     constexpr int t__ = ((m) % (4 * NT)) / 4;                                    \
     constexpr int b__ = (m) % 4;                                                 \
     constexpr int g__ = s__ * NT + t__;              /* W fragment number */     \
     constexpr int e__ = ((P) * 2 * NT + g__) % 4;    /* its ring entry */        \
-    acc[t__][b__] = mfma16<T>(afr[e__], bfr[s__][b__], acc[t__][b__]);           \
-    if constexpr (b__ == 3) {                                                    \
-      /* the ring entry just retired takes fragment g + 4 */                     \
-      if constexpr (g__ + 4 < 2 * NT) {                                          \
-        read_a(cur, (g__ + 4) / NT, (g__ + 4) % NT, e__);                        \
-      } else {                                                                   \
-        read_a(nxt, 0, g__ + 4 - 2 * NT, e__);                                   \
+    if constexpr (MM) {                                                          \
+      acc[t__][b__] = mfma16<T>(afr[e__], bfr[s__][b__], acc[t__][b__]);         \
+      if constexpr (b__ == 3) {                                                  \
+        /* the ring entry just retired takes fragment g + 4 */                   \
+        if constexpr (g__ + 4 < 2 * NT) {                                        \
+          read_a(cur, (g__ + 4) / NT, (g__ + 4) % NT, e__);                      \
+        } else {                                                                 \
+          read_a(nxt, 0, g__ + 4 - 2 * NT, e__);                                 \
+        }                                                                        \
       }                                                                          \
-    }                                                                            \
-    if constexpr (s__ == 0 && t__ >= NT - 4 && b__ == 1) {                       \
-      read_b(xs_cur, 1, t__ - (NT - 4));                                         \
-    }                                                                            \
-    if constexpr ((m) == kNS - 12 || (m) == kNS - 11 || (m) == kNS - 10 ||       \
-                  (m) == kNS - 8) {                                              \
-      read_b(xs_nxt, 0, (m) == kNS - 8 ? 3 : (m) - (kNS - 12));                  \
+      if constexpr (s__ == 0 && t__ >= NT - 4 && b__ == 1) {                     \
+        read_b(xs_cur, 1, t__ - (NT - 4));                                       \
+      }                                                                          \
+      if constexpr ((m) == kNS - 12 || (m) == kNS - 11 || (m) == kNS - 10 ||     \
+                    (m) == kNS - 8) {                                            \
+        read_b(xs_nxt, 0, (m) == kNS - 8 ? 3 : (m) - (kNS - 12));                \
+      }                                                                          \
     }                                                                            \
     if constexpr ((m) == 0) {                                                    \
       QMM_LOAD_W(k2);                                                            \
@@ -562,12 +569,12 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     __builtin_amdgcn_sched_barrier(0);                                           \
   }
 
-#define QMM_SLOTS8(m0, P)                                                        \
-  QMM_SLOT((m0) + 0, P) QMM_SLOT((m0) + 1, P) QMM_SLOT((m0) + 2, P)              \
-  QMM_SLOT((m0) + 3, P) QMM_SLOT((m0) + 4, P) QMM_SLOT((m0) + 5, P)              \
-  QMM_SLOT((m0) + 6, P) QMM_SLOT((m0) + 7, P)
+#define QMM_SLOTS8(m0, P, MM)                                                    \
+  QMM_SLOT((m0) + 0, P, MM) QMM_SLOT((m0) + 1, P, MM) QMM_SLOT((m0) + 2, P, MM)  \
+  QMM_SLOT((m0) + 3, P, MM) QMM_SLOT((m0) + 4, P, MM) QMM_SLOT((m0) + 5, P, MM)  \
+  QMM_SLOT((m0) + 6, P, MM) QMM_SLOT((m0) + 7, P, MM)
 
-#define QMM_STEP(tt, P)                                                          \
+#define QMM_STEP(tt, P, MM)                                                      \
   {                                                                              \
     const int cur = (P);                                                         \
     const int nxt = (P) ^ 1;                                                     \
@@ -587,8 +594,9 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
     ColDequant<T, (WN ? BITS : 4)> cdq;                                          \
     uint32_t dqv[16];                                                            \
     __builtin_amdgcn_sched_barrier(0);                                           \
-    QMM_SLOTS8(0, P) QMM_SLOTS8(8, P) QMM_SLOTS8(16, P) QMM_SLOTS8(24, P)        \
-    QMM_SLOTS8(32, P) QMM_SLOTS8(40, P) QMM_SLOTS8(48, P) QMM_SLOTS8(56, P)      \
+    QMM_SLOTS8(0, P, MM) QMM_SLOTS8(8, P, MM) QMM_SLOTS8(16, P, MM)              \
+    QMM_SLOTS8(24, P, MM) QMM_SLOTS8(32, P, MM) QMM_SLOTS8(40, P, MM)            \
+    QMM_SLOTS8(48, P, MM) QMM_SLOTS8(56, P, MM)                                  \
     /* the packed W fetched in slot 0 is older than the four x loads: it has    \
        had the whole step to arrive */                                          \
     asm volatile("s_waitcnt vmcnt(4)" ::: "memory");                             \
@@ -604,12 +612,24 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   }
 
   int t = 0;
-  for (; t + 1 < nk; t += 2) {
-    QMM_STEP(t, 0)
-    QMM_STEP(t + 1, 1)
-  }
-  if (t < nk) {
-    QMM_STEP(t, 0)
+  // uniform per wavefront: does any of its 64 rows lie below M
+  const bool has_rows = __builtin_amdgcn_readfirstlane(m0 + wm * 64 < M ? 1 : 0) != 0;
+  if (has_rows) {
+    for (; t + 1 < nk; t += 2) {
+      QMM_STEP(t, 0, true)
+      QMM_STEP(t + 1, 1, true)
+    }
+    if (t < nk) {
+      QMM_STEP(t, 0, true)
+    }
+  } else {
+    for (; t + 1 < nk; t += 2) {
+      QMM_STEP(t, 0, false)
+      QMM_STEP(t + 1, 1, false)
+    }
+    if (t < nk) {
+      QMM_STEP(t, 0, false)
+    }
   }
 #undef QMM_STEP
 #undef QMM_SLOTS8

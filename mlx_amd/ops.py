@@ -809,15 +809,20 @@ def qqmm(
     _require_gpu("qqmm", x, w, scales)
     lib = _lib.load()
     xc = _contiguous(x)
-    xhat = torch.empty_like(xc)
-    if xc.numel():
-        _lib.check(
-            lib.mlxrocm_fp_quantize_dequantize(
-                xc.data_ptr(), xhat.data_ptr(), xc.numel(), _MODE_CODE[mode],
-                _DTYPE_CODE[xc.dtype], _stream_ptr(xc),
-            )
+    wc = w if _last_two_dense(w) else _contiguous(w)
+    sc = scales if _last_two_dense(scales) else _contiguous(scales)
+    M, K = xc.shape
+    N = wc.shape[0]
+    code = _DTYPE_CODE[xc.dtype]
+    out = torch.empty((M, N), dtype=xc.dtype, device=xc.device)
+    ws_bytes = lib.mlxrocm_fp_qqmm_workspace_size(M, N, K, _MODE_CODE[mode], code)
+    ws = torch.empty(max(int(ws_bytes), 256), dtype=torch.uint8, device=xc.device)
+    _lib.check(
+        lib.mlxrocm_fp_qqmm(
+            xc.data_ptr(), wc.data_ptr(), sc.data_ptr(), out.data_ptr(), M, N, K,
+            _MODE_CODE[mode], code, ws.data_ptr(), ws_bytes, _stream_ptr(xc),
         )
-    out = quantized_matmul(xhat, w, scales, None, True, group_size, bits, mode)
+    )
     if len(in_shape) > 2:
         return out.reshape(in_shape[:-1] + (out.shape[-1],))
     if len(in_shape) == 1:

@@ -273,39 +273,26 @@ void QQMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
   }
 
   out.set_data(allocator::malloc(out.nbytes()));
-  array xhat(x.shape(), x.dtype(), nullptr, {});
-  xhat.set_data(allocator::malloc(xhat.nbytes()));
-  enc.add_temporary(xhat);
-  rocm::check(mlxrocm_fp_quantize_dequantize(
-      rocm::gpu_ptr<void>(x, enc.stream()),
-      rocm::gpu_ptr<void>(xhat, enc.stream()),
-      x.size(),
-      mode,
-      dt,
-      enc.stream()));
+  // x is quantized inside the call: to codes for the block-scaled matrix
+  // instruction (MX modes, 16 rows or more), else to x_hat in its own type
   const size_t ws_bytes =
-      mlxrocm_fp_qmm_workspace_size(static_cast<int>(rows), N, K, 1, 0, mode, dt, 1);
+      mlxrocm_fp_qqmm_workspace_size(static_cast<int>(rows), N, K, mode, dt);
   void* ws_ptr = nullptr;
   if (ws_bytes > 0) {
     array ws = workspace_array(ws_bytes);
     enc.add_temporary(ws);
     ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
   }
-  rocm::check(mlxrocm_fp_qmm(
-      rocm::gpu_ptr<void>(xhat, enc.stream()),
+  rocm::check(mlxrocm_fp_qqmm(
+      rocm::gpu_ptr<void>(x, enc.stream()),
       rocm::gpu_ptr<uint32_t>(w, enc.stream()),
       rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
       rocm::gpu_ptr<void>(out, enc.stream()),
       static_cast<int>(rows),
       N,
       K,
-      1,
-      0,
-      0,
-      0,
       mode,
       dt,
-      1,
       ws_ptr,
       ws_bytes,
       enc.stream()));

@@ -314,6 +314,41 @@ def test_qqmm(fp_oracle, gpu, mode):
     assert mlx_amd.qqmm(x.reshape(8, 8, K).to(gpu), wq, scales, mode=mode).shape == (8, 8, N)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("mode", ("mxfp8", "mxfp4"))
+def test_qqmm_on_the_block_scaled_matrix_instruction(fp_oracle, gpu, mode, dtype):
+    """16 rows of x or more in the MX modes: both operands' codes are multiplied
+    as they are.  Every output against the fp64 product of the two dequantized
+    operands (x by the oracle's quantize-dequantize, w by the definition of the
+    format); ragged M and N, one and many K steps, groups of very different
+    scale; the first rows also against the route that fewer rows take."""
+    half_ulp = {torch.float32: 2.0 ** -24, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    for M, N, K, seed in ((16, 128, 128, 1), (77, 200, 256, 2), (300, 1000, 1024, 3), (513, 136, 4096, 4)):
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn((M, K), generator=g)
+        x[:, 32:64] *= 50.0
+        x[1, :32] = 0.0
+        w = torch.randn((N, K), generator=g)
+        w[:, :32] *= 0.01
+        x, w = x.to(dtype), w.to(dtype)
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+        got = mlx_amd.qqmm(x.to(gpu), wq, scales, mode=mode)
+        assert got.shape == (M, N) and got.dtype == dtype
+        x_hat = fp_oracle.quantize_dequantize(x, mode).double()
+        w_hat = fp_qref.exact_fp_weights(wq.cpu(), scales.cpu(), mode)
+        want = x_hat @ w_hat.T
+        mag = x_hat.abs() @ w_hat.abs().T + 1e-30
+        err = ((got.cpu().double() - want).abs() / mag).max().item()
+        # e2m1 products are summed exactly by the instruction; for e4m3 it keeps
+        # about 17 bits below the largest product of a 128-code step (16-bit
+        # results only: float32 problems take the fp32-accumulating kernels)
+        acc_tol = 2e-6 if (mode == "mxfp4" or dtype == torch.float32) else 2e-5
+        assert err <= acc_tol + half_ulp, (mode, dtype, (M, N, K), err)
+        few = mlx_amd.qqmm(x[:8].to(gpu), wq, scales, mode=mode)  # x_hat in dtype, streaming kernel
+        ferr = ((few.cpu().double() - got[:8].cpu().double()).abs() / mag[:8]).max().item()
+        assert ferr <= 2 * acc_tol + 2 * half_ulp, (mode, dtype, (M, N, K), ferr)
+
+
 def test_fp_mode_layers(gpu):
     import mlx_amd.nn as qnn
 
