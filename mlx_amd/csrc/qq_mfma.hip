@@ -17,6 +17,8 @@
 // XOR-swizzled so that fragment reads hit every bank once.  Wavefront (wm, wn)
 // owns a 64 x 64 block: W fragments are the instruction's A operand, x
 // fragments its B operand, so a lane holds four consecutive n of one row m of y.
+#include <type_traits>
+
 #include "mfma_loads.h"
 #include "qmm_args.h"
 
@@ -25,27 +27,30 @@ namespace mlxrocm {
 namespace {
 
 typedef int qq_i32x8 __attribute__((ext_vector_type(8)));
+typedef int qq_i32x4 __attribute__((ext_vector_type(4)));
 typedef float qq_f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kQqBM = 256;
-constexpr int kQqBN = 128;
 constexpr int kQqBK = 128; // codes per step
 constexpr int kQqThreads = 512;
 
-template <int BITS>
+// NI: 16-column tiles per wavefront along n (4 or 8): the workgroup's tile is
+// 256 x 32 NI.  The wider tile halves the bytes fetched per flop; 8-bit codes
+// keep the narrow one, whose three stages are what LDS holds.
+template <int BITS, int NI>
 struct QqShape {
+  static constexpr int kBN = 32 * NI;
   static constexpr int kRowBytes = kQqBK * BITS / 8;          // 128 or 64
   static constexpr int kSlots = kRowBytes / 16;                // 16-byte pieces per row: 8 or 4
   static constexpr int kRowsPerDma = 1024 / kRowBytes;         // rows one wavefront load moves: 8 or 16
   static constexpr int kXTile = kQqBM * kRowBytes;             // bytes
-  static constexpr int kWTile = kQqBN * kRowBytes;
-  static constexpr int kScaleBytes = (kQqBM + kQqBN) * 4 + 512; // one dword per row, 2 KiB moved
+  static constexpr int kWTile = kBN * kRowBytes;
   static constexpr int kStage = kXTile + kWTile + 2048;
-  static constexpr int kStages = BITS == 8 ? 3 : 6;
+  static constexpr int kStages = BITS == 8 ? 3 : (NI == 8 ? 4 : 6);
   static constexpr int kXDma = kQqBM / kRowsPerDma / 8;         // per wavefront and step: 4 or 2
-  static constexpr int kWDma = kQqBN / kRowsPerDma / 8;         // 2 or 1
+  static constexpr int kWDma = kBN / kRowsPerDma / 8;           // 1, 2 or 4
   static constexpr int kLoads = kXDma + kWDma + 1;              // + the scale dwords
-  static_assert(kScaleBytes <= 2048 + 512, "scale area");
+  static_assert(kQqBM + kBN <= 512, "one scale dword per thread");
 };
 
 struct QqArgs {
@@ -67,9 +72,10 @@ __device__ __forceinline__ int qq_slot(int row, int piece) {
   }
 }
 
-template <typename TO, int BITS>
+template <typename TO, int BITS, int NI>
 __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
-  using S = QqShape<BITS>;
+  using S = QqShape<BITS, NI>;
+  constexpr int kQqBN = S::kBN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -154,9 +160,9 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
     QQ_DMA4(soff, sbase + static_cast<size_t>(tc) * 4, stage + S::kXTile + S::kWTile + wave * 256);
   };
 
-  qq_f32x4 acc[4][4]; // [n tile][m tile]
+  qq_f32x4 acc[NI][4]; // [n tile][m tile]
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < NI; ++i) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -169,55 +175,98 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
   const int fr = lane & 15; // row inside a 16-row fragment
   const int kb = lane >> 4; // which 32 codes of the step
 
-  constexpr int kAhead = S::kStages - 1;
+  // A fragment: the 32 codes a lane supplies (eight registers of 8-bit codes,
+  // four of 4-bit codes).  Scale bytes travel packed, four rows to a register;
+  // the instruction's op_sel picks the row's byte.
+  using Frag = std::conditional_t<BITS == 8, qq_i32x8, qq_i32x4>;
+  struct Frags {
+    Frag af[NI], bf[4];
+    int sa[NI / 4], sb;
+  };
+  auto fragment = [&](const uint8_t* row_base, int r) -> Frag {
+    const uint8_t* row = row_base + r * S::kRowBytes;
+    if constexpr (BITS == 8) {
+      // 8-bit operands: registers 0..3 of lane block kb hold codes 16 kb .. 16 kb + 15
+      // of the step, registers 4..7 codes 64 + 16 kb ..; the scale of the codes
+      // [32 b, 32 b + 32) is the one lane block b supplies
+      const uint4 v0 = *reinterpret_cast<const uint4*>(row + qq_slot<8>(r, kb) * 16);
+      const uint4 v1 = *reinterpret_cast<const uint4*>(row + qq_slot<8>(r, 4 + kb) * 16);
+      return qq_i32x8{(int)v0.x, (int)v0.y, (int)v0.z, (int)v0.w, (int)v1.x, (int)v1.y, (int)v1.z, (int)v1.w};
+    } else {
+      const uint4 v0 = *reinterpret_cast<const uint4*>(row + qq_slot<4>(r, kb) * 16);
+      return qq_i32x4{(int)v0.x, (int)v0.y, (int)v0.z, (int)v0.w};
+    }
+  };
+  auto operand = [](const Frag& f) -> qq_i32x8 {
+    if constexpr (BITS == 8) {
+      return f;
+    } else {
+      return qq_i32x8{f[0], f[1], f[2], f[3], 0, 0, 0, 0};
+    }
+  };
+  // byte kb of four rows' scale dwords, packed (row j in byte j)
+  auto pack_scales = [&](uint32_t d0, uint32_t d1, uint32_t d2, uint32_t d3) {
+    const int sh = 8 * kb;
+    return static_cast<int>(
+        ((d0 >> sh) & 0xffu) | (((d1 >> sh) & 0xffu) << 8) | (((d2 >> sh) & 0xffu) << 16) |
+        ((d3 >> sh) << 24));
+  };
+  // the fragments and scale bytes of step t, from its stage
+  auto read_step = [&](int t, Frags& f) {
+    const uint8_t* st = smem + (t % S::kStages) * S::kStage;
+    const uint32_t* sc = reinterpret_cast<const uint32_t*>(st + S::kXTile + S::kWTile);
+    const int xr0 = wm * 64 + fr; // x tile rows xr0 + 16 j
 #pragma unroll
-  for (int t = 0; t < kAhead; ++t) {
+    for (int j = 0; j < 4; ++j) {
+      f.bf[j] = fragment(st, xr0 + 16 * j);
+    }
+    f.sb = pack_scales(sc[xr0], sc[xr0 + 16], sc[xr0 + 32], sc[xr0 + 48]);
+    const int wr0 = wn * 16 * NI + fr; // W tile rows wr0 + 16 i
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      f.af[i] = fragment(st + S::kXTile, wr0 + 16 * i);
+    }
+#pragma unroll
+    for (int q = 0; q < NI / 4; ++q) {
+      const uint32_t* sw = sc + kQqBM + wr0 + 64 * q;
+      f.sa[q] = pack_scales(sw[0], sw[16], sw[32], sw[48]);
+    }
+  };
+  // cbsz / blgp: the operand formats (0 = e4m3, 4 = e2m1); op_sel: which byte of
+  // the scale registers
+#define QQ_MMA(i, j)                                                             \
+  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(                  \
+      operand(f.af[i]), operand(f.bf[j]), acc[i][j], BITS == 8 ? 0 : 4,          \
+      BITS == 8 ? 0 : 4, (i) % 4, f.sa[(i) / 4], (j), f.sb);
+#define QQ_MMA_ROW(i)                                                            \
+  if constexpr ((i) < NI) {                                                      \
+    QQ_MMA(i, 0) QQ_MMA(i, 1) QQ_MMA(i, 2) QQ_MMA(i, 3)                          \
+  }
+  auto multiply = [&](const Frags& f) {
+    QQ_MMA_ROW(0) QQ_MMA_ROW(1) QQ_MMA_ROW(2) QQ_MMA_ROW(3)
+    QQ_MMA_ROW(4) QQ_MMA_ROW(5) QQ_MMA_ROW(6) QQ_MMA_ROW(7)
+  };
+#undef QQ_MMA_ROW
+#undef QQ_MMA
+
+  // Steps 0 .. kStages - 2 are requested up front; iteration t waits for step t,
+  // asks for step t + kStages - 1 (into the stage that iteration t - 1 read) and
+  // multiplies step t.  (Reading the fragments one iteration ahead of their
+  // matrix instructions, from a second register set, changed nothing for the
+  // 4-bit kernel and cost the 8-bit one, with its three stages, a step of lead.)
+  constexpr int kS = S::kStages;
+#pragma unroll
+  for (int t = 0; t < kS - 1; ++t) {
     issue(t);
   }
   for (int t = 0; t < nk; ++t) {
-    // the loads of steps t + 1 .. t + kAhead - 1 may still be in flight
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * S::kLoads) : "memory");
+    // the loads of steps t + 1 .. t + kStages - 2 may still be in flight
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kS - 2) * S::kLoads) : "memory");
     __syncthreads(); // step t is in LDS for everyone; stage (t - 1) % kStages is free
-    issue(t + kAhead);
-    const uint8_t* st = smem + (t % S::kStages) * S::kStage;
-    const uint32_t* sc = reinterpret_cast<const uint32_t*>(st + S::kXTile + S::kWTile);
-    qq_i32x8 af[4], bf[4];
-    int sa[4], sb[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int wr = wn * 64 + 16 * i + fr; // W tile row
-      const int xr = wm * 64 + 16 * i + fr; // x tile row
-      const uint8_t* wrow = st + S::kXTile + wr * S::kRowBytes;
-      const uint8_t* xrow = st + xr * S::kRowBytes;
-      if constexpr (BITS == 8) {
-        // 8-bit operands: registers 0..3 of lane block kb hold codes 16 kb .. 16 kb + 15
-        // of the step, registers 4..7 codes 64 + 16 kb ..; the scale of the codes
-        // [32 b, 32 b + 32) is the one lane block b supplies
-        const uint4 w0 = *reinterpret_cast<const uint4*>(wrow + qq_slot<8>(wr, kb) * 16);
-        const uint4 w1 = *reinterpret_cast<const uint4*>(wrow + qq_slot<8>(wr, 4 + kb) * 16);
-        const uint4 x0 = *reinterpret_cast<const uint4*>(xrow + qq_slot<8>(xr, kb) * 16);
-        const uint4 x1 = *reinterpret_cast<const uint4*>(xrow + qq_slot<8>(xr, 4 + kb) * 16);
-        af[i] = qq_i32x8{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
-        bf[i] = qq_i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
-      } else {
-        const uint4 w0 = *reinterpret_cast<const uint4*>(wrow + qq_slot<4>(wr, kb) * 16);
-        const uint4 x0 = *reinterpret_cast<const uint4*>(xrow + qq_slot<4>(xr, kb) * 16);
-        af[i] = qq_i32x8{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, 0, 0, 0, 0};
-        bf[i] = qq_i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, 0, 0, 0, 0};
-      }
-      // the row's four scale bytes of this step; this lane's block is byte kb
-      sa[i] = static_cast<int>((sc[kQqBM + wr] >> (8 * kb)) & 0xffu);
-      sb[i] = static_cast<int>((sc[xr] >> (8 * kb)) & 0xffu);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // cbsz / blgp: the operand formats (0 = e4m3, 4 = e2m1)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-            af[i], bf[j], acc[i][j], BITS == 8 ? 0 : 4, BITS == 8 ? 0 : 4, 0, sa[i], 0, sb[j]);
-      }
-    }
+    issue(t + kS - 1);
+    Frags f;
+    read_step(t, f);
+    multiply(f);
   }
   // the clamped extra loads must have landed before the workgroup's LDS is given up
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -236,8 +285,8 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
       continue;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + wn * 64 + 16 * i + 4 * quad;
+    for (int i = 0; i < NI; ++i) {
+      const int n = n0 + wn * 16 * NI + 16 * i + 4 * quad;
       if (n >= N) {
         continue;
       }
@@ -263,16 +312,17 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
   }
 }
 
-template <typename TO, int BITS>
+template <typename TO, int BITS, int NI>
 int launch_qq(const QqArgs& a, hipStream_t s) {
-  using S = QqShape<BITS>;
+  using S = QqShape<BITS, NI>;
+  constexpr int kQqBN = S::kBN;
   constexpr size_t smem = static_cast<size_t>(S::kStages) * S::kStage;
   static_assert(smem <= 160 * 1024, "LDS");
   const dim3 grid((a.N + kQqBN - 1) / kQqBN, (a.M + kQqBM - 1) / kQqBM, 1);
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qqmm] M=%d exceeds the grid", a.M);
   }
-  auto kern = qq_mfma_kernel<TO, BITS>;
+  auto kern = qq_mfma_kernel<TO, BITS, NI>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -323,9 +373,14 @@ int launch_qq_mfma(
   return dispatch_dtype(dtype, [&](auto tval) {
     using T = decltype(tval);
     if (mode == MLXROCM_MXFP8) {
-      return launch_qq<T, 8>(a, s);
+      return launch_qq<T, 8, 4>(a, s);
     }
-    return launch_qq<T, 4>(a, s);
+    // the wide tile where it still fills the chip
+    const long wide = static_cast<long>((M + kQqBM - 1) / kQqBM) * ((N + 255) / 256);
+    if (wide >= compute_units()) {
+      return launch_qq<T, 4, 8>(a, s);
+    }
+    return launch_qq<T, 4, 4>(a, s);
   });
 }
 
