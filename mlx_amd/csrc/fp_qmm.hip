@@ -252,12 +252,20 @@ constexpr int kFp16Waves = 4;
 
 // 16-bit element types, K % (128 / BITS) == 0.  MB rows of x per pass (1, 2 or
 // 4), RPW rows of w per wavefront.
-template <typename T, int GS, int BITS, int MB, int RPW>
+// XL: the workgroup's four wavefronts work on the same codes of different rows of
+// W, so the step's slice of x (MB rows x 64 lanes x kCodes elements) is fetched
+// once per workgroup into LDS -- piece j of lane l at ((m P + j) 64 + l) 16 bytes,
+// so that 16-byte reads of neighbouring lanes hit every bank once -- instead of
+// once per wavefront from the caches: with four rows of x those re-reads were
+// four times the bytes of the weights and set the kernel's time.
+template <typename T, int GS, int BITS, int MB, int RPW, bool XL = false>
 __global__ __launch_bounds__(64 * kFp16Waves) void fp_qmv16_kernel(const QmmArgs a) {
   constexpr int kCodes = 128 / BITS; // codes per lane and step: 32 or 16
   constexpr int kPairs = kCodes / 2;
+  constexpr int kPieces = kPairs / 4; // 16-byte pieces of x per lane, row and step
   constexpr int kGroups = kCodes / GS > 0 ? kCodes / GS : 1;
   constexpr int kPairsPerGroup = kPairs / kGroups;
+  __shared__ __attribute__((aligned(16))) uint4 xs[XL ? MB * kPieces * 64 : 1];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const FpProblem p = fp_resolve(a, blockIdx.z, sizeof(T));
@@ -265,8 +273,10 @@ __global__ __launch_bounds__(64 * kFp16Waves) void fp_qmv16_kernel(const QmmArgs
   const int N = a.N;
   const int m0 = blockIdx.y * MB;
   const int n0 = (blockIdx.x * kFp16Waves + wave) * RPW;
-  if (n0 >= N) {
-    return;
+  if constexpr (!XL) {
+    if (n0 >= N) {
+      return;
+    }
   }
   const size_t row_bytes = static_cast<size_t>(K) * BITS / 8;
   const int groups = K / GS;
@@ -288,30 +298,67 @@ __global__ __launch_bounds__(64 * kFp16Waves) void fp_qmv16_kernel(const QmmArgs
     wrow[r] = p.w + static_cast<size_t>(n) * row_bytes;
     srow[r] = p.scales + static_cast<size_t>(n) * groups;
   }
-  for (int k0 = lane * kCodes; k0 < K; k0 += 64 * kCodes) {
+  // every lane takes every step (the staged form has barriers inside): a lane
+  // whose codes lie past K multiplies zero codes
+  for (int kbase = 0; kbase < K; kbase += 64 * kCodes) {
+    const int k0 = kbase + lane * kCodes;
+    const bool live = k0 < K;
+    if constexpr (!XL) {
+      if (!live) {
+        break; // no barriers here, and the lanes past K stay past K
+      }
+    }
     uint4 wv[RPW];
     uint32_t sb[RPW][kGroups];
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
-      wv[r] = load_once(wrow[r] + static_cast<size_t>(k0) * BITS / 8);
+      wv[r] = live ? load_once(wrow[r] + static_cast<size_t>(k0) * BITS / 8) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int g = 0; g < kGroups; ++g) {
-        sb[r][g] = srow[r][k0 / GS + g];
+        sb[r][g] = live ? srow[r][k0 / GS + g] : 0x7fu;
       }
     }
     // this lane's slice of the rows of x, as pairs
     uint32_t xr[MB][kPairs];
+    if constexpr (XL) {
+      __syncthreads(); // the previous step's slice has been read
+      // the slice is MB rows of 64 kPieces pieces; thread t takes pieces t, t + 256, ..
+      for (int i = threadIdx.x; i < MB * 64 * kPieces; i += 64 * kFp16Waves) {
+        const int m = i / (64 * kPieces);
+        const int piece = i % (64 * kPieces); // along k: lane piece / kPieces, its piece % kPieces
+        const int row = m0 + m < a.M ? m0 + m : a.M - 1;
+        const int k = kbase + piece * 8;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (k < K) {
+          v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(row) * K + k);
+        }
+        xs[(m * kPieces + piece % kPieces) * 64 + piece / kPieces] = v;
+      }
+      __syncthreads();
 #pragma unroll
-    for (int m = 0; m < MB; ++m) {
-      const int row = m0 + m < a.M ? m0 + m : a.M - 1;
-      const uint4* src = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row) * K + k0);
+      for (int m = 0; m < MB; ++m) {
 #pragma unroll
-      for (int j = 0; j < kPairs / 4; ++j) {
-        const uint4 v = src[j];
-        xr[m][4 * j + 0] = v.x;
-        xr[m][4 * j + 1] = v.y;
-        xr[m][4 * j + 2] = v.z;
-        xr[m][4 * j + 3] = v.w;
+        for (int j = 0; j < kPieces; ++j) {
+          const uint4 v = xs[(m * kPieces + j) * 64 + lane];
+          xr[m][4 * j + 0] = v.x;
+          xr[m][4 * j + 1] = v.y;
+          xr[m][4 * j + 2] = v.z;
+          xr[m][4 * j + 3] = v.w;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+        const int row = m0 + m < a.M ? m0 + m : a.M - 1;
+        const uint4* src = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row) * K + k0);
+#pragma unroll
+        for (int j = 0; j < kPieces; ++j) {
+          const uint4 v = src[j];
+          xr[m][4 * j + 0] = v.x;
+          xr[m][4 * j + 1] = v.y;
+          xr[m][4 * j + 2] = v.z;
+          xr[m][4 * j + 3] = v.w;
+        }
       }
     }
 #pragma unroll
@@ -482,7 +529,7 @@ int fp_check(const char* who, int M, int N, int K, int L, int mode, int dtype, i
 // From this many rows of x on, 16-bit problems with transpose=true run on the
 // matrix-core tile kernel (one pass over W, K split into ranges while the tiles
 // do not fill the chip) instead of one streaming pass per four rows.  bf16
-// [M, 4096] x [14336, 4096], mxfp4 / mxfp8 / nvfp4: streaming 43 / 36 / 36 us at
+// [M, 4096] x [14336, 4096], mxfp4 / mxfp8 / nvfp4: streaming 30 / 35 / 35 us at
 // 8 rows (two passes); the tile kernel with its scale pre-pass 37 / 39 / 40 us at
 // 9 rows, 39 / 41 / 43 at 64, 70 / 73 / 75 at 512.
 constexpr int kFpTileMinM = 9;
@@ -528,17 +575,21 @@ int fp_launch(const QmmArgs& a, int mode, int dtype, bool transpose, hipStream_t
         fp_qmm_n_kernel<T, G, B><<<grid, 256, 0, s>>>(a);
       } else if (a.K % (128 / B) == 0 && !std::is_same_v<T, float>) {
         if constexpr (!std::is_same_v<T, float>) {
-          constexpr int kRows = 2; // rows of w per wavefront
+          // Two rows of w per wavefront: with four or eight, measured at
+          // [14336, 4096], 2..8 rows of x took the same time or longer (fewer
+          // wavefronts); what sets the time with several rows of x is the rate of
+          // v_dot2 (a quarter of the plain vector rate), not the bytes.
+          constexpr int kRows = 2;
           const int mb = a.M == 1 ? 1 : (a.M == 2 ? 2 : 4);
           MLXROCM_REHEARSE("fp_qmv16(mb=%d)", mb);
           const int rows_per_wg = kFp16Waves * kRows;
           const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, (a.M + mb - 1) / mb, a.L);
           if (mb == 1) {
-            fp_qmv16_kernel<T, G, B, 1, kRows><<<grid, 64 * kFp16Waves, 0, s>>>(a);
+            fp_qmv16_kernel<T, G, B, 1, kRows, false><<<grid, 64 * kFp16Waves, 0, s>>>(a);
           } else if (mb == 2) {
-            fp_qmv16_kernel<T, G, B, 2, kRows><<<grid, 64 * kFp16Waves, 0, s>>>(a);
+            fp_qmv16_kernel<T, G, B, 2, kRows, true><<<grid, 64 * kFp16Waves, 0, s>>>(a);
           } else {
-            fp_qmv16_kernel<T, G, B, 4, kRows><<<grid, 64 * kFp16Waves, 0, s>>>(a);
+            fp_qmv16_kernel<T, G, B, 4, kRows, true><<<grid, 64 * kFp16Waves, 0, s>>>(a);
           }
         }
       } else if (a.K % (128 / B) == 0) {

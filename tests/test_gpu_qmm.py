@@ -43,15 +43,17 @@ def _check_qmm(oracle, gpu, x, w, gs, bits, transpose=True, rows=None, quantized
     c = 1e-5 if x.dtype == torch.float32 else 2e-2
     bare = c * math.sqrt(K) * x_absmax * w_absmax  # the stated bound
     tol_ref = bare
+    discount = 0.0
     if x.dtype != torch.float32:
         # The x86 CPU reference accumulates 16-bit types in the element type
         # (cpu/quantized.cpp:177-206); at K >= 4096 its own distance from the
         # exact product already exceeds the bound, so that measured distance is
         # discounted.  The fp64 check above is the strict one.
-        tol_ref += float((ref - exact).abs().max())
+        discount = float((ref - exact).abs().max())
+        tol_ref += discount
     print(f"qmm M={x.shape[0]} K={K} b{bits} g{gs} {x.dtype}: |gpu-oracle|={err_ref:.3e} "
-          f"bare bound={bare:.3e} (margin {bare - err_ref:+.3e}); |gpu-fp64|={err_exact:.3e} "
-          f"bound={tol_exact:.3e}")
+          f"bare bound={bare:.3e} (margin {bare - err_ref:+.3e}) |oracle-fp64|={discount:.3e}; "
+          f"|gpu-fp64|={err_exact:.3e} bound={tol_exact:.3e}")
     assert err_ref <= tol_ref, f"vs oracle: {err_ref} > {tol_ref}"
     return got.cpu()
 
