@@ -256,6 +256,87 @@ def test_fp_quantized_matmul_batched(fp_oracle, gpu, mode):
     assert z.shape == (0, 64)
 
 
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_quantized_matmul_batched_prefill_and_edges(fp_oracle, gpu, mode):
+    """A stack of weights with enough rows of x for the tile kernel (one scale
+    image per batch entry), a broadcast weight through the C ABI (stride 0), and
+    the empty cases: no rows, no columns, K == 0 (zeros)."""
+    from mlx_amd import _lib
+    from mlx_amd.ops import _MODE_CODE
+
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(17)
+    L, M, N, K = 3, 40, 96, 256
+    w = torch.randn((L, N, K), generator=g).to(dtype)
+    x = torch.randn((L, M, K), generator=g).to(dtype)
+    wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+    got = mlx_amd.quantized_matmul(x.to(gpu), wq, scales, mode=mode)
+    assert got.shape == (L, M, N)
+    for l in range(L):
+        _check_product(got[l].cpu(), x[l], wq[l].cpu(), scales[l].cpu(), mode, True, None, dtype)
+    # one weight for every batch entry, batch kept (stride 0) instead of folded
+    lib = _lib.load()
+    xg = x.to(gpu).contiguous()
+    out = torch.empty((L, M, N), dtype=dtype, device=gpu)
+    ws_bytes = lib.mlxrocm_fp_qmm_workspace_size(M, N, K, L, 0, _MODE_CODE[mode], _lib.BFLOAT16, 1)
+    ws = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=gpu)
+    _lib.check(lib.mlxrocm_fp_qmm(
+        xg.data_ptr(), wq[1].contiguous().data_ptr(), scales[1].contiguous().data_ptr(),
+        out.data_ptr(), M, N, K, L, M * K, 0, 0, _MODE_CODE[mode], _lib.BFLOAT16, 1,
+        ws.data_ptr(), ws_bytes, torch.cuda.current_stream().cuda_stream))
+    for l in range(L):
+        _check_product(out[l].cpu(), x[l], wq[1].cpu(), scales[1].cpu(), mode, True, None, dtype)
+    # empty shapes
+    assert mlx_amd.quantized_matmul(xg[0, :0], wq[0], scales[0], mode=mode).shape == (0, N)
+    gs = fp_qref.GROUP_SIZE[mode]
+    bits = fp_qref.BITS[mode]
+    wq0 = torch.zeros((N, 0), dtype=torch.uint32, device=gpu)
+    sc0 = torch.zeros((N, 0), dtype=torch.uint8, device=gpu)
+    y0 = mlx_amd.quantized_matmul(torch.zeros((4, 0), dtype=dtype, device=gpu), wq0, sc0, mode=mode)
+    assert y0.shape == (4, N) and float(y0.abs().max()) == 0.0
+    assert (K * bits) % 32 == 0 and K % gs == 0
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_gather_qmm_many_pairs_bad_indices_and_no_pairs(fp_oracle, gpu, mode):
+    """70,000 pairs (more than one launch's grid depth), a pair whose index is out
+    of range (zeros, as the affine path), and an empty index list."""
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(23)
+    E, N, K = 5, 32, 64
+    w = torch.randn((E, N, K), generator=g).to(dtype)
+    x = torch.randn((7, 1, K), generator=g).to(dtype)
+    wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode)
+    n_pairs = 70000
+    lhs = torch.randint(0, 7, (n_pairs,), generator=g, dtype=torch.int32)
+    rhs = torch.randint(0, E, (n_pairs,), generator=g, dtype=torch.int32)
+    got = mlx_amd.gather_qmm(x.to(gpu), wq, scales, None, lhs.to(gpu), rhs.to(gpu), mode=mode)
+    assert got.shape == (n_pairs, 1, N)
+    w_hat = fp_qref.exact_fp_weights(wq.cpu(), scales.cpu(), mode)  # [E, N, K]
+    want = torch.einsum("pk,pnk->pn", x[lhs.long(), 0].double(), w_hat[rhs.long()])
+    mag = torch.einsum("pk,pnk->pn", x[lhs.long(), 0].double().abs(), w_hat[rhs.long()].abs()) + 1e-30
+    err = ((got[:, 0].cpu().double() - want).abs() / mag).max().item()
+    assert err <= 1e-3 + 2.0 ** -11, (mode, err)
+    # through the C ABI: an out-of-range expert index yields zeros for that pair
+    from mlx_amd import _lib
+    from mlx_amd.ops import _MODE_CODE
+
+    lib = _lib.load()
+    lhs_u = torch.tensor([0, 1, 2], dtype=torch.int32, device=gpu).view(torch.uint32)
+    rhs_u = torch.tensor([1, E, 3], dtype=torch.int32, device=gpu).view(torch.uint32)
+    out = torch.full((3, 1, N), 7.0, dtype=dtype, device=gpu)
+    xg = x.to(gpu).contiguous()
+    _lib.check(lib.mlxrocm_fp_gather_qmm(
+        xg.data_ptr(), wq.data_ptr(), scales.data_ptr(), lhs_u.data_ptr(), rhs_u.data_ptr(),
+        out.data_ptr(), 1, N, K, 3, 7, E, K, wq.stride(0), scales.stride(0), _MODE_CODE[mode],
+        _lib.FLOAT16, 1, torch.cuda.current_stream().cuda_stream))
+    assert float(out[1].abs().max()) == 0.0
+    assert float(out[0].abs().max()) > 0.0 and float(out[2].abs().max()) > 0.0
+    # no pairs
+    empty = torch.zeros((0,), dtype=torch.int32, device=gpu)
+    assert mlx_amd.gather_qmm(xg, wq, scales, None, empty, empty, mode=mode).shape == (0, 1, N)
+
+
 @pytest.mark.parametrize("transpose", (True, False))
 @pytest.mark.parametrize("mode", MODES)
 def test_fp_gather_qmm(fp_oracle, gpu, mode, transpose):
