@@ -29,28 +29,44 @@ namespace {
 typedef int qq_i32x8 __attribute__((ext_vector_type(8)));
 typedef int qq_i32x4 __attribute__((ext_vector_type(4)));
 typedef float qq_f32x4 __attribute__((ext_vector_type(4)));
+typedef float qq_f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kQqBM = 256;
 constexpr int kQqBK = 128; // codes per step
-constexpr int kQqThreads = 512;
 
-// NI: 16-column tiles per wavefront along n (4 or 8): the workgroup's tile is
-// 256 x 32 NI.  The wider tile halves the bytes fetched per flop; 8-bit codes
-// keep the narrow one, whose three stages are what LDS holds.
-template <int BITS, int NI>
+// Shape of a workgroup: WM x WN wavefronts, each with MI x NI tiles of 16 x 16
+// (m x n).
+//   <8, 4, 4, 4, 2>: 256 x 128, eight wavefronts  (8-bit codes: three stages fit)
+//   <4, 4, 8, 4, 2>: 256 x 256, eight wavefronts  (4-bit codes, enough tiles)
+//   <4, 4, 4, 4, 2>: 256 x 128                    (4-bit codes, few tiles)
+// What the shapes trade is bytes fetched per flop: measured at [8192, 4096] x
+// [14336, 4096], 4-bit, the 256 x 256 tile runs at 2.5 PFLOP/s and the 256 x 128
+// tile at 2.0 -- both 4.7-4.8 TB/s of global -> LDS traffic, which is what this
+// loop is bound by (the matrix pipe alone does 6.9).  Four wavefronts of
+// 128 x 128 (one per SIMD, 256 accumulators in AGPRs, fewer LDS bytes per flop)
+// fetch the same bytes and were slower (2.3).
+template <int BITS, int MI, int NI, int WM, int WN>
 struct QqShape {
-  static constexpr int kBN = 32 * NI;
+  static constexpr int kThreads = 64 * WM * WN;
+  static constexpr int kWaves = WM * WN;
+  static constexpr int kBM = 16 * MI * WM;
+  static constexpr int kBN = 16 * NI * WN;
   static constexpr int kRowBytes = kQqBK * BITS / 8;          // 128 or 64
   static constexpr int kSlots = kRowBytes / 16;                // 16-byte pieces per row: 8 or 4
   static constexpr int kRowsPerDma = 1024 / kRowBytes;         // rows one wavefront load moves: 8 or 16
-  static constexpr int kXTile = kQqBM * kRowBytes;             // bytes
+  static constexpr int kXTile = kBM * kRowBytes;               // bytes
   static constexpr int kWTile = kBN * kRowBytes;
-  static constexpr int kStage = kXTile + kWTile + 2048;
-  static constexpr int kStages = BITS == 8 ? 3 : (NI == 8 ? 4 : 6);
-  static constexpr int kXDma = kQqBM / kRowsPerDma / 8;         // per wavefront and step: 4 or 2
-  static constexpr int kWDma = kBN / kRowsPerDma / 8;           // 1, 2 or 4
-  static constexpr int kLoads = kXDma + kWDma + 1;              // + the scale dwords
-  static_assert(kQqBM + kBN <= 512, "one scale dword per thread");
+  // one scale dword per tile row, x rows first, padded to whole wavefront loads
+  static constexpr int kSDma = (kBM + kBN + kThreads - 1) / kThreads; // per wavefront and step
+  static constexpr int kScaleBytes = kSDma * kThreads * 4;
+  static constexpr int kStage = kXTile + kWTile + kScaleBytes;
+  static constexpr int kStages = (160 * 1024) / kStage > 6 ? 6 : (160 * 1024) / kStage;
+  static constexpr int kXDma = kBM / kRowsPerDma / kWaves;     // per wavefront and step
+  static constexpr int kWDma = kBN / kRowsPerDma / kWaves;
+  static constexpr int kLoads = kXDma + kWDma + kSDma;
+  static_assert(kBM % 64 == 0 && kBN % 64 == 0, "a wavefront's scale load stays on one operand");
+  static_assert(kBM % (kRowsPerDma * kWaves) == 0 && kBN % (kRowsPerDma * kWaves) == 0, "DMA split");
+  static_assert(kStages >= 3, "the loop needs three stages");
+  static_assert(MI % 4 == 0 && NI % 4 == 0, "scale bytes travel four to a register");
 };
 
 struct QqArgs {
@@ -72,19 +88,26 @@ __device__ __forceinline__ int qq_slot(int row, int piece) {
   }
 }
 
-template <typename TO, int BITS, int NI>
-__global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
-  using S = QqShape<BITS, NI>;
-  constexpr int kQqBN = S::kBN;
+// BIG (4-bit codes): 32 x 32 x 64 instructions instead of 16 x 16 x 128.  With
+// nothing but matrix instructions in a loop this GPU runs e2m1 operands at
+// 3.97 PFLOP/s in the 16 x 16 x 128 form -- the rate of e4m3 operands, 3.94 --
+// and at 6.9 PFLOP/s in the 32 x 32 x 64 form (e4m3: 3.8): only the larger form
+// has the doubled 4-bit rate.
+template <typename TO, int BITS, int MI, int NI, int WM, int WN, bool BIG = false>
+__global__ __launch_bounds__(64 * WM * WN) void qq_mfma_kernel(const QqArgs a) {
+  static_assert(!BIG || BITS == 4, "the 32 x 32 x 64 form pays for 4-bit codes only");
+  using S = QqShape<BITS, MI, NI, WM, WN>;
+  constexpr int kBM = S::kBM;
+  constexpr int kBN = S::kBN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wn = wave & 1;
-  const int wm = wave >> 1;
+  const int wn = wave % WN;
+  const int wm = wave / WN;
   const int M = a.M, N = a.N, K = a.K;
-  const int n0 = blockIdx.x * kQqBN;
-  const int m0 = blockIdx.y * kQqBM;
+  const int n0 = blockIdx.x * kBN;
+  const int m0 = blockIdx.y * kBM;
   const int nk = K / kQqBK;
   const uint32_t row_bytes = static_cast<uint32_t>(K) * BITS / 8;
   const uint32_t srow_bytes = static_cast<uint32_t>(K) / 32;
@@ -94,7 +117,7 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
   // the logical piece that belongs there.
   const int drow = lane / S::kSlots;
   const int dslot = lane % S::kSlots;
-  uint32_t xoff[S::kXDma], woff[S::kWDma];
+  uint32_t xoff[S::kXDma], woff[S::kWDma], soff[S::kSDma];
 #pragma unroll
   for (int j = 0; j < S::kXDma; ++j) {
     const int r = (wave * S::kXDma + j) * S::kRowsPerDma + drow; // tile row
@@ -107,20 +130,23 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
     const int n = n0 + r < N ? n0 + r : N - 1;
     woff[j] = static_cast<uint32_t>(n) * row_bytes + qq_slot<BITS>(r, dslot) * 16;
   }
-  // scale dwords: thread t < 256 fetches x row t's, t < 384 w row t - 256's, the
-  // rest repeat the last w row (same value, a place nobody reads)
-  uint32_t soff;
-  const uint8_t* sbase;
-  if (tid < kQqBM) {
-    const int m = m0 + tid < M ? m0 + tid : M - 1;
-    soff = static_cast<uint32_t>(m) * srow_bytes;
-  } else {
-    const int r = tid - kQqBM < kQqBN ? tid - kQqBM : kQqBN - 1;
-    const int n = n0 + r < N ? n0 + r : N - 1;
-    soff = static_cast<uint32_t>(n) * srow_bytes;
+  // scale dwords: load j of wavefront w fills dwords (j kWaves + w) 64 .. + 63 of
+  // the scale area; dword d < kBM is x row d's, d < kBM + kBN w row d - kBM's, the
+  // rest repeat the last w row (a place nobody reads).  Which operand a load
+  // reads is uniform per wavefront (kBM is a multiple of 64).
+  auto scale_dword = [&](int j) { return (j * S::kWaves + wave) * 64 + lane; };
+#pragma unroll
+  for (int j = 0; j < S::kSDma; ++j) {
+    const int d = scale_dword(j);
+    if (d < kBM) {
+      const int m = m0 + d < M ? m0 + d : M - 1;
+      soff[j] = static_cast<uint32_t>(m) * srow_bytes;
+    } else {
+      const int r = d - kBM < kBN ? d - kBM : kBN - 1;
+      const int n = n0 + r < N ? n0 + r : N - 1;
+      soff[j] = static_cast<uint32_t>(n) * srow_bytes;
+    }
   }
-  // waves 0..3 hold x rows, 4..7 w rows: uniform per wavefront
-  sbase = wave < 4 ? a.xs : a.ws;
 
   auto lds_addr = [&](int byte_off) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
@@ -157,14 +183,150 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
     for (int j = 0; j < S::kWDma; ++j) {
       QQ_DMA16(woff[j], wg, stage + S::kXTile + (wave * S::kWDma + j) * 1024);
     }
-    QQ_DMA4(soff, sbase + static_cast<size_t>(tc) * 4, stage + S::kXTile + S::kWTile + wave * 256);
+#pragma unroll
+    for (int j = 0; j < S::kSDma; ++j) {
+      const int first = (j * S::kWaves + wave) * 64; // uniform
+      const uint8_t* sg = (first < kBM ? a.xs : a.ws) + static_cast<size_t>(tc) * 4;
+      QQ_DMA4(soff[j], sg, stage + S::kXTile + S::kWTile + first * 4);
+    }
   };
 
-  qq_f32x4 acc[NI][4]; // [n tile][m tile]
+  if constexpr (BIG) {
+    // ---- 32 x 32 tiles: MI / 2 x NI / 2 per wavefront, two instructions (the
+    // halves of the 128-code step) per tile and step.  Lane l supplies row l % 32
+    // and the 32 codes [64 h + 32 (l / 32), + 32) of half h: piece 2 h + l / 32.
+    constexpr int MT = MI / 2;
+    constexpr int NT = NI / 2;
+    static_assert(NT % 2 == 0 && (MT == 1 || MT % 2 == 0), "scale bytes travel packed");
+    qq_f32x16 acc[NT][MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          acc[i][j][r] = 0.0f;
+        }
+      }
+    }
+    const int fr = lane & 31;
+    const int kblk = lane >> 5;
+    constexpr int kS = S::kStages;
+#pragma unroll
+    for (int t = 0; t < kS - 1; ++t) {
+      issue(t);
+    }
+    for (int t = 0; t < nk; ++t) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kS - 2) * S::kLoads) : "memory");
+      __syncthreads();
+      issue(t + kS - 1);
+      const uint8_t* st = smem + (t % kS) * S::kStage;
+      const uint32_t* sc = reinterpret_cast<const uint32_t*>(st + S::kXTile + S::kWTile);
+      qq_i32x4 af[2][NT], bf[2][MT];
+      // scale bytes: register q holds tiles 2 q and 2 q + 1, bytes (tile % 2) 2 + h
+      int sa[(NT + 1) / 2], sb[(MT + 1) / 2];
+      auto two_bytes = [&](uint32_t d) {
+        // the blocks of this lane in the two halves: kblk and 2 + kblk
+        return ((d >> (8 * kblk)) & 0xffu) | (((d >> (8 * (2 + kblk))) & 0xffu) << 8);
+      };
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        const int xr = wm * 16 * MI + 32 * j + fr;
+        const uint8_t* row = st + xr * S::kRowBytes;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const uint4 v = *reinterpret_cast<const uint4*>(row + qq_slot<4>(xr, 2 * h + kblk) * 16);
+          bf[h][j] = qq_i32x4{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+        }
+        const uint32_t two = two_bytes(sc[xr]);
+        if (j % 2 == 0) {
+          sb[j / 2] = static_cast<int>(two);
+        } else {
+          sb[j / 2] |= static_cast<int>(two << 16);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const int wr = wn * 16 * NI + 32 * i + fr;
+        const uint8_t* row = st + S::kXTile + wr * S::kRowBytes;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const uint4 v = *reinterpret_cast<const uint4*>(row + qq_slot<4>(wr, 2 * h + kblk) * 16);
+          af[h][i] = qq_i32x4{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+        }
+        const uint32_t two = two_bytes(sc[kBM + wr]);
+        if (i % 2 == 0) {
+          sa[i / 2] = static_cast<int>(two);
+        } else {
+          sa[i / 2] |= static_cast<int>(two << 16);
+        }
+      }
+      auto wide = [](const qq_i32x4& f) { return qq_i32x8{f[0], f[1], f[2], f[3], 0, 0, 0, 0}; };
+#define QQ_MMA32(i, j, h)                                                        \
+  if constexpr ((i) < NT && (j) < MT) {                                          \
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                 \
+        wide(af[h][i]), wide(bf[h][j]), acc[i][j], 4, 4, ((i) % 2) * 2 + (h),    \
+        sa[(i) / 2], ((j) % 2) * 2 + (h), sb[(j) / 2]);                          \
+  }
+#define QQ_MMA32_ROW(i, h)                                                       \
+  QQ_MMA32(i, 0, h) QQ_MMA32(i, 1, h) QQ_MMA32(i, 2, h) QQ_MMA32(i, 3, h)
+      QQ_MMA32_ROW(0, 0) QQ_MMA32_ROW(1, 0) QQ_MMA32_ROW(2, 0) QQ_MMA32_ROW(3, 0)
+      QQ_MMA32_ROW(0, 1) QQ_MMA32_ROW(1, 1) QQ_MMA32_ROW(2, 1) QQ_MMA32_ROW(3, 1)
+#undef QQ_MMA32_ROW
+#undef QQ_MMA32
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // D[n][m] 32 x 32: register i of lane (col, half) holds n = 8 (i / 4) + 4 half
+    // + i % 4, m = col
+    TO* out = static_cast<TO*>(a.out);
+    const int col = lane & 31;
+    const int half = lane >> 5;
+    const bool vec_ok = (N % 4) == 0;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      const int m = m0 + wm * 16 * MI + 32 * j + col;
+      if (m >= M) {
+        continue;
+      }
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int n = n0 + wn * 16 * NI + 32 * i + 8 * g4 + 4 * half;
+          if (n >= N) {
+            continue;
+          }
+          const float v0 = acc[i][j][4 * g4 + 0], v1 = acc[i][j][4 * g4 + 1];
+          const float v2 = acc[i][j][4 * g4 + 2], v3 = acc[i][j][4 * g4 + 3];
+          TO* dst = out + static_cast<size_t>(m) * N + n;
+          if (vec_ok && n + 4 <= N) {
+            if constexpr (sizeof(TO) == 4) {
+              *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
+            } else {
+              uint2 v;
+              v.x = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, from_f32<TO>(v0))) |
+                  (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, from_f32<TO>(v1))) << 16);
+              v.y = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, from_f32<TO>(v2))) |
+                  (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, from_f32<TO>(v3))) << 16);
+              *reinterpret_cast<uint2*>(dst) = v;
+            }
+          } else {
+            const float vals[4] = {v0, v1, v2, v3};
+            for (int r = 0; r < 4 && n + r < N; ++r) {
+              dst[r] = from_f32<TO>(vals[r]);
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
+
+  qq_f32x4 acc[NI][MI]; // [n tile][m tile]
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < MI; ++j) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         acc[i][j][r] = 0.0f;
@@ -180,8 +342,8 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
   // the instruction's op_sel picks the row's byte.
   using Frag = std::conditional_t<BITS == 8, qq_i32x8, qq_i32x4>;
   struct Frags {
-    Frag af[NI], bf[4];
-    int sa[NI / 4], sb;
+    Frag af[NI], bf[MI];
+    int sa[NI / 4], sb[MI / 4];
   };
   auto fragment = [&](const uint8_t* row_base, int r) -> Frag {
     const uint8_t* row = row_base + r * S::kRowBytes;
@@ -205,22 +367,25 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
     }
   };
   // byte kb of four rows' scale dwords, packed (row j in byte j)
-  auto pack_scales = [&](uint32_t d0, uint32_t d1, uint32_t d2, uint32_t d3) {
+  auto pack_scales = [&](const uint32_t* d) {
     const int sh = 8 * kb;
     return static_cast<int>(
-        ((d0 >> sh) & 0xffu) | (((d1 >> sh) & 0xffu) << 8) | (((d2 >> sh) & 0xffu) << 16) |
-        ((d3 >> sh) << 24));
+        ((d[0] >> sh) & 0xffu) | (((d[16] >> sh) & 0xffu) << 8) | (((d[32] >> sh) & 0xffu) << 16) |
+        ((d[48] >> sh) << 24));
   };
   // the fragments and scale bytes of step t, from its stage
   auto read_step = [&](int t, Frags& f) {
     const uint8_t* st = smem + (t % S::kStages) * S::kStage;
     const uint32_t* sc = reinterpret_cast<const uint32_t*>(st + S::kXTile + S::kWTile);
-    const int xr0 = wm * 64 + fr; // x tile rows xr0 + 16 j
+    const int xr0 = wm * 16 * MI + fr; // x tile rows xr0 + 16 j
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < MI; ++j) {
       f.bf[j] = fragment(st, xr0 + 16 * j);
     }
-    f.sb = pack_scales(sc[xr0], sc[xr0 + 16], sc[xr0 + 32], sc[xr0 + 48]);
+#pragma unroll
+    for (int q = 0; q < MI / 4; ++q) {
+      f.sb[q] = pack_scales(sc + xr0 + 64 * q);
+    }
     const int wr0 = wn * 16 * NI + fr; // W tile rows wr0 + 16 i
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -228,20 +393,20 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
     }
 #pragma unroll
     for (int q = 0; q < NI / 4; ++q) {
-      const uint32_t* sw = sc + kQqBM + wr0 + 64 * q;
-      f.sa[q] = pack_scales(sw[0], sw[16], sw[32], sw[48]);
+      f.sa[q] = pack_scales(sc + kBM + wr0 + 64 * q);
     }
   };
   // cbsz / blgp: the operand formats (0 = e4m3, 4 = e2m1); op_sel: which byte of
   // the scale registers
 #define QQ_MMA(i, j)                                                             \
-  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(                  \
-      operand(f.af[i]), operand(f.bf[j]), acc[i][j], BITS == 8 ? 0 : 4,          \
-      BITS == 8 ? 0 : 4, (i) % 4, f.sa[(i) / 4], (j), f.sb);
-#define QQ_MMA_ROW(i)                                                            \
-  if constexpr ((i) < NI) {                                                      \
-    QQ_MMA(i, 0) QQ_MMA(i, 1) QQ_MMA(i, 2) QQ_MMA(i, 3)                          \
+  if constexpr ((i) < NI && (j) < MI) {                                          \
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(                \
+        operand(f.af[i]), operand(f.bf[j]), acc[i][j], BITS == 8 ? 0 : 4,        \
+        BITS == 8 ? 0 : 4, (i) % 4, f.sa[(i) / 4], (j) % 4, f.sb[(j) / 4]);      \
   }
+#define QQ_MMA_ROW(i)                                                            \
+  QQ_MMA(i, 0) QQ_MMA(i, 1) QQ_MMA(i, 2) QQ_MMA(i, 3)                            \
+  QQ_MMA(i, 4) QQ_MMA(i, 5) QQ_MMA(i, 6) QQ_MMA(i, 7)
   auto multiply = [&](const Frags& f) {
     QQ_MMA_ROW(0) QQ_MMA_ROW(1) QQ_MMA_ROW(2) QQ_MMA_ROW(3)
     QQ_MMA_ROW(4) QQ_MMA_ROW(5) QQ_MMA_ROW(6) QQ_MMA_ROW(7)
@@ -279,8 +444,8 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
   const int quad = lane >> 4;
   const bool vec_ok = (N % 4) == 0;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int m = m0 + wm * 64 + 16 * j + col;
+  for (int j = 0; j < MI; ++j) {
+    const int m = m0 + wm * 16 * MI + 16 * j + col;
     if (m >= M) {
       continue;
     }
@@ -312,17 +477,16 @@ __global__ __launch_bounds__(kQqThreads) void qq_mfma_kernel(const QqArgs a) {
   }
 }
 
-template <typename TO, int BITS, int NI>
+template <typename TO, int BITS, int MI, int NI, int WM, int WN, bool BIG = false>
 int launch_qq(const QqArgs& a, hipStream_t s) {
-  using S = QqShape<BITS, NI>;
-  constexpr int kQqBN = S::kBN;
+  using S = QqShape<BITS, MI, NI, WM, WN>;
   constexpr size_t smem = static_cast<size_t>(S::kStages) * S::kStage;
   static_assert(smem <= 160 * 1024, "LDS");
-  const dim3 grid((a.N + kQqBN - 1) / kQqBN, (a.M + kQqBM - 1) / kQqBM, 1);
+  const dim3 grid((a.N + S::kBN - 1) / S::kBN, (a.M + S::kBM - 1) / S::kBM, 1);
   if (grid.y > 65535u) {
     return fail(MLXROCM_UNSUPPORTED, "[qqmm] M=%d exceeds the grid", a.M);
   }
-  auto kern = qq_mfma_kernel<TO, BITS, NI>;
+  auto kern = qq_mfma_kernel<TO, BITS, MI, NI, WM, WN, BIG>;
   static bool configured = false; // per instantiation
   if (!configured) {
     MLXROCM_HIP_TRY(hipFuncSetAttribute(
@@ -331,7 +495,7 @@ int launch_qq(const QqArgs& a, hipStream_t s) {
         static_cast<int>(smem)));
     configured = true;
   }
-  kern<<<grid, kQqThreads, smem, s>>>(a);
+  kern<<<grid, S::kThreads, smem, s>>>(a);
   MLXROCM_HIP_TRY(hipGetLastError());
   return static_cast<int>(MLXROCM_OK);
 }
@@ -373,14 +537,14 @@ int launch_qq_mfma(
   return dispatch_dtype(dtype, [&](auto tval) {
     using T = decltype(tval);
     if (mode == MLXROCM_MXFP8) {
-      return launch_qq<T, 8, 4>(a, s);
+      return launch_qq<T, 8, 4, 4, 4, 2>(a, s);
     }
     // the wide tile where it still fills the chip
-    const long wide = static_cast<long>((M + kQqBM - 1) / kQqBM) * ((N + 255) / 256);
+    const long wide = static_cast<long>((M + 255) / 256) * ((N + 255) / 256);
     if (wide >= compute_units()) {
-      return launch_qq<T, 4, 8>(a, s);
+      return launch_qq<T, 4, 4, 8, 4, 2, true>(a, s);
     }
-    return launch_qq<T, 4, 4>(a, s);
+    return launch_qq<T, 4, 4, 4, 4, 2, true>(a, s);
   });
 }
 
