@@ -40,10 +40,9 @@ constexpr int kQqBK = 128; // codes per step
 //   <4, 4, 4, 4, 2>: 256 x 128                    (4-bit codes, few tiles)
 // What the shapes trade is bytes fetched per flop: measured at [8192, 4096] x
 // [14336, 4096], 4-bit, the 256 x 256 tile runs at 2.5 PFLOP/s and the 256 x 128
-// tile at 2.0 -- both 4.7-4.8 TB/s of global -> LDS traffic, which is what this
-// loop is bound by (the matrix pipe alone does 6.9).  Four wavefronts of
-// 128 x 128 (one per SIMD, 256 accumulators in AGPRs, fewer LDS bytes per flop)
-// fetch the same bytes and were slower (2.3).
+// tile at 2.0 (the matrix pipe alone does 6.9).  Four wavefronts of 128 x 128
+// (one per SIMD, 256 accumulators in AGPRs, fewer LDS bytes per flop) fetch the
+// same bytes and were slower (2.3).
 template <int BITS, int MI, int NI, int WM, int WN>
 struct QqShape {
   static constexpr int kThreads = 64 * WM * WN;
