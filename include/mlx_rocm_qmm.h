@@ -237,6 +237,31 @@ int mlxrocm_fp_qqmm(
     size_t workspace_bytes,
     mlxrocm_stream_t stream);
 
+/* mlxrocm_qmm_plan for the two entry points above: what a call with these
+ * shape arguments and this much workspace would launch, written into `plan`
+ * as "a+b+c" without touching a device, or the error it would return. */
+int mlxrocm_fp_qmm_plan(
+    int M,
+    int N,
+    int K,
+    int L,
+    int batched_weights,
+    int mode,
+    int dtype,
+    int transpose,
+    size_t workspace_bytes,
+    char* plan,
+    size_t plan_bytes);
+int mlxrocm_fp_qqmm_plan(
+    int M,
+    int N,
+    int K,
+    int mode,
+    int dtype,
+    size_t workspace_bytes,
+    char* plan,
+    size_t plan_bytes);
+
 /* gather_qmm for the floating-point modes (mlx/ops.cpp:5553-5629 with
  * mode != "affine"; CPU: mlx/backend/cpu/quantized.cpp:806-900 fp_bs_qmm_dispatch_mode).
  * Arguments as mlxrocm_gather_qmm without biases; pair i multiplies

@@ -60,6 +60,8 @@ SIGNATURES = {
     "mlxrocm_fp_qmm": (_i, [_p] * 4 + [_i] * 4 + [_i64] * 3 + [_i] * 3 + [_p, _sz, _p]),
     "mlxrocm_fp_qqmm_workspace_size": (_sz, [_i] * 5),
     "mlxrocm_fp_qqmm": (_i, [_p] * 4 + [_i] * 5 + [_p, _sz, _p]),
+    "mlxrocm_fp_qmm_plan": (_i, [_i] * 8 + [_sz, ctypes.c_char_p, _sz]),
+    "mlxrocm_fp_qqmm_plan": (_i, [_i] * 5 + [_sz, ctypes.c_char_p, _sz]),
     "mlxrocm_fp_gather_qmm": (_i, [_p] * 6 + [_i] * 6 + [_i64] * 3 + [_i] * 3 + [_p]),
     "mlxrocm_qmm_kernel_name": (ctypes.c_char_p, [_i] * 8),
     "mlxrocm_qmm_plan": (_i, [_i] * 9 + [_sz, ctypes.c_char_p, _sz]),
@@ -155,6 +157,29 @@ def gather_qmm_plan(M, N, K, n_indices, x_batches, n_experts, group_size=64, bit
     buf = ctypes.create_string_buffer(1024)
     rc = lib.mlxrocm_gather_qmm_plan(M, N, K, n_indices, x_batches, n_experts, group_size, bits,
                                      dtype, int(transpose), workspace_bytes, buf, len(buf))
+    return rc, buf.value.decode()
+
+
+def fp_qmm_plan(M, N, K, L=1, batched_weights=False, mode=MXFP4, dtype=BFLOAT16, transpose=True,
+                workspace_bytes=None):
+    """(status, plan) of mlxrocm_fp_qmm for these arguments; the workspace
+    defaults to what mlxrocm_fp_qmm_workspace_size asks for."""
+    lib = load()
+    if workspace_bytes is None:
+        workspace_bytes = lib.mlxrocm_fp_qmm_workspace_size(
+            M, N, K, L, int(batched_weights), mode, dtype, int(transpose))
+    buf = ctypes.create_string_buffer(512)
+    rc = lib.mlxrocm_fp_qmm_plan(M, N, K, L, int(batched_weights), mode, dtype, int(transpose),
+                                 workspace_bytes, buf, len(buf))
+    return rc, buf.value.decode()
+
+
+def fp_qqmm_plan(M, N, K, mode=MXFP4, dtype=BFLOAT16, workspace_bytes=None):
+    lib = load()
+    if workspace_bytes is None:
+        workspace_bytes = lib.mlxrocm_fp_qqmm_workspace_size(M, N, K, mode, dtype)
+    buf = ctypes.create_string_buffer(512)
+    rc = lib.mlxrocm_fp_qqmm_plan(M, N, K, mode, dtype, workspace_bytes, buf, len(buf))
     return rc, buf.value.decode()
 
 

@@ -834,6 +834,52 @@ extern "C" int mlxrocm_fp_qqmm(
       static_cast<char*>(workspace) + xhat_bytes, workspace_bytes - xhat_bytes, stream);
 }
 
+namespace {
+
+// Stand-ins for device pointers in a rehearsal: aligned, never dereferenced.
+void* fake_pointer(int which) {
+  return reinterpret_cast<void*>(uintptr_t{1} << 40 | static_cast<uintptr_t>(which) << 32);
+}
+
+} // namespace
+
+extern "C" int mlxrocm_fp_qmm_plan(
+    int M,
+    int N,
+    int K,
+    int L,
+    int batched_weights,
+    int mode,
+    int dtype,
+    int transpose,
+    size_t workspace_bytes,
+    char* plan,
+    size_t plan_bytes) {
+  RehearsalScope rehearsal(plan, plan_bytes);
+  const int64_t w_stride = batched_weights ? int64_t{1} << 28 : 0;
+  return fp_qmm_entry(
+      fake_pointer(0), static_cast<const uint32_t*>(fake_pointer(1)),
+      static_cast<const uint8_t*>(fake_pointer(2)), fake_pointer(3), M, N, K, L,
+      static_cast<int64_t>(M) * K, w_stride, w_stride, mode, dtype, transpose,
+      workspace_bytes != 0 ? fake_pointer(4) : nullptr, workspace_bytes, nullptr);
+}
+
+extern "C" int mlxrocm_fp_qqmm_plan(
+    int M,
+    int N,
+    int K,
+    int mode,
+    int dtype,
+    size_t workspace_bytes,
+    char* plan,
+    size_t plan_bytes) {
+  RehearsalScope rehearsal(plan, plan_bytes);
+  return mlxrocm_fp_qqmm(
+      fake_pointer(0), static_cast<const uint32_t*>(fake_pointer(1)),
+      static_cast<const uint8_t*>(fake_pointer(2)), fake_pointer(3), M, N, K, mode, dtype,
+      workspace_bytes != 0 ? fake_pointer(4) : nullptr, workspace_bytes, nullptr);
+}
+
 extern "C" size_t mlxrocm_fp_qmm_workspace_size(
     int M, int N, int K, int L, int batched_weights, int mode, int dtype, int transpose) {
   if (fp_check("quantized_matmul", M, N, K, L, mode, dtype, transpose) != MLXROCM_OK ||

@@ -467,6 +467,7 @@ extern "C" int mlxrocm_fp_quantize_dequantize(
     return fail(MLXROCM_UNSUPPORTED, "[quantize_dequantize] %zu elements exceed the grid", n_elems);
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
+  MLXROCM_REHEARSE("fp_quantize_dequantize");
   return dispatch_dtype(dtype, [&](auto tval) {
     using T = decltype(tval);
     return dispatch_mode(mode, [&](auto gval, auto bval) {

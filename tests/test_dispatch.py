@@ -125,3 +125,71 @@ def test_rule_table_is_listed():
     lib = _lib.load()
     assert lib.mlxrocm_qmm_rule_name(len(rules)) is None
     assert lib.mlxrocm_qmm_rule_name(-1) is None
+
+
+# ---- floating-point modes -------------------------------------------------
+FP_MODES = {"mxfp4": _lib.MXFP4, "mxfp8": _lib.MXFP8, "nvfp4": _lib.NVFP4}
+
+
+def test_fp_qmm_workspace_size_is_exact_and_plans_name_the_kernels():
+    """mlxrocm_fp_qmm / mlxrocm_fp_qqmm rehearsed on the CPU: the call goes
+    through with exactly the workspace its size function names and is refused
+    with one byte fewer; decode, prefill and qqmm shapes take the kernels the
+    design notes name."""
+    lib = _lib.load()
+    for mode in FP_MODES.values():
+        for dtype in (_lib.BFLOAT16, _lib.FLOAT16, _lib.FLOAT32):
+            for transpose in (True, False):
+                for (M, N, K, L, batched) in ((1, 14336, 4096, 1, False), (8, 4096, 14336, 1, False),
+                                              (9, 14336, 4096, 1, False), (300, 1000, 256, 1, False),
+                                              (2048, 14336, 4096, 1, False), (40, 96, 256, 3, True),
+                                              (40, 96, 256, 3, False), (5, 64, 48, 1, False)):
+                    if K % (16 if mode == _lib.NVFP4 else 32) or (not transpose and N % 32):
+                        continue
+                    need = lib.mlxrocm_fp_qmm_workspace_size(M, N, K, L, int(batched), mode, dtype,
+                                                             int(transpose))
+                    rc, plan = _lib.fp_qmm_plan(M, N, K, L, batched, mode, dtype, transpose, need)
+                    assert rc == _lib.OK and plan, (mode, dtype, transpose, M, N, K, L, plan)
+                    tiled = "fp_qmm_t_tile" in plan
+                    assert tiled == (need > 0), (plan, need)
+                    if need:
+                        rc, _ = _lib.fp_qmm_plan(M, N, K, L, batched, mode, dtype, transpose, need - 1)
+                        assert rc == _lib.INVALID_ARGUMENT
+            for (M, N, K) in ((1, 14336, 4096), (15, 128, 256), (16, 128, 256), (8192, 14336, 4096),
+                              (64, 128, 96)):
+                if K % (16 if mode == _lib.NVFP4 else 32):
+                    continue
+                need = lib.mlxrocm_fp_qqmm_workspace_size(M, N, K, mode, dtype)
+                assert need > 0
+                rc, plan = _lib.fp_qqmm_plan(M, N, K, mode, dtype, need)
+                assert rc == _lib.OK and plan
+                rc, _ = _lib.fp_qqmm_plan(M, N, K, mode, dtype, need - 1)
+                assert rc == _lib.INVALID_ARGUMENT
+
+    bf16 = _lib.BFLOAT16
+    for mode in FP_MODES.values():
+        assert _lib.fp_qmm_plan(1, 14336, 4096, mode=mode)[1] == "fp_qmv16(mb=1)"
+        assert _lib.fp_qmm_plan(8, 14336, 4096, mode=mode)[1] == "fp_qmv16(mb=4)"
+        assert _lib.fp_qmm_plan(9, 14336, 4096, mode=mode)[1] == \
+            "fp_scale_image+fp_qmm_t_tile(ksplit=4)+reduce_k_splits(4)"
+        assert _lib.fp_qmm_plan(2048, 14336, 4096, mode=mode)[1] == "fp_scale_image+fp_qmm_t_tile(nt=7)"
+        assert _lib.fp_qmm_plan(64, 14336, 4096, mode=mode, dtype=_lib.FLOAT32)[1] == "fp_qmv"
+        assert _lib.fp_qmm_plan(64, 14336, 4096, mode=mode, transpose=False)[1] == "fp_qmm_n"
+    assert _lib.fp_qmm_plan(5, 64, 48, mode=_lib.NVFP4)[1] == "fp_qmm_naive_t"
+    # qqmm: block-scaled matrix instruction from 16 rows on, MX modes, K % 128 == 0
+    assert _lib.fp_qqmm_plan(8192, 14336, 4096, _lib.MXFP4, bf16)[1] == \
+        "fp_quantize_activations+qq_mfma(e2m1)"
+    assert _lib.fp_qqmm_plan(8192, 14336, 4096, _lib.MXFP8, bf16)[1] == \
+        "fp_quantize_activations+qq_mfma(e4m3)"
+    assert _lib.fp_qqmm_plan(16, 128, 256, _lib.MXFP4, _lib.FLOAT32)[1] == \
+        "fp_quantize_activations+qq_mfma(e2m1)"
+    # 8-bit codes in float32 stay on the fp32-accumulating kernels
+    assert _lib.fp_qqmm_plan(8192, 14336, 4096, _lib.MXFP8, _lib.FLOAT32)[1] == \
+        "fp_quantize_dequantize+fp_qmv"
+    # fewer than 16 rows: x_hat in the element type, then quantized_matmul's kernels
+    assert _lib.fp_qqmm_plan(15, 128, 256, _lib.MXFP4, bf16)[1] == \
+        "fp_quantize_dequantize+fp_scale_image+fp_qmm_t_tile(nt=5)"
+    assert _lib.fp_qqmm_plan(8, 128, 256, _lib.MXFP4, bf16)[1] == "fp_quantize_dequantize+fp_qmv16(mb=4)"
+    assert _lib.fp_qqmm_plan(64, 128, 96, _lib.MXFP4, bf16)[1].startswith("fp_quantize_dequantize+")
+    assert _lib.fp_qqmm_plan(8192, 14336, 4096, _lib.NVFP4, bf16)[1] == \
+        "fp_quantize_dequantize+fp_scale_image+fp_qmm_t_tile(nt=7)"
