@@ -177,3 +177,53 @@ def test_matmul_equals_the_dense_product(port, mode):
         exact = x.double() @ (w_hat.T if transpose else w_hat)
         assert float((y - exact).abs().max()) <= 1e-5 * (K ** 0.5) * float(x.abs().max()) * float(
             w_hat.abs().max())
+
+
+# ---- golden vectors written by the reference translation unit -------------
+# (tests/golden/make_fp_golden.py); these pin the port where the reference
+# checkout, and with it oracle/_ref, is absent.
+@pytest.fixture(scope="module")
+def golden():
+    import numpy as np
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fp_modes_ref.npz")
+    return np.load(path, allow_pickle=False)
+
+
+def test_converters_match_the_golden_vectors(port, golden):
+    import numpy as np
+
+    for c in range(256):
+        got = np.array([port.port.fpq_from_fp8(c)], dtype=np.float32).view(np.uint32)[0]
+        assert got == golden["from_fp8"][c], c
+    probes = golden["probe_bits"]
+    assert probes.size > 12000
+    for u, want8, want_e, want4 in zip(probes, golden["to_fp8"], golden["e8m0"], golden["e2m1"]):
+        f = struct.unpack("f", struct.pack("I", int(u)))[0]
+        assert port.port.fpq_to_fp8(f) == want8, f
+        assert port.port.fpq_e8m0(f) == want_e, f
+        assert port.port.fpq_e2m1(f) == want4, f
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("dname", ("f32", "f16", "bf16"))
+@pytest.mark.parametrize("transpose", (True, False))
+def test_matmul_matches_the_golden_vectors(port, golden, mode, dname, transpose):
+    import numpy as np
+
+    dtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dname]
+    tag = f"{mode}_{dname}_{'t' if transpose else 'n'}"
+
+    def tensor(name, dt):
+        a = golden[tag + name]
+        if dt in (torch.uint32, torch.uint8):
+            return torch.from_numpy(a.copy())
+        return torch.from_numpy(a.view(np.int32 if dt == torch.float32 else np.int16).copy()).view(dt)
+
+    wq = tensor("_wq", torch.uint32)
+    scales = tensor("_scales", torch.uint8)
+    x = tensor("_x", dtype)
+    want = tensor("_y", dtype)
+    got = port.port_qmm(x, wq, scales, mode, transpose)
+    assert torch.equal(qref_raw(got), qref_raw(want)), tag
