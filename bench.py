@@ -25,6 +25,7 @@ import time
 
 HBM_PEAK_GBPS = 8000.0
 BF16_PEAK_TFLOPS = 2500.0
+FP4_PEAK_TFLOPS = 10100.0
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes, scaled by
 # a copy of known size (profiles/qmv_stream_4bit_g64_bf16_14336x4096.md and
 # profiles/qmm_t_mfma_4bit_g64_bf16_M2048_14336x4096.md).
@@ -271,7 +272,7 @@ def sweep(torch, mlx_amd, dev) -> list:
             launcher.run(10)
             torch.cuda.synchronize()
             first = hip_event_ms(lib, launcher, 10)
-            per_region = max(10, int(5.0 / max(first, 1e-3)))
+            per_region = max(50, int(10.0 / max(first, 1e-3)))
             ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
         wshape = f"[{n},{k}]" if transpose else f"[{k},{n}] transpose=False"
         name = f"x {str(dtype)[6:]} [{M},{k}] W {wshape} b{bits} g{gs}"
@@ -474,7 +475,7 @@ def sweep(torch, mlx_amd, dev) -> list:
             launcher.run(10)
             torch.cuda.synchronize()
             first = hip_event_ms(lib, launcher, 10)
-            per_region = max(10, int(5.0 / max(first, 1e-3)))
+            per_region = max(50, int(10.0 / max(first, 1e-3)))
             ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
         name = f"{mode}: x bfloat16 [{M},{k}] W [{n},{k}]"
         if small:
@@ -504,7 +505,7 @@ def sweep(torch, mlx_amd, dev) -> list:
         launcher.run(10)
         torch.cuda.synchronize()
         first = hip_event_ms(lib, launcher, 10)
-        per_region = max(10, int(5.0 / max(first, 1e-3)))
+        per_region = max(50, int(10.0 / max(first, 1e-3)))
         ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
         add("f4", f"qqmm {mode}: x bfloat16 [{M},{k}] W [{n},{k}] (x quantized in the call)", ms,
             flops=2.0 * M * n * k)
@@ -568,6 +569,92 @@ def sweep(torch, mlx_amd, dev) -> list:
     return rows
 
 
+def fp_mode_figures(torch, mlx_amd, lib, dev) -> dict:
+    """The same shapes in the mxfp4 mode (floating-point codes, one e8m0 scale
+    byte per 32): decode GEMV over a ring of 18 weight copies (graph replays, HIP
+    events, median of 3 regions of 1800 launches), the prefill GEMM at 2048 rows
+    and qqmm -- x quantized inside the call, both operands' codes on the
+    block-scaled matrix instruction -- at 2048 and 8192 rows.  Extra figures
+    beside the headline ones, each with the peak it is priced against."""
+    from mlx_amd import _lib
+
+    g = torch.Generator().manual_seed(7)
+    bf16 = torch.bfloat16
+    mode, mcode = "mxfp4", _lib.MXFP4
+    w = torch.randn((N, K), generator=g, dtype=torch.float32).to(bf16).to(dev)
+    q = mlx_amd.quantize(w, mode=mode)
+    del w
+    ring = [q] + [tuple(t.clone() for t in q) for _ in range(RING - 1)]
+    out = {"mode": mode}
+
+    x1 = torch.randn((1, K), generator=g, dtype=torch.float32).to(bf16).to(dev)
+    y1 = torch.empty((1, N), dtype=bf16, device=dev)
+
+    def decode_step(i, stream):
+        wq_, s_ = ring[i % RING]
+        rc = lib.mlxrocm_fp_qmm(x1.data_ptr(), wq_.data_ptr(), s_.data_ptr(), y1.data_ptr(),
+                                1, N, K, 1, K, 0, 0, mcode, _lib.BFLOAT16, 1, None, 0, stream)
+        if rc != 0:
+            raise RuntimeError(_lib.last_error())
+
+    launcher = Launcher(torch, decode_step, RING, True)
+    launcher.run(2 * RING)
+    torch.cuda.synchronize()
+    launches = -(-QMV_MIN_LAUNCHES // RING) * RING
+    ms, samples = median_event_ms(lib, launcher, launches, repeats=3)
+    nbytes = N * K // 2 + N * (K // 32) + K * 2 + N * 2
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    out["qmv"] = {
+        "workload": f"x bf16 [1,{K}], W [{N},{K}] mxfp4",
+        "bytes_per_launch": nbytes, "us_per_launch": round(ms * 1e3, 3),
+        "value": round(gbps, 2), "unit": "GB/s", "bound": "hbm", "peak": HBM_PEAK_GBPS,
+        "frac": round(gbps / HBM_PEAK_GBPS, 4), "launches_timed": launches, "repeats": len(samples),
+    }
+
+    def big(name, M, entry, peak, what):
+        x = torch.randn((M, K), generator=g, dtype=torch.float32).to(bf16).to(dev)
+        y = torch.empty((M, N), dtype=bf16, device=dev)
+        if entry == "qmm":
+            ws_bytes = lib.mlxrocm_fp_qmm_workspace_size(M, N, K, 1, 0, mcode, _lib.BFLOAT16, 1)
+        else:
+            ws_bytes = lib.mlxrocm_fp_qqmm_workspace_size(M, N, K, mcode, _lib.BFLOAT16)
+        ws = torch.empty(max(int(ws_bytes), 256), dtype=torch.uint8, device=dev)
+
+        def step(i, stream):
+            wq_, s_ = ring[i % RING]
+            if entry == "qmm":
+                rc = lib.mlxrocm_fp_qmm(x.data_ptr(), wq_.data_ptr(), s_.data_ptr(), y.data_ptr(),
+                                        M, N, K, 1, M * K, 0, 0, mcode, _lib.BFLOAT16, 1,
+                                        ws.data_ptr(), ws_bytes, stream)
+            else:
+                rc = lib.mlxrocm_fp_qqmm(x.data_ptr(), wq_.data_ptr(), s_.data_ptr(), y.data_ptr(),
+                                         M, N, K, mcode, _lib.BFLOAT16, ws.data_ptr(), ws_bytes, stream)
+            if rc != 0:
+                raise RuntimeError(_lib.last_error())
+
+        launcher = Launcher(torch, step, RING, False)
+        launcher.run(10)
+        torch.cuda.synchronize()
+        first = hip_event_ms(lib, launcher, 10)
+        per_region = max(50, int(10.0 / max(first, 1e-3)))
+        ms, samples = median_event_ms(lib, launcher, per_region, repeats=3)
+        tflops = 2.0 * M * N * K / (ms * 1e-3) / 1e12
+        out[name] = {
+            "workload": f"x bf16 [{M},{K}], W [{N},{K}] mxfp4; {what}",
+            "us_per_launch": round(ms * 1e3, 2), "value": round(tflops, 2), "unit": "TFLOP/s",
+            "bound": "mfma", "peak": peak, "frac": round(tflops / peak, 4),
+            "launches_timed": per_region, "repeats": len(samples),
+        }
+
+    big("qmm_t", QMM_M, "qmm", BF16_PEAK_TFLOPS,
+        "weights widened to bf16 in the tile kernel (bf16 MFMA peak)")
+    big("qqmm_2048", QMM_M, "qqmm", FP4_PEAK_TFLOPS,
+        "x quantized inside the call, block-scaled fp4 MFMA (fp4 peak)")
+    big("qqmm_8192", 8192, "qqmm", FP4_PEAK_TFLOPS,
+        "x quantized inside the call, block-scaled fp4 MFMA (fp4 peak)")
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -577,6 +664,8 @@ def main() -> int:
     ap.add_argument("--only", choices=("qmv", "qmm_t"), default=None)
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying a HIP graph")
+    ap.add_argument("--no-fp", action="store_true",
+                    help="skip the extra figures of the mxfp4 mode (fp_modes)")
     ap.add_argument("--no-floor", action="store_true",
                     help="skip the read-only probe (roofline.read_only_floor_us)")
     ap.add_argument("--sweep", action="store_true",
@@ -811,6 +900,9 @@ def main() -> int:
             "us_per_launch_min_median_max": [round(samples_p[0] * 1e3, 2), round(ms_p * 1e3, 2),
                                              round(samples_p[-1] * 1e3, 2)],
         }
+
+    if args.only is None and not args.no_fp:
+        result["fp_modes"] = fp_mode_figures(torch, mlx_amd, lib, dev)
 
     if not args.no_cpu and args.only in (None, "qmv"):
         wq0, s0, b0 = ring[0]
