@@ -272,7 +272,7 @@ def sweep(torch, mlx_amd, dev) -> list:
             launcher.run(10)
             torch.cuda.synchronize()
             first = hip_event_ms(lib, launcher, 10)
-            per_region = max(50, int(10.0 / max(first, 1e-3)))
+            per_region = max(10, int(5.0 / max(first, 1e-3)))
             ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
         wshape = f"[{n},{k}]" if transpose else f"[{k},{n}] transpose=False"
         name = f"x {str(dtype)[6:]} [{M},{k}] W {wshape} b{bits} g{gs}"
@@ -475,7 +475,7 @@ def sweep(torch, mlx_amd, dev) -> list:
             launcher.run(10)
             torch.cuda.synchronize()
             first = hip_event_ms(lib, launcher, 10)
-            per_region = max(50, int(10.0 / max(first, 1e-3)))
+            per_region = max(10, int(5.0 / max(first, 1e-3)))
             ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
         name = f"{mode}: x bfloat16 [{M},{k}] W [{n},{k}]"
         if small:
@@ -505,7 +505,7 @@ def sweep(torch, mlx_amd, dev) -> list:
         launcher.run(10)
         torch.cuda.synchronize()
         first = hip_event_ms(lib, launcher, 10)
-        per_region = max(50, int(10.0 / max(first, 1e-3)))
+        per_region = max(10, int(5.0 / max(first, 1e-3)))
         ms, _ = median_event_ms(lib, launcher, per_region, repeats=5)
         add("f4", f"qqmm {mode}: x bfloat16 [{M},{k}] W [{n},{k}] (x quantized in the call)", ms,
             flops=2.0 * M * n * k)
