@@ -902,7 +902,10 @@ def main() -> int:
         }
 
     if args.only is None and not args.no_fp:
-        result["fp_modes"] = fp_mode_figures(torch, mlx_amd, lib, dev)
+        try:
+            result["fp_modes"] = fp_mode_figures(torch, mlx_amd, lib, dev)
+        except Exception as exc:  # extra figures: the headline line is printed regardless
+            result["fp_modes"] = {"error": f"{type(exc).__name__}: {exc}"}
 
     if not args.no_cpu and args.only in (None, "qmv"):
         wq0, s0, b0 = ring[0]
