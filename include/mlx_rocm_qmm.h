@@ -289,6 +289,101 @@ int mlxrocm_fp_gather_qmm(
     mlxrocm_stream_t stream);
 
 /*
+ * gather_qqmm (mlx/ops.cpp:5631-5681; GPU only in the reference:
+ * GatherQQMM::eval_gpu, mlx/backend/cuda/quantized/qqmm.cpp:210-281 -- the CPU
+ * backend throws "NYI", mlx/backend/cpu/quantized.cpp:1362-1364): every matrix
+ * of x is quantized and dequantized in its own type, then pair i multiplies
+ * x_hat[lhs_indices[i]] by the transposed w[rhs_indices[i]].  Arguments as
+ * mlxrocm_fp_gather_qmm with transpose = 1; x_batch_stride >= M * K.
+ * global_scale_x / global_scale_w: both null, or (nvfp4) both one float32 on
+ * the device, as in mlxrocm_nvfp4_qqmm_global.  workspace:
+ * mlxrocm_fp_gather_qqmm_workspace_size bytes (x_hat), 256-byte aligned, used
+ * only during the call.
+ */
+size_t mlxrocm_fp_gather_qqmm_workspace_size(int M, int K, int x_batches, int dtype);
+int mlxrocm_fp_gather_qqmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const uint32_t* lhs_indices,
+    const uint32_t* rhs_indices,
+    const float* global_scale_x,
+    const float* global_scale_w,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int64_t x_batch_stride,
+    int64_t w_expert_stride,
+    int64_t scales_expert_stride,
+    int mode,
+    int dtype,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream);
+
+/*
+ * nvfp4 with a tensor-wide scale (`global_scale` of mx.quantize / mx.dequantize
+ * / mx.qqmm, mlx/ops.cpp:4756-4782, 5101-5131, 5342-5398; one float32 on the
+ * device, usually max |w|).  The reference implements it on the GPU only
+ * (mlx/ops.cpp:4760-4766); these entry points follow the CUDA kernels' fp32
+ * arithmetic (mlx/backend/cuda/quantized/fp_quantize.cuh:73-215, 548-592):
+ *   scale_enc = 448 * 6 / global_scale
+ *   scale byte = e4m3(max |group| / 6 * scale_enc)
+ *   code = e2m1, nearest with ties to even, of w * (scale_enc / value(scale byte))
+ *   dequantize: code value * (value(scale byte) * (global_scale / (448 * 6)))
+ * Layouts as in mlxrocm_fp_quantize / mlxrocm_fp_dequantize with mode nvfp4.
+ */
+int mlxrocm_nvfp4_quantize_global(
+    const void* w,
+    const float* global_scale,
+    uint32_t* wq,
+    uint8_t* scales,
+    size_t n_elems,
+    int dtype,
+    mlxrocm_stream_t stream);
+int mlxrocm_nvfp4_dequantize_global(
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const float* global_scale,
+    void* out,
+    size_t n_elems,
+    int dtype,
+    mlxrocm_stream_t stream);
+/* fp_quantize_dequantize with a tensor-wide scale
+ * (mlx/backend/cuda/quantized/fp_quantize.cuh:73-145): what qqmm applies to x. */
+int mlxrocm_nvfp4_quantize_dequantize_global(
+    const void* x,
+    const float* global_scale,
+    void* out,
+    size_t n_elems,
+    int dtype,
+    mlxrocm_stream_t stream);
+/* qqmm in nvfp4 with both tensor-wide scales (QQMatmul::eval_gpu,
+ * mlx/backend/cuda/quantized/qqmm.cpp:100-208, the route it takes without a
+ * block-scaled GEMM library): x_hat = quantize_dequantize(x, global_scale_x) in
+ * dtype; y = (x_hat . codes-times-block-scales^T) * (global_scale_w / (448 * 6)),
+ * the factor applied to the fp32 sums (mlx/backend/cuda/quantized/qmm/qmv.cu:163-165).
+ * workspace: mlxrocm_fp_qqmm_workspace_size(M, N, K, MLXROCM_NVFP4, dtype) bytes. */
+int mlxrocm_nvfp4_qqmm_global(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const float* global_scale_x,
+    const float* global_scale_w,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int dtype,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream);
+
+/*
  * GGML tensor types the GGUF loader keeps quantized (ids as in the GGUF file
  * format; every other quantized type is dequantized to fp16 by MLX's loader,
  * mlx/io/gguf.cpp, and is not handled here).

@@ -51,6 +51,18 @@ __device__ __forceinline__ float scale_value(uint32_t s) {
   }
 }
 
+// Factor of the fp32 sums: weights quantized with a tensor-wide scale (nvfp4
+// only; mlx/backend/cuda/quantized/qmm/qmv.cu:163-165), 1 otherwise.
+template <int GS>
+__device__ __forceinline__ float fp_out_factor(const QmmArgs& a) {
+  if constexpr (GS == 16) {
+    if (a.out_scale != nullptr) {
+      return *a.out_scale / (448.0f * 6.0f);
+    }
+  }
+  return 1.0f;
+}
+
 struct FpProblem {
   const uint8_t* x;
   const uint8_t* w;
@@ -166,11 +178,12 @@ __global__ __launch_bounds__(64 * kFpWaves) void fp_qmv_kernel(const QmmArgs a) 
       }
     }
   }
+  const float out_factor = fp_out_factor<GS>(a);
 #pragma unroll
   for (int r = 0; r < kFpRowsPerWave; ++r) {
 #pragma unroll
     for (int m = 0; m < kFpRowBlock; ++m) {
-      const float y = wave_sum(acc[r][m]);
+      const float y = wave_sum(acc[r][m]) * out_factor;
       if (lane == 0 && m < rows && n0 + r < N) {
         reinterpret_cast<T*>(p.out)[static_cast<size_t>(m0 + m) * N + n0 + r] =
             from_f32<T>(p.valid ? y : 0.0f);
@@ -403,11 +416,12 @@ __global__ __launch_bounds__(64 * kFp16Waves) void fp_qmv16_kernel(const QmmArgs
       }
     }
   }
+  const float out_factor = fp_out_factor<GS>(a);
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
-      const float y = wave_sum(acc[r][m]);
+      const float y = wave_sum(acc[r][m]) * out_factor;
       if (lane == 0 && m0 + m < a.M && n0 + r < N) {
         reinterpret_cast<T*>(p.out)[static_cast<size_t>(m0 + m) * N + n0 + r] =
             from_f32<T>(p.valid ? y : 0.0f);
@@ -445,6 +459,7 @@ __global__ __launch_bounds__(256) void fp_qmm_naive_t_kernel(const QmmArgs a) {
     }
     acc = fmaf(scale_value<GS>(sc[g]), part, acc);
   }
+  acc *= fp_out_factor<GS>(a);
   reinterpret_cast<T*>(p.out)[static_cast<size_t>(m) * a.N + n] = from_f32<T>(p.valid ? acc : 0.0f);
 }
 
@@ -638,7 +653,8 @@ int fp_qmm_entry(
     int transpose,
     void* workspace,
     size_t workspace_bytes,
-    mlxrocm_stream_t stream) {
+    mlxrocm_stream_t stream,
+    const float* out_scale = nullptr) {
   int rc = fp_check("quantized_matmul", M, N, K, L, mode, dtype, transpose);
   if (rc != MLXROCM_OK) {
     return rc;
@@ -676,6 +692,7 @@ int fp_qmm_entry(
   a.sb_batch_stride = scales_batch_stride;
   a.x_batches = L;
   a.n_experts = L;
+  a.out_scale = out_scale;
   if (fp_tile_applies(M, N, K, L, mode, dtype, transpose != 0)) {
     const int batches = scales_batch_stride != 0 ? L : 1;
     const size_t need = fp_tile_workspace(M, N, K, L, batches);
@@ -892,7 +909,9 @@ extern "C" size_t mlxrocm_fp_qmm_workspace_size(
   return fp_tile_workspace(M, N, K, L, batched_weights ? L : 1);
 }
 
-extern "C" int mlxrocm_fp_gather_qmm(
+namespace {
+
+int fp_gather_entry(
     const void* x,
     const uint32_t* wq,
     const uint8_t* scales,
@@ -911,8 +930,8 @@ extern "C" int mlxrocm_fp_gather_qmm(
     int mode,
     int dtype,
     int transpose,
-    mlxrocm_stream_t stream) {
-  mlxrocm::ApiRange api_range("mlxrocm_fp_gather_qmm");
+    mlxrocm_stream_t stream,
+    const float* out_scale) {
   int rc = fp_check("gather_qmm", M, N, K, n_indices, mode, dtype, transpose);
   if (rc != MLXROCM_OK) {
     return rc;
@@ -954,10 +973,202 @@ extern "C" int mlxrocm_fp_gather_qmm(
     a.rhs_indices = rhs_indices + first;
     a.x_batches = x_batches;
     a.n_experts = n_experts;
+    a.out_scale = out_scale;
     rc = fp_launch(a, mode, dtype, transpose != 0, s);
     if (rc != MLXROCM_OK) {
       return rc;
     }
   }
   return MLXROCM_OK;
+}
+
+// The two tensor-wide scales of nvfp4: both or neither, and only in that mode.
+int check_global_scales(const char* who, int mode, const float* gx, const float* gw) {
+  if ((gx == nullptr) != (gw == nullptr)) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[%s] For nvfp4 mode, either both global_scale_x and global_scale_w must be provided, "
+        "or neither.", who);
+  }
+  if (gx != nullptr && mode != MLXROCM_NVFP4) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[%s] Global scale is only supported for 'nvfp4' mode.", who);
+  }
+  if ((reinterpret_cast<uintptr_t>(gx) & 3u) != 0 || (reinterpret_cast<uintptr_t>(gw) & 3u) != 0) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[%s] a global scale must point at one float32", who);
+  }
+  return MLXROCM_OK;
+}
+
+} // namespace
+
+extern "C" int mlxrocm_fp_gather_qmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const uint32_t* lhs_indices,
+    const uint32_t* rhs_indices,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int64_t x_batch_stride,
+    int64_t w_expert_stride,
+    int64_t scales_expert_stride,
+    int mode,
+    int dtype,
+    int transpose,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_fp_gather_qmm");
+  return fp_gather_entry(
+      x, wq, scales, lhs_indices, rhs_indices, out, M, N, K, n_indices, x_batches, n_experts,
+      x_batch_stride, w_expert_stride, scales_expert_stride, mode, dtype, transpose, stream,
+      nullptr);
+}
+
+extern "C" size_t mlxrocm_fp_gather_qqmm_workspace_size(int M, int K, int x_batches, int dtype) {
+  if (!valid_dtype(dtype) || M <= 0 || K <= 0 || x_batches <= 0) {
+    return 0;
+  }
+  return round256(static_cast<size_t>(x_batches) * M * K * dtype_size(dtype));
+}
+
+extern "C" int mlxrocm_fp_gather_qqmm(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const uint32_t* lhs_indices,
+    const uint32_t* rhs_indices,
+    const float* global_scale_x,
+    const float* global_scale_w,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int64_t x_batch_stride,
+    int64_t w_expert_stride,
+    int64_t scales_expert_stride,
+    int mode,
+    int dtype,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_fp_gather_qqmm");
+  int rc = fp_check("gather_qqmm", M, N, K, n_indices, mode, dtype, 1);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  rc = check_global_scales("gather_qqmm", mode, global_scale_x, global_scale_w);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (static_cast<int64_t>(M) * N * n_indices == 0) {
+    return MLXROCM_OK;
+  }
+  if (K == 0) {
+    return launch_zero_fill(
+        out, static_cast<size_t>(M) * N * n_indices * dtype_size(dtype),
+        static_cast<hipStream_t>(stream));
+  }
+  if (!x) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qqmm] null device pointer");
+  }
+  const int64_t rows_elems = static_cast<int64_t>(M) * K;
+  if (x_batches <= 0 || x_batch_stride < rows_elems) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qqmm] invalid batch description");
+  }
+  const size_t need = mlxrocm_fp_gather_qqmm_workspace_size(M, K, x_batches, dtype);
+  if (workspace == nullptr || workspace_bytes < need ||
+      (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[gather_qqmm] needs a 256-byte aligned workspace of %zu bytes "
+        "(mlxrocm_fp_gather_qqmm_workspace_size); got %zu",
+        need, workspace_bytes);
+  }
+  // x_hat: every matrix of x quantized and dequantized in its own type, packed
+  const size_t esize = dtype_size(dtype);
+  const bool packed = x_batch_stride == rows_elems;
+  const int calls = packed ? 1 : x_batches;
+  const size_t per_call = static_cast<size_t>(rows_elems) * (packed ? x_batches : 1);
+  for (int b = 0; b < calls; ++b) {
+    const char* src = static_cast<const char*>(x) + static_cast<size_t>(b) * x_batch_stride * esize;
+    char* dst = static_cast<char*>(workspace) + static_cast<size_t>(b) * rows_elems * esize;
+    rc = global_scale_x != nullptr
+        ? mlxrocm_nvfp4_quantize_dequantize_global(src, global_scale_x, dst, per_call, dtype, stream)
+        : mlxrocm_fp_quantize_dequantize(src, dst, per_call, mode, dtype, stream);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+  }
+  return fp_gather_entry(
+      workspace, wq, scales, lhs_indices, rhs_indices, out, M, N, K, n_indices, x_batches,
+      n_experts, rows_elems, w_expert_stride, scales_expert_stride, mode, dtype, 1, stream,
+      global_scale_w);
+}
+
+extern "C" int mlxrocm_nvfp4_qqmm_global(
+    const void* x,
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const float* global_scale_x,
+    const float* global_scale_w,
+    void* out,
+    int M,
+    int N,
+    int K,
+    int dtype,
+    void* workspace,
+    size_t workspace_bytes,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_nvfp4_qqmm_global");
+  const int mode = MLXROCM_NVFP4;
+  int rc = fp_check("qqmm", M, N, K, 1, mode, dtype, 1);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (global_scale_x == nullptr || global_scale_w == nullptr) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[qqmm] both global scales must be given");
+  }
+  rc = check_global_scales("qqmm", mode, global_scale_x, global_scale_w);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (static_cast<int64_t>(M) * N == 0) {
+    return MLXROCM_OK;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (K == 0) {
+    return launch_zero_fill(out, static_cast<size_t>(M) * N * dtype_size(dtype), s);
+  }
+  if (!x || !wq || !scales || !out) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[qqmm] null device pointer");
+  }
+  const size_t need = mlxrocm_fp_qqmm_workspace_size(M, N, K, mode, dtype);
+  if (workspace == nullptr || workspace_bytes < need ||
+      (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) {
+    return fail(
+        MLXROCM_INVALID_ARGUMENT,
+        "[qqmm] needs a 256-byte aligned workspace of %zu bytes (mlxrocm_fp_qqmm_workspace_size); "
+        "got %zu",
+        need, workspace_bytes);
+  }
+  if (!aligned16(x) || !aligned16(wq) || !aligned16(out)) {
+    return fail(MLXROCM_UNSUPPORTED, "[qqmm] operands must keep 16-byte alignment");
+  }
+  const size_t n_elems = static_cast<size_t>(M) * K;
+  rc = mlxrocm_nvfp4_quantize_dequantize_global(x, global_scale_x, workspace, n_elems, dtype, stream);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  const size_t xhat_bytes = round256(n_elems * dtype_size(dtype));
+  return fp_qmm_entry(
+      workspace, wq, scales, out, M, N, K, 1, 0, 0, 0, mode, dtype, 1,
+      static_cast<char*>(workspace) + xhat_bytes, workspace_bytes - xhat_bytes, stream,
+      global_scale_w);
 }

@@ -23,6 +23,17 @@
 // Quantize-dequantize of activations: fp_quantize_dequantize<T>
 // (mlx/backend/cpu/quantized.cpp:1049-1128), fp32 arithmetic, e2m1 ties to the
 // even mantissa.
+// nvfp4 with a tensor-wide scale (`global_scale`, one float on the device): the
+// CPU path has no such mode, so these kernels follow the CUDA backend's
+// arithmetic (mlx/backend/cuda/quantized/fp_quantize.cuh:73-145, 147-215,
+// 548-592), all in fp32:
+//   scale_enc = 448 * 6 / global_scale
+//   byte      = to_fp8(max(abs(group)) / 6 * scale_enc)
+//   code      = e2m1 nearest, ties to even, of w * (scale_enc / from_fp8(byte))
+//   dequantize:          code value * (from_fp8(byte) * (global_scale / (448 * 6)))
+//   quantize-dequantize: code value * (from_fp8(byte) * (1 / scale_enc))
+// A group of zeros gets the byte 0 and, through 0 * inf, the code of a NaN
+// (+6); it decodes to zeros.
 #include "common.h"
 
 namespace mlxrocm {
@@ -306,6 +317,78 @@ __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
   }
 }
 
+constexpr float kNvfp4Span = 448.0f * 6.0f;
+
+// One thread: 8 consecutive elements, two threads per group of 16.
+// OUT == 0: codes and scale bytes; OUT == 1: the dequantized elements.
+template <typename T, int OUT>
+__global__ __launch_bounds__(kFpBlock) void nvfp4_global_quantize_kernel(
+    const T* w, const float* global_scale, uint8_t* wq, uint8_t* scales, T* out, size_t n_units) {
+  const size_t u = static_cast<size_t>(blockIdx.x) * kFpBlock + threadIdx.x;
+  const float scale_enc = kNvfp4Span / *global_scale;
+  float v[8];
+  const bool live = u < n_units;
+  if (live) {
+    load8<T>(w + u * 8, v);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[i] = 0.0f;
+    }
+  }
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    m = fmaxf(m, fabsf(v[i]));
+  }
+  m = group_max(m, 2);
+  float scale_dec_b = m / 6.0f;
+  scale_dec_b *= scale_enc;
+  const uint32_t scale_byte = to_fp8_bits(scale_dec_b);
+  const float sv = from_fp8_bits(scale_byte);
+  const float scale_enc_b = scale_enc / sv;
+  if (!live) {
+    return;
+  }
+  uint32_t word = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    word |= fp4_nearest_even(v[i] * scale_enc_b) << (4 * i);
+  }
+  if constexpr (OUT == 0) {
+    reinterpret_cast<uint32_t*>(wq)[u] = word;
+    if ((u & 1) == 0) {
+      scales[u / 2] = static_cast<uint8_t>(scale_byte);
+    }
+  } else {
+    const float scale_dec = sv * (1.0f / scale_enc);
+    float o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      o[i] = fp4_value((word >> (4 * i)) & 0xFu) * scale_dec;
+    }
+    store8<T>(out + u * 8, o);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kFpBlock) void nvfp4_global_dequantize_kernel(
+    const uint8_t* wq, const uint8_t* scales, const float* global_scale, T* out, size_t n_units) {
+  const size_t u = static_cast<size_t>(blockIdx.x) * kFpBlock + threadIdx.x;
+  if (u >= n_units) {
+    return;
+  }
+  const float inv_scale_enc = *global_scale / kNvfp4Span;
+  const float s = from_fp8_bits(scales[u / 2]) * inv_scale_enc;
+  const uint32_t word = reinterpret_cast<const uint32_t*>(wq)[u];
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    v[i] = s * fp4_value((word >> (4 * i)) & 0xFu);
+  }
+  store8<T>(out + u * 8, v);
+}
+
 int check_mode(const char* who, int mode, int dtype, size_t n_elems) {
   if (mode != MLXROCM_MXFP4 && mode != MLXROCM_MXFP8 && mode != MLXROCM_NVFP4) {
     return fail(MLXROCM_INVALID_ARGUMENT, "[%s] unknown quantization mode %d", who, mode);
@@ -478,5 +561,118 @@ extern "C" int mlxrocm_fp_quantize_dequantize(
       MLXROCM_HIP_TRY(hipGetLastError());
       return static_cast<int>(MLXROCM_OK);
     });
+  });
+}
+
+namespace {
+
+// Shared argument checks of the nvfp4 entry points that take a tensor-wide scale.
+int check_global(const char* who, int dtype, size_t n_elems, const void* global_scale, size_t* blocks) {
+  int rc = check_mode(who, MLXROCM_NVFP4, dtype, n_elems);
+  if (rc != MLXROCM_OK) {
+    return rc;
+  }
+  if (global_scale == nullptr || (reinterpret_cast<uintptr_t>(global_scale) & 3u) != 0) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[%s] global_scale must point at one float32 on the device", who);
+  }
+  *blocks = (n_elems / 8 + kFpBlock - 1) / kFpBlock;
+  if (*blocks > 0x7fffffffull) {
+    return fail(MLXROCM_UNSUPPORTED, "[%s] %zu elements exceed the grid", who, n_elems);
+  }
+  return MLXROCM_OK;
+}
+
+} // namespace
+
+extern "C" int mlxrocm_nvfp4_quantize_global(
+    const void* w,
+    const float* global_scale,
+    uint32_t* wq,
+    uint8_t* scales,
+    size_t n_elems,
+    int dtype,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_nvfp4_quantize_global");
+  size_t blocks = 0;
+  int rc = check_global("quantize", dtype, n_elems, global_scale, &blocks);
+  if (rc != MLXROCM_OK || n_elems == 0) {
+    return rc;
+  }
+  if (!w || !wq || !scales) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[quantize] null device pointer");
+  }
+  if ((reinterpret_cast<uintptr_t>(w) & 15u) || (reinterpret_cast<uintptr_t>(wq) & 7u)) {
+    return fail(MLXROCM_UNSUPPORTED, "[quantize] operand pointers must be 16-byte aligned");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dispatch_dtype(dtype, [&](auto tval) {
+    using T = decltype(tval);
+    nvfp4_global_quantize_kernel<T, 0><<<static_cast<unsigned>(blocks), kFpBlock, 0, s>>>(
+        static_cast<const T*>(w), global_scale, reinterpret_cast<uint8_t*>(wq), scales, nullptr,
+        n_elems / 8);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
+  });
+}
+
+extern "C" int mlxrocm_nvfp4_dequantize_global(
+    const uint32_t* wq,
+    const uint8_t* scales,
+    const float* global_scale,
+    void* out,
+    size_t n_elems,
+    int dtype,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_nvfp4_dequantize_global");
+  size_t blocks = 0;
+  int rc = check_global("dequantize", dtype, n_elems, global_scale, &blocks);
+  if (rc != MLXROCM_OK || n_elems == 0) {
+    return rc;
+  }
+  if (!wq || !scales || !out) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[dequantize] null device pointer");
+  }
+  if ((reinterpret_cast<uintptr_t>(out) & 15u) || (reinterpret_cast<uintptr_t>(wq) & 7u)) {
+    return fail(MLXROCM_UNSUPPORTED, "[dequantize] operand pointers must be 16-byte aligned");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dispatch_dtype(dtype, [&](auto tval) {
+    using T = decltype(tval);
+    nvfp4_global_dequantize_kernel<T><<<static_cast<unsigned>(blocks), kFpBlock, 0, s>>>(
+        reinterpret_cast<const uint8_t*>(wq), scales, global_scale, static_cast<T*>(out),
+        n_elems / 8);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
+  });
+}
+
+extern "C" int mlxrocm_nvfp4_quantize_dequantize_global(
+    const void* x,
+    const float* global_scale,
+    void* out,
+    size_t n_elems,
+    int dtype,
+    mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_nvfp4_quantize_dequantize_global");
+  size_t blocks = 0;
+  int rc = check_global("quantize_dequantize", dtype, n_elems, global_scale, &blocks);
+  if (rc != MLXROCM_OK || n_elems == 0) {
+    return rc;
+  }
+  if (!x || !out) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[quantize_dequantize] null device pointer");
+  }
+  if ((reinterpret_cast<uintptr_t>(x) & 15u) || (reinterpret_cast<uintptr_t>(out) & 15u)) {
+    return fail(MLXROCM_UNSUPPORTED, "[quantize_dequantize] operand pointers must be 16-byte aligned");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MLXROCM_REHEARSE("nvfp4_global_quantize_dequantize");
+  return dispatch_dtype(dtype, [&](auto tval) {
+    using T = decltype(tval);
+    nvfp4_global_quantize_kernel<T, 1><<<static_cast<unsigned>(blocks), kFpBlock, 0, s>>>(
+        static_cast<const T*>(x), global_scale, nullptr, nullptr, static_cast<T*>(out),
+        n_elems / 8);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
   });
 }

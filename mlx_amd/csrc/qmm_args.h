@@ -49,6 +49,11 @@ struct QmmArgs {
   const uint32_t* w_alt;
   const void* scales_alt;
   const void* biases_alt;
+  // nvfp4 weights quantized with a tensor-wide scale (one float on the device):
+  // the fp32 sums are multiplied by *out_scale / (448 * 6) before they are
+  // rounded (mlx/backend/cuda/quantized/qmm/qmv.cu:163-165).  Null otherwise;
+  // read only by the kernels of the floating-point modes with groups of 16.
+  const float* out_scale;
 };
 
 // Resolved operand pointers of problem l.  `valid` is false when a gathered

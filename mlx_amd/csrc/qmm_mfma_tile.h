@@ -103,6 +103,7 @@ constexpr int wstore_at(int m, int ns) {
 // FP != 0: the codes are e2m1 / e4m3 numbers (FpPairDequant's modes) instead of
 // affine integers; the pair image then holds, per 32 codes, the scale of the
 // first 16 in the low half and of the last 16 in the high half (gs_shift == 5).
+// FP == 3 (nvfp4) also honours QmmArgs::out_scale.
 template <typename T, typename TS, typename TO, int BITS, int NT, bool GROUPED, bool WN = false,
           bool SBI = false, int FP = 0>
 __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
@@ -650,6 +651,24 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   // stay allocated until the wait
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   QMM_PIN_W();
+  if constexpr (FP == 3) {
+    // nvfp4 weights quantized with a tensor-wide scale: the fp32 sums (of a K
+    // range, when K is split: the factor distributes over the ranges) take the
+    // factor before they are rounded
+    if (a.out_scale != nullptr) {
+      const float out_factor = *a.out_scale / (448.0f * 6.0f);
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            acc[i][j][r] *= out_factor;
+          }
+        }
+      }
+    }
+  }
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
     __syncthreads(); // LDS is free: K loop (pass 0) or the previous half is done

@@ -77,26 +77,24 @@ def _check_fp_params(tag: str, mode: str, group_size: int, bits: int) -> None:
         )
 
 
-def _no_global_scale(tag: str, mode: str, *global_scales) -> None:
-    # validate_global_scale, mlx/ops.cpp:4756-4782
-    for g in global_scales:
-        if g is None:
-            continue
-        if mode != "nvfp4":
-            raise ValueError(
-                f"[{tag}] Global scale is only supported for 'nvfp4' quantization mode."
-            )
-        if g.numel() != 1:
-            raise ValueError(
-                f"[{tag}] Global scale must be a scalar but got shape {tuple(g.shape)}."
-            )
-        if g.dtype != torch.float32:
-            raise ValueError(
-                f"[{tag}] Global scale must have dtype float32 but got {g.dtype}."
-            )
-        raise RuntimeError(
-            f"[{tag}] nvfp4 with a global scale has no ROCm implementation."
+def _global_scale(tag: str, mode: str, g, like: torch.Tensor):
+    """validate_global_scale, mlx/ops.cpp:4756-4782; returns the scale as one
+    float32 on ``like``'s device, or None."""
+    if g is None:
+        return None
+    if mode != "nvfp4":
+        raise ValueError(
+            f"[{tag}] Global scale is only supported for 'nvfp4' quantization mode."
         )
+    if g.numel() != 1:
+        raise ValueError(
+            f"[{tag}] Global scale must be a scalar but got shape {tuple(g.shape)}."
+        )
+    if g.dtype != torch.float32:
+        raise ValueError(
+            f"[{tag}] Global scale must have dtype float32 but got {g.dtype}."
+        )
+    return g.detach().reshape(1).to(like.device).contiguous()
 
 
 def _validate_mode_with_type(tag, scales, biases, out_type, mode):
@@ -220,7 +218,7 @@ def quantize(
             f"quantization group size {group_size}. However the provided  matrix has "
             f"shape {tuple(w.shape)}"
         )
-    _no_global_scale("quantize", mode, global_scale)
+    gscale = _global_scale("quantize", mode, global_scale, w)
     if mode == "affine":
         _check_affine_params("quantize", group_size, bits)
     else:
@@ -234,6 +232,15 @@ def quantize(
     if mode != "affine":
         # fp_quantize, mlx/ops.cpp:5101-5205: two outputs, one scale byte per group
         scales = torch.empty(lead + (K // group_size,), dtype=torch.uint8, device=w.device)
+        if gscale is not None:
+            # the reference's GPU-only variant, mlx/backend/cuda/quantized/fp_quantize.cuh:147-215
+            _lib.check(
+                lib.mlxrocm_nvfp4_quantize_global(
+                    w.data_ptr(), gscale.data_ptr(), wq.data_ptr(), scales.data_ptr(), w.numel(),
+                    _DTYPE_CODE[w.dtype], _stream_ptr(w),
+                )
+            )
+            return wq, scales
         _lib.check(
             lib.mlxrocm_fp_quantize(
                 w.data_ptr(), wq.data_ptr(), scales.data_ptr(), w.numel(),
@@ -266,9 +273,9 @@ def dequantize(
     fp_dequantize :5342-5462)."""
     out_type, mode = _validate_mode_with_type("dequantize", scales, biases, dtype, mode)
     group_size, bits = _params_from_mode(mode, group_size, bits)
-    _no_global_scale("dequantize", mode, global_scale)
+    gscale = _global_scale("dequantize", mode, global_scale, w)
     if mode != "affine":
-        return _fp_dequantize(w, scales, group_size, bits, mode, out_type)
+        return _fp_dequantize(w, scales, group_size, bits, mode, out_type, gscale)
     if bits <= 0:
         raise ValueError(f"[dequantize] Invalid value for bits: {bits}")
     if group_size <= 0:
@@ -316,7 +323,7 @@ def dequantize(
     return _astype(out, out_type)  # astype, :5502-5505
 
 
-def _fp_dequantize(w, scales, group_size, bits, mode, out_type):
+def _fp_dequantize(w, scales, group_size, bits, mode, out_type, gscale=None):
     # fp_dequantize, mlx/ops.cpp:5342-5462
     if bits <= 0:
         raise ValueError(f"[dequantize] Invalid value for bits: {bits}")
@@ -344,6 +351,15 @@ def _fp_dequantize(w, scales, group_size, bits, mode, out_type):
     w = _contiguous(w)
     scales = _contiguous(scales)
     out = torch.empty(tuple(w.shape[:-1]) + (out_size,), dtype=out_type, device=w.device)
+    if gscale is not None:
+        # mlx/backend/cuda/quantized/fp_quantize.cuh:548-592
+        _lib.check(
+            lib.mlxrocm_nvfp4_dequantize_global(
+                w.data_ptr(), scales.data_ptr(), gscale.data_ptr(), out.data_ptr(), out.numel(),
+                _DTYPE_CODE[out_type], _stream_ptr(w),
+            )
+        )
+        return out
     _lib.check(
         lib.mlxrocm_fp_dequantize(
             w.data_ptr(), scales.data_ptr(), out.data_ptr(), out.numel(),
@@ -792,7 +808,8 @@ def qqmm(
             "[qqmm] For nvfp4 mode, either both global_scale_x and global_scale_w "
             "must be provided, or neither."
         )
-    _no_global_scale("qqmm", mode, global_scale_x, global_scale_w)
+    gx = _global_scale("qqmm", mode, global_scale_x, x)
+    gw = _global_scale("qqmm", mode, global_scale_w, x)
     _check_fp_params("qqmm", mode, group_size, bits)
     if w.dtype != torch.uint32:
         # extract_qqmm_dims, :4896-4924
@@ -801,7 +818,7 @@ def qqmm(
                 f"[qqmm] Last dimension of first input with shape {tuple(x.shape)} must "
                 f"match last dimension of second input with shape {tuple(w.shape)}."
             )
-        w, scales = quantize(_astype(w, x.dtype), group_size, bits, mode)
+        w, scales = quantize(_astype(w, x.dtype), group_size, bits, mode, global_scale=gw)
     else:
         _extract_dims("qqmm", x, w, scales, None, True, group_size, bits)
     if scales.dtype != torch.uint8:
@@ -817,14 +834,124 @@ def qqmm(
     out = torch.empty((M, N), dtype=xc.dtype, device=xc.device)
     ws_bytes = lib.mlxrocm_fp_qqmm_workspace_size(M, N, K, _MODE_CODE[mode], code)
     ws = torch.empty(max(int(ws_bytes), 256), dtype=torch.uint8, device=xc.device)
-    _lib.check(
-        lib.mlxrocm_fp_qqmm(
-            xc.data_ptr(), wc.data_ptr(), sc.data_ptr(), out.data_ptr(), M, N, K,
-            _MODE_CODE[mode], code, ws.data_ptr(), ws_bytes, _stream_ptr(xc),
+    if gx is not None:
+        _lib.check(
+            lib.mlxrocm_nvfp4_qqmm_global(
+                xc.data_ptr(), wc.data_ptr(), sc.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                out.data_ptr(), M, N, K, code, ws.data_ptr(), ws_bytes, _stream_ptr(xc),
+            )
         )
-    )
+    else:
+        _lib.check(
+            lib.mlxrocm_fp_qqmm(
+                xc.data_ptr(), wc.data_ptr(), sc.data_ptr(), out.data_ptr(), M, N, K,
+                _MODE_CODE[mode], code, ws.data_ptr(), ws_bytes, _stream_ptr(xc),
+            )
+        )
     if len(in_shape) > 2:
         return out.reshape(in_shape[:-1] + (out.shape[-1],))
     if len(in_shape) == 1:
         return out.squeeze(0)
+    return out
+
+
+def gather_qqmm(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    scales: Optional[torch.Tensor] = None,
+    lhs_indices: Optional[torch.Tensor] = None,
+    rhs_indices: Optional[torch.Tensor] = None,
+    group_size: Optional[int] = None,
+    bits: Optional[int] = None,
+    mode: str = "nvfp4",
+    global_scale_x: Optional[torch.Tensor] = None,
+    global_scale_w: Optional[torch.Tensor] = None,
+    sorted_indices: bool = False,
+):
+    """``mx.gather_qqmm`` (mlx/ops.cpp:5631-5681; GatherQQMM::eval_gpu,
+    mlx/backend/cuda/quantized/qqmm.cpp:210-281 -- the CPU backend has none):
+    every matrix of x is quantized and dequantized in its own type, then pair i
+    multiplies ``x_hat[lhs_indices[i]]`` by the transposed quantized
+    ``w[rhs_indices[i]]``.  A floating-point w is quantized first."""
+    mode = _mode("gather_qqmm", mode)
+    group_size, bits = _params_from_mode(mode, group_size, bits)
+    if mode == "affine":
+        raise ValueError("[gather_qqmm] Affine quantization is not supported for qqmm.")
+    if x.dtype not in _FLOATING:
+        raise ValueError(
+            "[gather_qqmm] Only real floating types except float64 are supported but "
+            f"first argument dtype == {x.dtype}."
+        )
+    if (global_scale_x is None) != (global_scale_w is None):
+        raise ValueError(
+            "[gather_qqmm] For nvfp4 mode, either both global_scale_x and global_scale_w "
+            "must be provided, or neither."
+        )
+    gx = _global_scale("gather_qqmm", mode, global_scale_x, x)
+    gw = _global_scale("gather_qqmm", mode, global_scale_w, x)
+    _check_fp_params("gather_qqmm", mode, group_size, bits)
+    if x.dim() < 2:
+        raise ValueError(
+            "[gather_qqmm] Input must have at least two dimensions but got input with "
+            f"shape {tuple(x.shape)}."
+        )
+    if w.dtype != torch.uint32:
+        # extract_qqmm_dims, mlx/ops.cpp:4896-4924
+        if w.dtype not in _FLOATING:
+            raise ValueError(
+                "[gather_qqmm] Only real floating types except float64 are supported but "
+                f"second argument dtype == {w.dtype}."
+            )
+        if x.shape[-1] != w.shape[-1]:
+            raise ValueError(
+                f"[gather_qqmm] Last dimension of first input with shape {tuple(x.shape)} must "
+                f"match last dimension of second input with shape {tuple(w.shape)}."
+            )
+        w, scales = quantize(_astype(w, x.dtype), group_size, bits, mode, global_scale=gw)
+    else:
+        if scales is None:
+            raise ValueError(
+                "[gather_qqmm] Scales must be provided if second argument is quantized."
+            )
+        _extract_dims("gather_qqmm", x, w, scales, None, True, group_size, bits)
+    if scales.dtype != torch.uint8:
+        raise ValueError(
+            f"[gather_qqmm] Scale type must be uint8 but received type {scales.dtype}."
+        )
+    w_outer = w.shape[-2]
+    lhs = _indices_or_default("[gather_qqmm]", lhs_indices, x)
+    rhs = _indices_or_default("[gather_qqmm]", rhs_indices, w)
+    _require_gpu("gather_qqmm", x, w, scales, lhs, rhs)
+    lib = _lib.load()
+    if lhs.shape != rhs.shape:
+        lhs, rhs = torch.broadcast_tensors(lhs, rhs)
+    M, K = x.shape[-2], x.shape[-1]
+    xb = _contiguous(x).reshape(-1, M, K)
+
+    def experts(t):
+        if t.dim() == 3 and _last_two_dense(t):
+            return t, t.stride(0)
+        t = _contiguous(t).reshape(-1, *t.shape[-2:])
+        return t, t.shape[-1] * t.shape[-2]
+
+    wb, w_stride = experts(w)
+    sb, sb_stride = experts(scales)
+    n_idx = rhs.numel()
+    lhs_u = _as_uint32(lhs) if n_idx else lhs.reshape(-1)
+    rhs_u = _as_uint32(rhs) if n_idx else rhs.reshape(-1)
+    out = torch.empty(tuple(rhs.shape) + (M, w_outer), dtype=x.dtype, device=x.device)
+    code = _DTYPE_CODE[x.dtype]
+    ws_bytes = lib.mlxrocm_fp_gather_qqmm_workspace_size(M, K, xb.shape[0], code)
+    ws = torch.empty(max(int(ws_bytes), 256), dtype=torch.uint8, device=x.device)
+    _lib.check(
+        lib.mlxrocm_fp_gather_qqmm(
+            xb.data_ptr(), wb.data_ptr(), sb.data_ptr(),
+            lhs_u.data_ptr() if n_idx else None, rhs_u.data_ptr() if n_idx else None,
+            gx.data_ptr() if gx is not None else None,
+            gw.data_ptr() if gw is not None else None,
+            out.data_ptr(), M, w_outer, K, n_idx, xb.shape[0], wb.shape[0],
+            M * K, w_stride, sb_stride, _MODE_CODE[mode], code,
+            ws.data_ptr(), ws_bytes, _stream_ptr(x),
+        )
+    )
     return out

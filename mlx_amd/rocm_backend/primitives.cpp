@@ -85,7 +85,6 @@ ROCM_NO_UNARY(Negative)
 ROCM_NO_UNARY(NotEqual)
 ROCM_NO_UNARY(Partition)
 ROCM_NO_UNARY(Power)
-ROCM_NO_UNARY(GatherQQMM)
 ROCM_NO_UNARY(RandomBits)
 ROCM_NO_UNARY(Real)
 ROCM_NO_UNARY(Reduce)

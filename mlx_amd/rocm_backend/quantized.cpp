@@ -1,5 +1,5 @@
 // quantized.cpp -- eval_gpu of the quantization primitives for the ROCm
-// backend: QuantizedMatmul, QQMatmul, GatherQMM and fast::Quantize
+// backend: QuantizedMatmul, QQMatmul, GatherQMM, GatherQQMM and fast::Quantize
 // (mlx/primitives.h:1616-1717, mlx/fast_primitives.h:337-371), in the affine
 // mode and the floating-point modes mxfp4 / mxfp8 / nvfp4.
 //
@@ -55,13 +55,9 @@ int fp_mode_code(QuantizationMode mode) {
 }
 
 // nvfp4 takes an optional tensor-wide scale as a trailing input
-// (mlx/ops.cpp:5124-5128, 5393-5397): not implemented by these kernels.
-void no_global_scale(bool present, const char* who) {
-  if (present) {
-    std::ostringstream msg;
-    msg << "[" << who << "] nvfp4 with a global scale has no ROCm implementation.";
-    throw std::runtime_error(msg.str());
-  }
+// (mlx/ops.cpp:5124-5128, 5393-5397, 4966-4969): one float32 on the device.
+const float* global_scale_ptr(const array& g, rocm::CommandEncoder& enc) {
+  return rocm::gpu_ptr<float>(g, enc.stream());
 }
 
 array ensure_row_contiguous(
@@ -225,6 +221,42 @@ void QuantizedMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
       enc.stream()));
 }
 
+namespace {
+
+// mx.quantize of a floating-point second operand inside qqmm / gather_qqmm,
+// with the tensor-wide scale when there is one (quantize_input,
+// mlx/backend/cuda/quantized/qqmm.cpp:17-54).
+void quantize_weights(
+    const array& w,
+    array& wq,
+    array& scales,
+    const float* global_scale,
+    int mode,
+    int dt,
+    rocm::CommandEncoder& enc) {
+  if (global_scale != nullptr) {
+    rocm::check(mlxrocm_nvfp4_quantize_global(
+        rocm::gpu_ptr<void>(w, enc.stream()),
+        global_scale,
+        rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+        rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+        w.size(),
+        dt,
+        enc.stream()));
+    return;
+  }
+  rocm::check(mlxrocm_fp_quantize(
+      rocm::gpu_ptr<void>(w, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+      rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+      w.size(),
+      mode,
+      dt,
+      enc.stream()));
+}
+
+} // namespace
+
 // x is quantized and dequantized on the fly in its own type, then multiplied by
 // the transposed quantized w: what QQMatmul::eval_cpu does for one row of x
 // (mlx/backend/cpu/quantized.cpp:1322-1360), here for any number of rows.  A
@@ -237,7 +269,12 @@ void QQMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
     throw std::runtime_error("[qqmm] Affine quantization is not supported.");
   }
   const bool w_quantized = inputs[1].dtype() == uint32;
-  no_global_scale(inputs.size() > (w_quantized ? 3u : 2u), "qqmm");
+  // nvfp4: {..., global_scale_x, global_scale_w} may follow (mlx/ops.cpp:4966-4969)
+  const size_t base_size = w_quantized ? 3u : 2u;
+  const bool has_global_scales =
+      mode_ == QuantizationMode::Nvfp4 && inputs.size() == base_size + 2;
+  const float* gx = has_global_scales ? global_scale_ptr(inputs[base_size], enc) : nullptr;
+  const float* gw = has_global_scales ? global_scale_ptr(inputs[base_size + 1], enc) : nullptr;
   const int mode = fp_mode_code(mode_);
 
   array x = ensure_row_contiguous(inputs[0], enc, s);
@@ -261,14 +298,7 @@ void QQMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
     scales.set_data(allocator::malloc(scales.nbytes()));
     enc.add_temporary(wq);
     enc.add_temporary(scales);
-    rocm::check(mlxrocm_fp_quantize(
-        rocm::gpu_ptr<void>(w, enc.stream()),
-        rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
-        rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
-        w.size(),
-        mode,
-        dt,
-        enc.stream()));
+    quantize_weights(w, wq, scales, gw, mode, dt, enc);
     w = wq;
   }
 
@@ -283,6 +313,23 @@ void QQMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
     enc.add_temporary(ws);
     ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
   }
+  if (has_global_scales) {
+    rocm::check(mlxrocm_nvfp4_qqmm_global(
+        rocm::gpu_ptr<void>(x, enc.stream()),
+        rocm::gpu_ptr<uint32_t>(w, enc.stream()),
+        rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+        gx,
+        gw,
+        rocm::gpu_ptr<void>(out, enc.stream()),
+        static_cast<int>(rows),
+        N,
+        K,
+        dt,
+        ws_ptr,
+        ws_bytes,
+        enc.stream()));
+    return;
+  }
   rocm::check(mlxrocm_fp_qqmm(
       rocm::gpu_ptr<void>(x, enc.stream()),
       rocm::gpu_ptr<uint32_t>(w, enc.stream()),
@@ -291,6 +338,91 @@ void QQMatmul::eval_gpu(const std::vector<array>& inputs, array& out) {
       static_cast<int>(rows),
       N,
       K,
+      mode,
+      dt,
+      ws_ptr,
+      ws_bytes,
+      enc.stream()));
+}
+
+// gather_qqmm (mlx/ops.cpp:5631-5681): inputs {x, w, lhs, rhs [, scales_w]
+// [, global_scale_x, global_scale_w]}.  Every matrix of x is quantized and
+// dequantized in its own type inside the call, then gathered pairs are
+// multiplied, as GatherQQMM::eval_gpu of the CUDA backend does
+// (mlx/backend/cuda/quantized/qqmm.cpp:210-281).
+void GatherQQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
+  auto& s = stream();
+  auto& enc = rocm::get_command_encoder(s);
+  if (mode_ == QuantizationMode::Affine) {
+    throw std::runtime_error("[gather_qqmm] Affine quantization is not supported.");
+  }
+  const bool w_quantized = inputs[1].dtype() == uint32;
+  const size_t base_size = w_quantized ? 5u : 4u;
+  const bool has_global_scales =
+      mode_ == QuantizationMode::Nvfp4 && inputs.size() == base_size + 2;
+  const float* gx = has_global_scales ? global_scale_ptr(inputs[base_size], enc) : nullptr;
+  const float* gw = has_global_scales ? global_scale_ptr(inputs[base_size + 1], enc) : nullptr;
+  const int mode = fp_mode_code(mode_);
+
+  array x = ensure_row_contiguous(inputs[0], enc, s);
+  array w = ensure_row_contiguous(inputs[1], enc, s);
+  array lhs = ensure_row_contiguous(inputs[2], enc, s);
+  array rhs = ensure_row_contiguous(inputs[3], enc, s);
+  const int K = x.shape(-1);
+  const int M = x.shape(-2);
+  const int N = out.shape(-1);
+  const int dt = dtype_code(x.dtype(), "gather_qqmm");
+
+  array scales = w_quantized ? ensure_row_contiguous(inputs[4], enc, s) : w;
+  if (!w_quantized) {
+    if (w.dtype() != x.dtype()) {
+      throw std::runtime_error("[gather_qqmm] x and a floating-point w must share one type");
+    }
+    auto q_shape = w.shape();
+    q_shape.back() = K * bits_ / 32;
+    auto s_shape = w.shape();
+    s_shape.back() = K / group_size_;
+    array wq(q_shape, uint32, nullptr, {});
+    scales = array(s_shape, uint8, nullptr, {});
+    wq.set_data(allocator::malloc(wq.nbytes()));
+    scales.set_data(allocator::malloc(scales.nbytes()));
+    enc.add_temporary(wq);
+    enc.add_temporary(scales);
+    quantize_weights(w, wq, scales, gw, mode, dt, enc);
+    w = wq;
+  }
+
+  out.set_data(allocator::malloc(out.nbytes()));
+  const int n_idx = static_cast<int>(lhs.size());
+  const int x_batches = (M == 0 || K == 0) ? 0 : static_cast<int>(x.size() / (size_t(K) * M));
+  const int n_experts = (N == 0 || w.shape(-1) == 0)
+      ? 0
+      : static_cast<int>(w.size() / (size_t(w.shape(-1)) * w.shape(-2)));
+  const size_t ws_bytes = mlxrocm_fp_gather_qqmm_workspace_size(M, K, x_batches, dt);
+  void* ws_ptr = nullptr;
+  if (ws_bytes > 0) {
+    array ws = workspace_array(ws_bytes);
+    enc.add_temporary(ws);
+    ws_ptr = rocm::gpu_ptr<void>(ws, enc.stream());
+  }
+  rocm::check(mlxrocm_fp_gather_qqmm(
+      rocm::gpu_ptr<void>(x, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(w, enc.stream()),
+      rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(lhs, enc.stream()),
+      rocm::gpu_ptr<uint32_t>(rhs, enc.stream()),
+      gx,
+      gw,
+      rocm::gpu_ptr<void>(out, enc.stream()),
+      M,
+      N,
+      K,
+      n_idx,
+      x_batches,
+      n_experts,
+      int64_t(M) * K,
+      int64_t(N) * w.shape(-1),
+      int64_t(N) * scales.shape(-1),
       mode,
       dt,
       ws_ptr,
@@ -404,11 +536,21 @@ void fast::Quantize::eval_gpu(
     // {wq, scales [, global_scale]} -> {w} (mlx/ops.cpp:5124-5128, 5393-5397)
     const int mode = fp_mode_code(mode_);
     if (dequantize_) {
-      no_global_scale(inputs.size() > 2, "dequantize");
       array wq = ensure_row_contiguous(inputs[0], enc, s);
       array scales = ensure_row_contiguous(inputs[1], enc, s);
       array& w = outputs[0];
       w.set_data(allocator::malloc(w.nbytes()));
+      if (inputs.size() > 2) {
+        rocm::check(mlxrocm_nvfp4_dequantize_global(
+            rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+            rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+            global_scale_ptr(inputs[2], enc),
+            rocm::gpu_ptr<void>(w, enc.stream()),
+            w.size(),
+            dtype_code(w.dtype(), "dequantize"),
+            enc.stream()));
+        return;
+      }
       rocm::check(mlxrocm_fp_dequantize(
           rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
           rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
@@ -418,12 +560,22 @@ void fast::Quantize::eval_gpu(
           dtype_code(w.dtype(), "dequantize"),
           enc.stream()));
     } else {
-      no_global_scale(inputs.size() > 1, "quantize");
       array w = ensure_row_contiguous(inputs[0], enc, s);
       array& wq = outputs[0];
       array& scales = outputs[1];
       wq.set_data(allocator::malloc(wq.nbytes()));
       scales.set_data(allocator::malloc(scales.nbytes()));
+      if (inputs.size() > 1) {
+        rocm::check(mlxrocm_nvfp4_quantize_global(
+            rocm::gpu_ptr<void>(w, enc.stream()),
+            global_scale_ptr(inputs[1], enc),
+            rocm::gpu_ptr<uint32_t>(wq, enc.stream()),
+            rocm::gpu_ptr<uint8_t>(scales, enc.stream()),
+            w.size(),
+            dtype_code(w.dtype(), "quantize"),
+            enc.stream()));
+        return;
+      }
       rocm::check(mlxrocm_fp_quantize(
           rocm::gpu_ptr<void>(w, enc.stream()),
           rocm::gpu_ptr<uint32_t>(wq, enc.stream()),

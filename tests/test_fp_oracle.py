@@ -227,3 +227,113 @@ def test_matmul_matches_the_golden_vectors(port, golden, mode, dname, transpose)
     want = tensor("_y", dtype)
     got = port.port_qmm(x, wq, scales, mode, transpose)
     assert torch.equal(qref_raw(got), qref_raw(want)), tag
+
+
+# ---- nvfp4 with a tensor-wide scale (numpy restatement of the CUDA kernels) ----
+
+def test_global_scale_converters_match_the_port_and_the_definition(port):
+    """The numpy e4m3 / e2m1 rounding used by the tensor-wide-scale functions
+    against the C port (itself checked against the reference's converters) and
+    against the formats' definition: no table entry is nearer."""
+    import numpy as np
+
+    rs = np.random.RandomState(3)
+    vals = np.abs(rs.randn(4000).astype(np.float32)) * np.exp(rs.randn(4000).astype(np.float32) * 3)
+    table = fp_qref._e4m3_values()[:127].numpy()
+    mid = ((table[:-1] + table[1:]) / 2).astype(np.float32)
+    vals = np.concatenate([vals, table.astype(np.float32), mid, np.float32([0, 447.9, 448, 464, 1e9])])
+    mine = fp_qref.e4m3_round(vals)
+    theirs = np.array([port.port.fpq_to_fp8(float(v)) for v in vals], dtype=np.uint8)
+    assert np.array_equal(mine, theirs)
+    err = np.abs(table[mine] - np.minimum(vals, 448).astype(np.float64))
+    assert np.all(err <= np.abs(table[None, :] - np.minimum(vals, 448)[:, None]).min(axis=1))
+
+    v4 = np.concatenate([
+        (rs.randn(4000) * 3).astype(np.float32),
+        np.float32([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5, -0.25, -0.75, -5, 7, -7, 0, -0.0,
+                    np.inf, -np.inf, np.nan])])
+    mine = fp_qref.e2m1_round(v4)
+    theirs = np.array([port.port.fpq_e2m1(float(v)) for v in v4], dtype=np.uint8)
+    assert np.array_equal(mine, theirs)
+    # ties go to the code with an even mantissa bit
+    assert list(fp_qref.e2m1_round(np.float32([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5]))) == \
+        [0, 2, 2, 4, 4, 6, 6]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_global_scale_quantize_picks_nearest_codes_and_round_trips(dtype):
+    """Every code is a nearest e2m1 value of w * scale_enc / scale (float64 check,
+    independent of the rounding routine); the scale byte is the nearest e4m3 of
+    amax / 6 * scale_enc; dequantize inverts up to the two fp32 roundings."""
+    import numpy as np
+
+    g = torch.Generator().manual_seed(9)
+    w = (torch.randn(32, 256, generator=g) * torch.exp(torch.randn(32, 1, generator=g))).to(dtype)
+    w[3, :16] = 0
+    gs = float(w.float().abs().max())
+    wq, scales = fp_qref.nvfp4_global_quantize(w, gs)
+    assert wq.shape == (32, 32) and scales.shape == (32, 16)
+    scale_enc = np.float32(np.float32(2688.0) / np.float32(gs))
+    amax = w.float().reshape(32, 16, 16).abs().amax(-1).numpy()
+    want = np.float32(np.float32(amax / np.float32(6)) * scale_enc)
+    table = fp_qref._e4m3_values()[:127].numpy()
+    sv = table[scales.numpy()]
+    assert np.all(np.abs(sv - want) <= np.abs(table[None, None, :] - want[..., None]).min(-1))
+    raw = wq.view(torch.uint8).numpy()
+    codes = np.stack((raw & 0xF, raw >> 4), -1).reshape(32, 16, 16)
+    vals = np.array(fp_qref.FP4_VALUES)[codes]
+    live = sv > 0
+    scaled = w.float().reshape(32, 16, 16).numpy().astype(np.float64) * \
+        np.float32(scale_enc / np.where(live, sv, 1).astype(np.float32))[..., None]
+    grid = np.array(fp_qref.FP4_VALUES[:8] + tuple(-v for v in fp_qref.FP4_VALUES[:8]))
+    best = np.abs(grid[None, None, None, :] - np.clip(scaled, -6, 6)[..., None]).min(-1)
+    # the kernels round the product to float32 before they pick the code: a product
+    # within an fp32 ulp of a midpoint may take either neighbour
+    slack = 2.0 ** -22 * np.abs(scaled)
+    assert np.all((np.abs(vals - np.clip(scaled, -6, 6)) <= best + slack)[live])
+    # a group of zeros: scale byte 0, decodes to zeros whatever the codes are
+    assert scales[3, 0] == 0
+    back = fp_qref.nvfp4_global_dequantize(wq, scales, gs, dtype)
+    assert torch.all(back[3, :16] == 0)
+    # half a code step at the top of the range (1 of 6) plus the e4m3 rounding of the scale
+    err = (back.float() - w.float()).reshape(32, 16, 16).abs().amax(-1)
+    assert torch.all(err <= torch.from_numpy(amax) * (1 / 6 + 1 / 16) + 1e-30)
+
+
+def test_global_scale_round_trip_of_the_reference_test(port):
+    """python/tests/test_quantized.py:124-190: table values with a 6 in every
+    group, + 3e-6, bfloat16; with global_scale = max |w| the round trip is within
+    1e-5 (the assertion of the reference's test)."""
+    g = torch.Generator().manual_seed(1)
+    lut = torch.tensor(fp_qref.FP4_VALUES)
+    w = lut[torch.randint(0, 16, (128, 512), generator=g)].reshape(-1, 16)
+    w[:, 0] = 6
+    w = (w + 3e-6).to(torch.bfloat16).reshape(128, 512)
+    gs = float(w.float().abs().max())
+    wq, scales = fp_qref.nvfp4_global_quantize(w, gs)
+    back = fp_qref.nvfp4_global_dequantize(wq, scales, gs, torch.bfloat16)
+    assert torch.allclose(w.float(), back.float(), rtol=1e-5, atol=1e-5)
+    zeros = torch.zeros(8, 64)
+    wq, scales = fp_qref.nvfp4_global_quantize(zeros, 1.0)
+    assert torch.all(fp_qref.nvfp4_global_dequantize(wq, scales, 1.0) == 0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_global_scale_reduces_to_the_reference_rules_for_power_of_two_scales(port, dtype):
+    """With global_scale = 448 * 6 the encode scale is 1, and for groups whose
+    maximum is 6 * 2^k every intermediate is exact: quantize-dequantize must then
+    equal the reference's CPU fp_quantize_dequantize (same e4m3 scale, same
+    ties-to-even codes)."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(64, 128, generator=g).reshape(-1, 16)
+    x = x / x.abs().amax(-1, keepdim=True) * 6  # every group's maximum is 6 ...
+    x = x * torch.exp2(torch.randint(-4, 5, (x.shape[0], 1), generator=g).float())  # ... times 2^k
+    x = x.reshape(64, 128).to(dtype)
+    amax = x.float().reshape(-1, 16).abs().amax(-1)
+    assert torch.all(torch.log2(amax / 6) == torch.round(torch.log2(amax / 6)))
+    got = fp_qref.nvfp4_global_quantize_dequantize(x, 2688.0)
+    want = port.quantize_dequantize(x, "nvfp4")
+    assert torch.equal(got.float(), want.float())
+    # and the codes / scale bytes equal those of dequantize(quantize()) at that scale
+    wq, scales = fp_qref.nvfp4_global_quantize(x, 2688.0)
+    assert torch.equal(fp_qref.nvfp4_global_dequantize(wq, scales, 2688.0, dtype).float(), got.float())

@@ -6,6 +6,7 @@ reference's translation unit where it was built) within the stated tolerance
 and against an fp64 product of the exactly decoded weights.  Cases follow
 python/tests/test_quantized.py:41-181 (quantize / dequantize per mode),
 :183-237 (qqmm), :300-360 (fp_qmm shapes), :1180-1266 (gather)."""
+import itertools
 import os
 
 import pytest
@@ -478,3 +479,215 @@ def test_fp_abi_rejects_bad_arguments(gpu):
         == _lib.INVALID_ARGUMENT
     # nothing to do
     assert lib.mlxrocm_fp_quantize(None, None, None, 0, _lib.MXFP4, 0, None) == _lib.OK
+
+
+# ---- nvfp4 with a tensor-wide scale, gather_qqmm ------------------------------
+# The reference has these on the GPU only (python/tests/test_quantized.py:183-190,
+# 192-300, 1268-1363), so the checker is the numpy restatement of the CUDA
+# kernels' fp32 arithmetic in oracle/fp_qref.py: codes, scale bytes and
+# dequantized elements bit for bit, products against float64.
+
+def _global_weights(dtype, seed):
+    """Rows of very different magnitude, a group of zeros, a group so small that
+    its scale underflows to the byte 0, and the tensor's maximum."""
+    w = _weights((40, 512), dtype, seed).float()
+    w[5, 32:48] = w.abs().max() * 1e-7
+    return w.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_nvfp4_global_scale_quantize_and_dequantize_bit_for_bit(gpu, dtype):
+    for seed, scale_of_max in ((31, 1.0), (32, 0.37), (33, 4.0)):
+        w = _global_weights(dtype, seed)
+        gs = float(w.float().abs().max()) * scale_of_max
+        gst = torch.tensor(gs, dtype=torch.float32)
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode="nvfp4", global_scale=gst.to(gpu))
+        want_q, want_s = fp_qref.nvfp4_global_quantize(w, gs)
+        assert torch.equal(scales.cpu(), want_s), (dtype, seed)
+        bad = (wq.cpu().view(torch.int32) != want_q.view(torch.int32)).sum().item()
+        assert bad == 0, (dtype, seed, bad)
+        assert (want_s == 0).any() and (want_s == 126).any() == (scale_of_max <= 1.0)
+        for out_dtype in DTYPES:
+            got = mlx_amd.dequantize(wq, scales, mode="nvfp4", dtype=out_dtype,
+                                     global_scale=gst)  # a host scalar is moved to the device
+            want = fp_qref.nvfp4_global_dequantize(want_q, want_s, gs, out_dtype)
+            assert got.dtype == out_dtype and _equal_bits(got.cpu(), want), (dtype, out_dtype, seed)
+    # every scale byte and code
+    g = torch.Generator().manual_seed(12)
+    wq = torch.randint(-2 ** 31, 2 ** 31, (32, 128), generator=g, dtype=torch.int64).to(torch.int32)
+    wq = wq.view(torch.uint32)
+    scales = (torch.arange(32 * 64, dtype=torch.int64).reshape(32, 64) % 127).to(torch.uint8)
+    got = mlx_amd.dequantize(wq.to(gpu), scales.to(gpu), mode="nvfp4", dtype=dtype,
+                             global_scale=torch.tensor(0.731, device=gpu))
+    assert _equal_bits(got.cpu(), fp_qref.nvfp4_global_dequantize(wq, scales, 0.731, dtype))
+
+
+def test_nvfp4_global_scale_round_trip_of_the_reference_test(gpu):
+    # python/tests/test_quantized.py:124-190
+    g = torch.Generator().manual_seed(1)
+    lut = torch.tensor(fp_qref.FP4_VALUES)
+    w = lut[torch.randint(0, 16, (128, 512), generator=g)].reshape(-1, 16)
+    w[:, 0] = 6
+    w = (w + 3e-6).to(torch.bfloat16).reshape(128, 512).to(gpu)
+    gs = w.abs().max().float()
+    wq, scales = mlx_amd.quantize(w, mode="nvfp4", global_scale=gs)
+    w_hat = mlx_amd.dequantize(wq, scales, group_size=16, bits=4, mode="nvfp4", global_scale=gs)
+    assert torch.allclose(w.float(), w_hat.float(), rtol=1e-5, atol=1e-5)
+    zeros = torch.zeros((256, 512), device=gpu)
+    wq, scales = mlx_amd.quantize(zeros, mode="nvfp4", global_scale=torch.ones((), device=gpu))
+    assert torch.all(mlx_amd.dequantize(wq, scales, mode="nvfp4",
+                                        global_scale=torch.ones((), device=gpu)) == 0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_nvfp4_global_scale_quantize_dequantize_bit_for_bit(gpu, dtype):
+    from mlx_amd import _lib
+    from mlx_amd.ops import _DTYPE_CODE
+
+    lib = _lib.load()
+    x = _global_weights(dtype, 41)
+    gs = float(x.float().abs().max())
+    xg, gst = x.to(gpu), torch.tensor([gs], dtype=torch.float32, device=gpu)
+    out = torch.empty_like(xg)
+    _lib.check(lib.mlxrocm_nvfp4_quantize_dequantize_global(
+        xg.data_ptr(), gst.data_ptr(), out.data_ptr(), xg.numel(), _DTYPE_CODE[dtype],
+        torch.cuda.current_stream().cuda_stream))
+    assert _equal_bits(out.cpu(), fp_qref.nvfp4_global_quantize_dequantize(x, gs)), dtype
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_qqmm_with_global_scales(gpu, dtype):
+    """python/tests/test_quantized.py:192-300 (test_qqmv, test_qqmm): shapes of
+    both tests plus shapes that take the tile kernel with and without a split K."""
+    half_ulp = {torch.float32: 2.0 ** -24, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    shapes = [(1, 256, 64), (1, 67, 512), (8, 128, 128), (32, 256, 256), (33, 128, 256),
+              (64, 256, 128), (5, 64, 48), (40, 96, 4096), (300, 520, 1024)]
+    for M, N, K in shapes:
+        g = torch.Generator().manual_seed(M * 7 + N)
+        x = torch.randn((M, K), generator=g).to(dtype)
+        w = torch.randn((N, K), generator=g).to(dtype)
+        gx, gw = x.float().abs().max(), w.float().abs().max()
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode="nvfp4", global_scale=gw.to(gpu))
+        got = mlx_amd.qqmm(x.to(gpu), wq, scales, mode="nvfp4",
+                           global_scale_x=gx.to(gpu), global_scale_w=gw.to(gpu))
+        assert got.shape == (M, N) and got.dtype == dtype
+        want, mag = fp_qref.nvfp4_global_qqmm_f64(x, wq.cpu(), scales.cpu(), float(gx), float(gw))
+        err = ((got.cpu().double() - want).abs() / (mag + 1e-30)).max().item()
+        assert err <= ACC_TOL[dtype] + half_ulp, (dtype, (M, N, K), err)
+        if dtype == torch.float32:
+            # the reference's own assertion: within 1e-3 of x_hat @ w_hat.T
+            x_hat = fp_qref.nvfp4_global_quantize_dequantize(x, float(gx)).double()
+            w_hat = fp_qref.nvfp4_global_dequantize(wq.cpu(), scales.cpu(), float(gw)).double()
+            assert (got.cpu().double() - x_hat @ w_hat.T).abs().max().item() < 1e-3
+        # a floating-point w is quantized inside the call, with its scale
+        got_w = mlx_amd.qqmm(x.to(gpu), w.to(gpu), mode="nvfp4",
+                             global_scale_x=gx.to(gpu), global_scale_w=gw.to(gpu))
+        assert torch.equal(got_w, got)
+    with pytest.raises(ValueError, match="either both"):
+        mlx_amd.qqmm(x.to(gpu), wq, scales, mode="nvfp4", global_scale_x=gx.to(gpu))
+
+
+_GATHER_QQMM_BATCHES = (
+    # python/tests/test_quantized.py:1275-1306
+    ((1,), (0,), (3,), (2, 1)),
+    ((1,), None, (3,), (2, 1)),
+    ((2,), None, (3,), (2, 1)),
+    ((3,), (0, 2), (1,), (0,)),
+    ((5,), (0, 2), (3,), (2, 1)),
+)
+
+
+@pytest.mark.parametrize("mode", ("nvfp4", "mxfp8", "mxfp4"))
+def test_gather_qqmm(fp_oracle, gpu, mode):
+    """python/tests/test_quantized.py:1268-1363: every pair against the float64
+    product of x_hat (the oracle's quantize-dequantize of that matrix of x) and
+    the exactly decoded expert; nvfp4 with both tensor-wide scales, as there."""
+    gsz = fp_qref.GROUP_SIZE[mode]
+    for (batch_a, lhs, batch_b, rhs), M, N, K in itertools.product(
+            _GATHER_QQMM_BATCHES, (1, 32), (32, 256), (32, 256)):
+        if K % gsz:
+            continue
+        g = torch.Generator().manual_seed(M + N + K + len(batch_a))
+        x = torch.randn(batch_a + (M, K), generator=g)
+        w = torch.randn(batch_b + (N, K), generator=g)
+        use_global = mode == "nvfp4"
+        gx = x.abs().max() if use_global else None
+        gw = w.abs().max() if use_global else None
+        kw = dict(global_scale=gw.to(gpu)) if use_global else {}
+        wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode, **kw)
+        li = None if lhs is None else torch.tensor(lhs, dtype=torch.int32, device=gpu)
+        ri = None if rhs is None else torch.tensor(rhs, dtype=torch.int32, device=gpu)
+        kw = dict(global_scale_x=gx.to(gpu), global_scale_w=gw.to(gpu)) if use_global else {}
+        got = mlx_amd.gather_qqmm(x.to(gpu), wq, scales, li, ri, mode=mode, **kw)
+        lhs_l = list(lhs) if lhs is not None else list(range(batch_a[0]))
+        rhs_l = list(rhs)
+        n = max(len(lhs_l), len(rhs_l))
+        lhs_l = lhs_l * (n // len(lhs_l))
+        rhs_l = rhs_l * (n // len(rhs_l))
+        assert got.shape == (n, M, N) and got.dtype == torch.float32
+        for i in range(n):
+            xi, e = x[lhs_l[i]], rhs_l[i]
+            if use_global:
+                want, mag = fp_qref.nvfp4_global_qqmm_f64(
+                    xi, wq[e].cpu(), scales[e].cpu(), float(gx), float(gw))
+            else:
+                x_hat = fp_oracle.quantize_dequantize(xi, mode).double()
+                w_hat = fp_qref.exact_fp_weights(wq[e].cpu(), scales[e].cpu(), mode)
+                want, mag = x_hat @ w_hat.T, x_hat.abs() @ w_hat.abs().T
+            err = ((got[i].cpu().double() - want).abs() / (mag + 1e-30)).max().item()
+            assert err <= ACC_TOL[torch.float32] + 2.0 ** -24, (mode, (M, N, K), i, err)
+        # a floating-point w is quantized inside the call
+        got_w = mlx_amd.gather_qqmm(x.to(gpu), w.to(gpu), None, li, ri, mode=mode, **kw)
+        assert torch.equal(got_w, got)
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16), ids=str)
+def test_gather_qqmm_sixteen_bit_and_bad_indices(fp_oracle, gpu, dtype):
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn((4, 3, 128), generator=g).to(dtype)
+    w = torch.randn((6, 72, 128), generator=g).to(dtype)
+    wq, scales = mlx_amd.quantize(w.to(gpu), mode="mxfp4")
+    lhs = torch.tensor([0, 3, 1, 2, 9, 0], dtype=torch.int64, device=gpu)   # 9: out of range
+    rhs = torch.tensor([5, 0, 2, 2, 1, 6], dtype=torch.int64, device=gpu)   # 6: out of range
+    got = mlx_amd.gather_qqmm(x.to(gpu), wq, scales, lhs, rhs, mode="mxfp4")
+    assert got.shape == (6, 3, 72) and got.dtype == dtype
+    assert torch.all(got[4] == 0) and torch.all(got[5] == 0)
+    half_ulp = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    for i in range(4):
+        x_hat = fp_oracle.quantize_dequantize(x[int(lhs[i])], "mxfp4").double()
+        w_hat = fp_qref.exact_fp_weights(wq[int(rhs[i])].cpu(), scales[int(rhs[i])].cpu(), "mxfp4")
+        err = ((got[i].cpu().double() - x_hat @ w_hat.T).abs() /
+               (x_hat.abs() @ w_hat.abs().T + 1e-30)).max().item()
+        assert err <= ACC_TOL[dtype] + half_ulp, (dtype, i, err)
+    # no pairs
+    none = mlx_amd.gather_qqmm(x.to(gpu), wq, scales, lhs[:0], rhs[:0], mode="mxfp4")
+    assert none.shape == (0, 3, 72)
+
+
+def test_global_scale_abi_rejects_bad_arguments(gpu):
+    from mlx_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device=gpu)
+    p = buf.data_ptr()
+    assert lib.mlxrocm_nvfp4_quantize_global(p, None, p, p, 64, 0, None) == _lib.INVALID_ARGUMENT
+    assert "global_scale" in _lib.last_error()
+    assert lib.mlxrocm_nvfp4_quantize_global(p, p, p, p, 40, 0, None) == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_nvfp4_dequantize_global(p, p, p + 2, p, 64, 0, None) == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_nvfp4_quantize_dequantize_global(p, p, p, 64, 9, None) == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_nvfp4_qqmm_global(p, p, p, p, None, p, 2, 8, 64, 0, p, 1 << 16, None) \
+        == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_nvfp4_qqmm_global(p, p, p, p, p, p, 2, 8, 64, 0, p, 16, None) \
+        == _lib.INVALID_ARGUMENT
+    assert "workspace" in _lib.last_error()
+    # gather_qqmm: one scale only; scales outside nvfp4; a workspace that is too small
+    args = (2, 8, 64, 1, 1, 1, 128, 0, 0)
+    assert lib.mlxrocm_fp_gather_qqmm(p, p, p, p, p, p, None, p, *args, _lib.NVFP4, 0, p, 1 << 16, None) \
+        == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_fp_gather_qqmm(p, p, p, p, p, p, p, p, *args, _lib.MXFP4, 0, p, 1 << 16, None) \
+        == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_fp_gather_qqmm(p, p, p, p, p, None, None, p, *args, _lib.MXFP4, 0, p, 16, None) \
+        == _lib.INVALID_ARGUMENT
+    assert lib.mlxrocm_fp_gather_qqmm_workspace_size(2, 64, 3, 0) == 2 * 64 * 3 * 4
+    # nothing to do
+    assert lib.mlxrocm_nvfp4_quantize_global(None, p, None, None, 0, 0, None) == _lib.OK

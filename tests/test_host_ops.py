@@ -141,7 +141,9 @@ def test_fp_mode_errors():
         mlx_amd.quantize(w, mode="mxfp8", global_scale=torch.ones(()))
     with pytest.raises(ValueError, match="scalar"):
         mlx_amd.quantize(w, mode="nvfp4", global_scale=torch.ones(2))
-    with pytest.raises(RuntimeError, match="global scale"):
+    with pytest.raises(ValueError, match="dtype float32"):
+        mlx_amd.quantize(w, mode="nvfp4", global_scale=torch.ones((), dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="GPU"):  # valid arguments: only the device is wrong
         mlx_amd.quantize(w, mode="nvfp4", global_scale=torch.ones(()))
 
 
@@ -164,3 +166,30 @@ def test_qqmm_errors():
         mlx_amd.qqmm(x, torch.zeros((8, 32)))
     with pytest.raises(RuntimeError, match="GPU"):
         mlx_amd.qqmm(x, wq, sc)
+
+
+def test_gather_qqmm_errors():
+    # gather_qqmm, mlx/ops.cpp:5631-5681 (extract_qqmm_dims :4896-4924)
+    x = torch.zeros((2, 4, 64))
+    wq = torch.zeros((3, 8, 8), dtype=torch.uint32)
+    sc = torch.zeros((3, 8, 4), dtype=torch.uint8)
+    idx = torch.zeros(2, dtype=torch.int32)
+    with pytest.raises(ValueError, match="Affine quantization is not supported"):
+        mlx_amd.gather_qqmm(x, wq, sc, rhs_indices=idx, mode="affine")
+    with pytest.raises(ValueError, match="Scales must be provided"):
+        mlx_amd.gather_qqmm(x, wq, rhs_indices=idx)
+    with pytest.raises(ValueError, match="first argument dtype"):
+        mlx_amd.gather_qqmm(x.to(torch.float64), wq, sc, rhs_indices=idx)
+    with pytest.raises(ValueError, match="either both"):
+        mlx_amd.gather_qqmm(x, wq, sc, rhs_indices=idx, global_scale_w=torch.ones(()))
+    with pytest.raises(ValueError, match="only supported for 'nvfp4'"):
+        mlx_amd.gather_qqmm(x, wq, sc, rhs_indices=idx, mode="mxfp4",
+                            global_scale_x=torch.ones(()), global_scale_w=torch.ones(()))
+    with pytest.raises(ValueError, match="must match last dimension"):
+        mlx_amd.gather_qqmm(x, torch.zeros((3, 8, 32)), rhs_indices=idx)
+    with pytest.raises(ValueError, match="integral"):
+        mlx_amd.gather_qqmm(x, wq, sc, rhs_indices=idx.float())
+    with pytest.raises(ValueError, match="at least two dimensions"):
+        mlx_amd.gather_qqmm(x[0, 0], wq, sc, rhs_indices=idx)
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.gather_qqmm(x, wq, sc, rhs_indices=idx)
