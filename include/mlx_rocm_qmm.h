@@ -289,6 +289,19 @@ int mlxrocm_fp_gather_qmm(
     mlxrocm_stream_t stream);
 
 /*
+ * mx.to_fp8 / mx.from_fp8 (mlx/ops.cpp:5519-5552; fast::ConvertFP8,
+ * mlx/backend/cpu/quantized.cpp:1282-1320 with detail::ToFP8 / FromFP8,
+ * mlx/backend/cpu/unary_ops.h:120-174): elementwise float <-> e4m3 bytes, round
+ * to nearest even, saturating at 448 (0x7E) with the sign carried over; the
+ * decoder has no NaN or infinity codes (0x7F is 480).  x / out in dtype, 16-byte
+ * aligned; the byte array 8-byte aligned; any n_elems.
+ */
+int mlxrocm_to_fp8(
+    const void* x, uint8_t* out, size_t n_elems, int dtype, mlxrocm_stream_t stream);
+int mlxrocm_from_fp8(
+    const uint8_t* x, void* out, size_t n_elems, int dtype, mlxrocm_stream_t stream);
+
+/*
  * gather_qqmm (mlx/ops.cpp:5631-5681; GPU only in the reference:
  * GatherQQMM::eval_gpu, mlx/backend/cuda/quantized/qqmm.cpp:210-281 -- the CPU
  * backend throws "NYI", mlx/backend/cpu/quantized.cpp:1362-1364): every matrix

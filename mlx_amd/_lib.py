@@ -69,6 +69,8 @@ SIGNATURES = {
     "mlxrocm_nvfp4_dequantize_global": (_i, [_p] * 4 + [_sz, _i, _p]),
     "mlxrocm_nvfp4_quantize_dequantize_global": (_i, [_p] * 3 + [_sz, _i, _p]),
     "mlxrocm_nvfp4_qqmm_global": (_i, [_p] * 6 + [_i] * 4 + [_p, _sz, _p]),
+    "mlxrocm_to_fp8": (_i, [_p, _p, _sz, _i, _p]),
+    "mlxrocm_from_fp8": (_i, [_p, _p, _sz, _i, _p]),
     "mlxrocm_qmm_kernel_name": (ctypes.c_char_p, [_i] * 8),
     "mlxrocm_qmm_plan": (_i, [_i] * 9 + [_sz, ctypes.c_char_p, _sz]),
     "mlxrocm_gather_qmm_plan": (_i, [_i] * 10 + [_sz, ctypes.c_char_p, _sz]),

@@ -389,6 +389,57 @@ __global__ __launch_bounds__(kFpBlock) void nvfp4_global_dequantize_kernel(
   store8<T>(out + u * 8, v);
 }
 
+// mx.to_fp8 / mx.from_fp8 (fast::ConvertFP8, mlx/backend/cpu/quantized.cpp:1282-1320
+// with detail::ToFP8 / FromFP8, mlx/backend/cpu/unary_ops.h:120-174).  One thread:
+// 8 consecutive elements; the tail of a length that is not a multiple of 8
+// element by element.
+template <typename T>
+__global__ __launch_bounds__(kFpBlock) void to_fp8_kernel(const T* x, uint8_t* out, size_t n) {
+  const size_t u = static_cast<size_t>(blockIdx.x) * kFpBlock + threadIdx.x;
+  const size_t first = u * 8;
+  if (first >= n) {
+    return;
+  }
+  if (first + 8 <= n) {
+    float v[8];
+    load8<T>(x + first, v);
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo |= to_fp8_bits(v[i]) << (8 * i);
+      hi |= to_fp8_bits(v[4 + i]) << (8 * i);
+    }
+    *reinterpret_cast<uint2*>(out + first) = make_uint2(lo, hi);
+  } else {
+    for (size_t i = first; i < n; ++i) {
+      out[i] = static_cast<uint8_t>(to_fp8_bits(to_f32(x[i])));
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kFpBlock) void from_fp8_kernel(const uint8_t* x, T* out, size_t n) {
+  const size_t u = static_cast<size_t>(blockIdx.x) * kFpBlock + threadIdx.x;
+  const size_t first = u * 8;
+  if (first >= n) {
+    return;
+  }
+  if (first + 8 <= n) {
+    const uint2 words = *reinterpret_cast<const uint2*>(x + first);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = from_fp8_bits((words.x >> (8 * i)) & 0xffu);
+      v[4 + i] = from_fp8_bits((words.y >> (8 * i)) & 0xffu);
+    }
+    store8<T>(out + first, v);
+  } else {
+    for (size_t i = first; i < n; ++i) {
+      out[i] = from_f32<T>(from_fp8_bits(x[i]));
+    }
+  }
+}
+
 int check_mode(const char* who, int mode, int dtype, size_t n_elems) {
   if (mode != MLXROCM_MXFP4 && mode != MLXROCM_MXFP8 && mode != MLXROCM_NVFP4) {
     return fail(MLXROCM_INVALID_ARGUMENT, "[%s] unknown quantization mode %d", who, mode);
@@ -672,6 +723,67 @@ extern "C" int mlxrocm_nvfp4_quantize_dequantize_global(
     nvfp4_global_quantize_kernel<T, 1><<<static_cast<unsigned>(blocks), kFpBlock, 0, s>>>(
         static_cast<const T*>(x), global_scale, nullptr, nullptr, static_cast<T*>(out),
         n_elems / 8);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
+  });
+}
+
+namespace {
+
+int check_convert(
+    const char* who, const void* wide, const void* bytes, size_t n, int dtype, size_t* blocks) {
+  if (!valid_dtype(dtype)) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[%s] unknown dtype %d", who, dtype);
+  }
+  *blocks = ((n + 7) / 8 + kFpBlock - 1) / kFpBlock;
+  if (n == 0) {
+    return MLXROCM_OK;
+  }
+  if (!wide || !bytes) {
+    return fail(MLXROCM_INVALID_ARGUMENT, "[%s] null device pointer", who);
+  }
+  if ((reinterpret_cast<uintptr_t>(wide) & 15u) || (reinterpret_cast<uintptr_t>(bytes) & 7u)) {
+    return fail(MLXROCM_UNSUPPORTED, "[%s] operand pointers must be 16-byte aligned", who);
+  }
+  if (*blocks > 0x7fffffffull) {
+    return fail(MLXROCM_UNSUPPORTED, "[%s] %zu elements exceed the grid", who, n);
+  }
+  return MLXROCM_OK;
+}
+
+} // namespace
+
+extern "C" int mlxrocm_to_fp8(
+    const void* x, uint8_t* out, size_t n_elems, int dtype, mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_to_fp8");
+  size_t blocks = 0;
+  int rc = check_convert("to_fp8", x, out, n_elems, dtype, &blocks);
+  if (rc != MLXROCM_OK || n_elems == 0) {
+    return rc;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dispatch_dtype(dtype, [&](auto tval) {
+    using T = decltype(tval);
+    to_fp8_kernel<T><<<static_cast<unsigned>(blocks), kFpBlock, 0, s>>>(
+        static_cast<const T*>(x), out, n_elems);
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return static_cast<int>(MLXROCM_OK);
+  });
+}
+
+extern "C" int mlxrocm_from_fp8(
+    const uint8_t* x, void* out, size_t n_elems, int dtype, mlxrocm_stream_t stream) {
+  mlxrocm::ApiRange api_range("mlxrocm_from_fp8");
+  size_t blocks = 0;
+  int rc = check_convert("from_fp8", out, x, n_elems, dtype, &blocks);
+  if (rc != MLXROCM_OK || n_elems == 0) {
+    return rc;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dispatch_dtype(dtype, [&](auto tval) {
+    using T = decltype(tval);
+    from_fp8_kernel<T><<<static_cast<unsigned>(blocks), kFpBlock, 0, s>>>(
+        x, static_cast<T*>(out), n_elems);
     MLXROCM_HIP_TRY(hipGetLastError());
     return static_cast<int>(MLXROCM_OK);
   });

@@ -955,3 +955,40 @@ def gather_qqmm(
         )
     )
     return out
+
+
+def to_fp8(x: torch.Tensor) -> torch.Tensor:
+    """``mx.to_fp8`` (mlx/ops.cpp:5539-5552): elementwise conversion to e4m3
+    bytes, round to nearest even, saturating at 448."""
+    if x.dtype not in _FLOATING:
+        raise ValueError(
+            f"[to_fp8] Only real floating types are supported but x.dtype() == {x.dtype}."
+        )
+    _require_gpu("to_fp8", x)
+    lib = _lib.load()
+    xc = _contiguous(x)
+    out = torch.empty(xc.shape, dtype=torch.uint8, device=xc.device)
+    _lib.check(
+        lib.mlxrocm_to_fp8(xc.data_ptr(), out.data_ptr(), xc.numel(), _DTYPE_CODE[xc.dtype],
+                           _stream_ptr(xc))
+    )
+    return out
+
+
+def from_fp8(x: torch.Tensor, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """``mx.from_fp8`` (mlx/ops.cpp:5519-5537): e4m3 bytes to ``dtype``."""
+    if x.dtype != torch.uint8:
+        raise ValueError(f"[from_fp8] Input must have type uint8 but x.dtype() == {x.dtype}.")
+    if dtype not in _FLOATING:
+        raise ValueError(
+            f"[from_fp8] Only real floating types are supported but dtype == {dtype}."
+        )
+    _require_gpu("from_fp8", x)
+    lib = _lib.load()
+    xc = _contiguous(x)
+    out = torch.empty(xc.shape, dtype=dtype, device=xc.device)
+    _lib.check(
+        lib.mlxrocm_from_fp8(xc.data_ptr(), out.data_ptr(), xc.numel(), _DTYPE_CODE[dtype],
+                             _stream_ptr(xc))
+    )
+    return out

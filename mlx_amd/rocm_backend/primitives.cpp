@@ -122,7 +122,6 @@ namespace fast {
 ROCM_NO_MULTI(RMSNormVJP)
 ROCM_NO_MULTI(LayerNormVJP)
 ROCM_NO_MULTI(ScaledDotProductAttentionVJP)
-ROCM_NO_MULTI(ConvertFP8)
 ROCM_NO_MULTI(CustomKernel)
 ROCM_NO_MULTI(RMSNorm)
 ROCM_NO_MULTI(LayerNorm)

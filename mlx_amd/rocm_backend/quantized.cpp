@@ -1,5 +1,6 @@
 // quantized.cpp -- eval_gpu of the quantization primitives for the ROCm
-// backend: QuantizedMatmul, QQMatmul, GatherQMM, GatherQQMM and fast::Quantize
+// backend: QuantizedMatmul, QQMatmul, GatherQMM, GatherQQMM, fast::Quantize and
+// fast::ConvertFP8
 // (mlx/primitives.h:1616-1717, mlx/fast_primitives.h:337-371), in the affine
 // mode and the floating-point modes mxfp4 / mxfp8 / nvfp4.
 //
@@ -523,6 +524,32 @@ void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
       ws_ptr,
       ws_bytes,
       enc.stream()));
+}
+
+// mx.to_fp8 / mx.from_fp8 (mlx/ops.cpp:5519-5552): elementwise, any shape.
+void fast::ConvertFP8::eval_gpu(
+    const std::vector<array>& inputs,
+    std::vector<array>& outputs) {
+  auto& s = stream();
+  auto& enc = rocm::get_command_encoder(s);
+  array in = ensure_row_contiguous(inputs[0], enc, s);
+  array& out = outputs[0];
+  out.set_data(allocator::malloc(out.nbytes()));
+  if (to_fp8_) {
+    rocm::check(mlxrocm_to_fp8(
+        rocm::gpu_ptr<void>(in, enc.stream()),
+        rocm::gpu_ptr<uint8_t>(out, enc.stream()),
+        in.size(),
+        dtype_code(in.dtype(), "to_fp8"),
+        enc.stream()));
+  } else {
+    rocm::check(mlxrocm_from_fp8(
+        rocm::gpu_ptr<uint8_t>(in, enc.stream()),
+        rocm::gpu_ptr<void>(out, enc.stream()),
+        in.size(),
+        dtype_code(out.dtype(), "from_fp8"),
+        enc.stream()));
+  }
 }
 
 void fast::Quantize::eval_gpu(

@@ -691,3 +691,38 @@ def test_global_scale_abi_rejects_bad_arguments(gpu):
     assert lib.mlxrocm_fp_gather_qqmm_workspace_size(2, 64, 3, 0) == 2 * 64 * 3 * 4
     # nothing to do
     assert lib.mlxrocm_nvfp4_quantize_global(None, p, None, None, 0, 0, None) == _lib.OK
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_to_fp8_and_from_fp8_bit_for_bit(fp_oracle, gpu, dtype):
+    """mx.to_fp8 / mx.from_fp8 against the reference's converters (the C port of
+    detail::ToFP8 / FromFP8, itself checked value by value against the reference's
+    translation unit): every bit pattern of the 16-bit types, sampled and edge
+    float32 values; every code back; lengths that are not a multiple of 8."""
+    port = fp_oracle.port
+    if dtype == torch.float32:
+        g = torch.Generator().manual_seed(3)
+        x = torch.randn(60001, generator=g) * torch.exp(torch.randn(60001, generator=g) * 4)
+        edge = torch.tensor([0.0, -0.0, 448.0, 447.9, 464.0, 465.0, 1e30, -1e30, float("inf"),
+                             float("-inf"), float("nan"), 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -10,
+                             0.015625, 0.0009765625, 17.0, 18.0, 19.0])
+        x = torch.cat([x, edge, -edge])
+    else:
+        x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+        x = torch.cat([x, x[:13]])  # a ragged tail
+    got = mlx_amd.to_fp8(x.to(gpu))
+    assert got.dtype == torch.uint8 and got.shape == x.shape
+    want = torch.tensor([port.fpq_to_fp8(float(v)) for v in x.float().tolist()], dtype=torch.uint8)
+    assert torch.equal(got.cpu(), want), dtype
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    for shape in ((256,), (4, 64), (251,)):
+        c = codes[: shape[0] * (shape[1] if len(shape) > 1 else 1)].reshape(shape)
+        back = mlx_amd.from_fp8(c.to(gpu), dtype)
+        vals = torch.tensor([port.fpq_from_fp8(int(v)) for v in c.flatten().tolist()]).reshape(shape)
+        assert back.dtype == dtype and torch.equal(back.cpu().float(), vals), (dtype, shape)
+    assert mlx_amd.from_fp8(codes.to(gpu)).dtype == torch.bfloat16  # the default
+    # python/tests/test_ops.py:4212-4217
+    vals = torch.tensor([448, 256, 192, 128, 96, 64, 48, 32, 24, 16, 12, 8, 6, 4, 3, 2, 0.015625])
+    for v in (vals, -vals):
+        assert torch.equal(mlx_amd.from_fp8(mlx_amd.to_fp8(v.to(dtype).to(gpu)), dtype).cpu().float(), v)
+    assert mlx_amd.to_fp8(torch.empty((0, 3), dtype=dtype, device=gpu)).shape == (0, 3)

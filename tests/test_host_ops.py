@@ -193,3 +193,17 @@ def test_gather_qqmm_errors():
         mlx_amd.gather_qqmm(x[0, 0], wq, sc, rhs_indices=idx)
     with pytest.raises(RuntimeError, match="GPU"):
         mlx_amd.gather_qqmm(x, wq, sc, rhs_indices=idx)
+
+
+def test_fp8_conversion_errors():
+    # mlx/ops.cpp:5519-5552
+    with pytest.raises(ValueError, match="Only real floating types"):
+        mlx_amd.to_fp8(torch.zeros(4, dtype=torch.int32))
+    with pytest.raises(ValueError, match="must have type uint8"):
+        mlx_amd.from_fp8(torch.zeros(4))
+    with pytest.raises(ValueError, match="Only real floating types"):
+        mlx_amd.from_fp8(torch.zeros(4, dtype=torch.uint8), torch.int32)
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.to_fp8(torch.zeros(4))
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlx_amd.from_fp8(torch.zeros(4, dtype=torch.uint8))
