@@ -109,6 +109,12 @@ __device__ __forceinline__ uint32_t fp4_nearest_even(float x) {
   return bits | sign;
 }
 
+// Mantissa bits of the float next to sqrt(2) (0x3FB504F3), and how far from it
+// the mantissa of a scale has to be for round(log2(scale)) to be decided without
+// evaluating the logarithm: 4096 steps of 2^-23 are 4.9e-4 in m, 5e-4 in log2(m).
+constexpr uint32_t kSqrt2Mant = 0x3504F3u;
+constexpr uint32_t kTieMargin = 4096u;
+
 // float log2, correctly rounded up to double rounding (evaluated in double)
 __device__ __forceinline__ float log2_rn(float x) {
   return static_cast<float>(log2(static_cast<double>(x)));
@@ -258,6 +264,8 @@ __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
   m = group_max(m, kLanes);
   float scale = m / (BITS == 4 ? 6.0f : 448.0f);
   uint32_t scale_byte;
+  float recip = 0.0f;
+  bool exact_recip = false;
   if constexpr (GS == 16) {
     scale_byte = to_fp8_bits(scale);
     scale = from_fp8_bits(scale_byte);
@@ -265,7 +273,19 @@ __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
     // to_fp8_e8m0 (:1049-1061): round(log2(scale)) half away from zero, clamped;
     // log2(0) = -inf clamps to -127, which decodes to 2^-127
     int n;
-    if (!(scale == scale) || fabsf(scale) == INFINITY) {
+    const uint32_t sbits = __float_as_uint(scale);
+    const uint32_t mant = sbits & 0x7fffffu;
+    if (sbits - 0x00800000u < 0x7e000000u &&
+        (mant < kSqrt2Mant - kTieMargin || mant > kSqrt2Mant + kTieMargin)) {
+      // a normal number 2^e m below 2^126, m in [1, 2), away from sqrt(2):
+      // log2 = e + log2(m) rounds to e below sqrt(2) and to e + 1 above, whatever
+      // the sign of e.  Evaluating log2 in float moves it by less than 2^-16; the
+      // margin keeps log2(m) 5e-4 away from one half.  The reciprocal of
+      // 2^n, |n| <= 126, is a normal float.
+      n = static_cast<int>(sbits >> 23) - 127 + (mant > kSqrt2Mant ? 1 : 0);
+      recip = __uint_as_float(static_cast<uint32_t>(127 - n) << 23);
+      exact_recip = true;
+    } else if (!(scale == scale) || fabsf(scale) == INFINITY) {
       n = 128; // code 0xFF: decodes to NaN as a bfloat16 pattern
     } else if (scale <= 0.0f) {
       n = -127;
@@ -280,11 +300,24 @@ __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
   if (!live) {
     return;
   }
+  // The scale of an MX mode is a power of two: multiplying by its reciprocal is
+  // the same single rounding as the reference's division.
+  if (exact_recip) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[i] *= recip;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[i] = scale == 0.0f ? 0.0f : v[i] / scale;
+    }
+  }
   if constexpr (CODES) {
     uint32_t lo = 0, hi = 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float w_el = scale == 0.0f ? 0.0f : v[i] / scale;
+      const float w_el = v[i];
       if constexpr (BITS == 8) {
         const uint32_t c = to_fp8_bits(w_el);
         if (i < 4) {
@@ -308,7 +341,7 @@ __global__ __launch_bounds__(kFpBlock) void fp_quantize_dequantize_kernel(
     float o[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float w_el = scale == 0.0f ? 0.0f : v[i] / scale;
+      const float w_el = v[i];
       const float val = BITS == 8 ? from_fp8_bits(to_fp8_bits(w_el))
                                   : fp4_value(fp4_nearest_even(w_el));
       o[i] = scale * val;

@@ -726,3 +726,55 @@ def test_to_fp8_and_from_fp8_bit_for_bit(fp_oracle, gpu, dtype):
     for v in (vals, -vals):
         assert torch.equal(mlx_amd.from_fp8(mlx_amd.to_fp8(v.to(dtype).to(gpu)), dtype).cpu().float(), v)
     assert mlx_amd.to_fp8(torch.empty((0, 3), dtype=dtype, device=gpu)).shape == (0, 3)
+
+
+@pytest.mark.parametrize("mode", ("mxfp4", "mxfp8"))
+def test_fp_quantize_dequantize_scales_next_to_a_tie_bit_for_bit(fp_oracle, gpu, mode):
+    """round(log2(scale)) flips where the scale's mantissa passes sqrt(2): groups
+    whose scale sits a few steps on either side of it (inside and outside the band
+    where the kernel evaluates the logarithm), over the whole exponent range,
+    subnormal scales and the largest finite values."""
+    from mlx_amd import _lib
+    from mlx_amd.ops import _DTYPE_CODE, _MODE_CODE
+
+    lib = _lib.load()
+    top = 6.0 if mode == "mxfp4" else 448.0
+    offs = (-70000, -4200, -4097, -4096, -4095, -300, -2, -1, 0, 1, 2, 300, 4095, 4096, 4097, 4200, 70000)
+    rows = []
+    g = torch.Generator().manual_seed(8)
+    for e in list(range(-126, 120, 5)) + [-126, -125, 118, 119]:
+        for off in offs:
+            bits = ((e + 127) << 23) | (0x3504F3 + off)
+            scale = torch.tensor([bits], dtype=torch.int32).view(torch.float32)
+            row = (torch.rand(32, generator=g) * 2 - 1) * scale * top
+            row[int(torch.randint(0, 32, (1,), generator=g))] = scale * top
+            rows.append(row)
+    # subnormal scales, zero, the largest finite elements
+    for amax in (1e-44, 3e-39, 1.2e-38 * top, 0.0, 3.4e38, 1.7e38):
+        row = (torch.rand(32, generator=g) * 2 - 1) * amax
+        row[3] = amax
+        rows.append(row)
+    x = torch.stack(rows)
+    x = torch.nan_to_num(x, nan=0.0, posinf=3.4e38, neginf=-3.4e38).contiguous()
+    xg = x.to(gpu)
+    out = torch.empty_like(xg)
+    _lib.check(lib.mlxrocm_fp_quantize_dequantize(
+        xg.data_ptr(), out.data_ptr(), xg.numel(), _MODE_CODE[mode], _DTYPE_CODE[torch.float32],
+        torch.cuda.current_stream().cuda_stream))
+    want = fp_oracle.quantize_dequantize(x, mode)
+    assert _equal_bits(out.cpu(), want), mode
+    # the same rule where x goes to codes for the block-scaled matrix instruction
+    # (16 rows or more, K a multiple of 128): against a diagonal w every output is
+    # one product, exact in float32, so the codes are checked bit for bit too
+    keep = (x.abs().amax(-1) < 1e12) & (x.abs().amax(-1) > 1e-12)
+    x2 = x[keep]
+    x2 = x2[: x2.shape[0] // 4 * 4].reshape(-1, 128)
+    assert x2.shape[0] >= 16
+    # e4m3 codes take the matrix instruction only for the 16-bit types
+    dtype = torch.float32 if mode == "mxfp4" else torch.bfloat16
+    x2 = x2.to(dtype)
+    wq, scales = mlx_amd.quantize(torch.eye(128, device=gpu, dtype=dtype), mode=mode)
+    y = mlx_amd.qqmm(x2.to(gpu), wq, scales, mode=mode)
+    w_hat = fp_qref.exact_fp_weights(wq.cpu(), scales.cpu(), mode)
+    want = (fp_oracle.quantize_dequantize(x2, mode).double() @ w_hat.T).to(dtype)
+    assert _equal_bits(y.cpu(), want), mode
