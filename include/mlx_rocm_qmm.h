@@ -266,7 +266,22 @@ int mlxrocm_fp_qqmm_plan(
  * mode != "affine"; CPU: mlx/backend/cpu/quantized.cpp:806-900 fp_bs_qmm_dispatch_mode).
  * Arguments as mlxrocm_gather_qmm without biases; pair i multiplies
  * x[lhs_indices[i]] by w[rhs_indices[i]]; a pair with an index out of range
- * writes zeros. */
+ * writes zeros.  workspace (optional, 256-byte aligned,
+ * mlxrocm_fp_gather_qmm_workspace_size bytes; batched_scales = scales_expert_stride
+ * != 0): with it, a call with one row of x per pair, a 16-bit dtype, transpose = 1
+ * and at least 32 pairs and four per expert sorts the pairs by expert and
+ * multiplies every expert's weights once for all its rows on the matrix cores;
+ * without it, or for other shapes, one streaming product per pair. */
+size_t mlxrocm_fp_gather_qmm_workspace_size(
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int n_experts,
+    int batched_scales,
+    int mode,
+    int dtype,
+    int transpose);
 int mlxrocm_fp_gather_qmm(
     const void* x,
     const uint32_t* wq,
@@ -286,6 +301,8 @@ int mlxrocm_fp_gather_qmm(
     int mode,
     int dtype,
     int transpose,
+    void* workspace,
+    size_t workspace_bytes,
     mlxrocm_stream_t stream);
 
 /*
@@ -310,10 +327,19 @@ int mlxrocm_from_fp8(
  * mlxrocm_fp_gather_qmm with transpose = 1; x_batch_stride >= M * K.
  * global_scale_x / global_scale_w: both null, or (nvfp4) both one float32 on
  * the device, as in mlxrocm_nvfp4_qqmm_global.  workspace:
- * mlxrocm_fp_gather_qqmm_workspace_size bytes (x_hat), 256-byte aligned, used
- * only during the call.
+ * mlxrocm_fp_gather_qqmm_workspace_size bytes (x_hat, then what
+ * mlxrocm_fp_gather_qmm asks for), 256-byte aligned, used only during the call.
  */
-size_t mlxrocm_fp_gather_qqmm_workspace_size(int M, int K, int x_batches, int dtype);
+size_t mlxrocm_fp_gather_qqmm_workspace_size(
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int x_batches,
+    int n_experts,
+    int batched_scales,
+    int mode,
+    int dtype);
 int mlxrocm_fp_gather_qqmm(
     const void* x,
     const uint32_t* wq,

@@ -62,8 +62,9 @@ SIGNATURES = {
     "mlxrocm_fp_qqmm": (_i, [_p] * 4 + [_i] * 5 + [_p, _sz, _p]),
     "mlxrocm_fp_qmm_plan": (_i, [_i] * 8 + [_sz, ctypes.c_char_p, _sz]),
     "mlxrocm_fp_qqmm_plan": (_i, [_i] * 5 + [_sz, ctypes.c_char_p, _sz]),
-    "mlxrocm_fp_gather_qmm": (_i, [_p] * 6 + [_i] * 6 + [_i64] * 3 + [_i] * 3 + [_p]),
-    "mlxrocm_fp_gather_qqmm_workspace_size": (_sz, [_i] * 4),
+    "mlxrocm_fp_gather_qmm_workspace_size": (_sz, [_i] * 9),
+    "mlxrocm_fp_gather_qmm": (_i, [_p] * 6 + [_i] * 6 + [_i64] * 3 + [_i] * 3 + [_p, _sz, _p]),
+    "mlxrocm_fp_gather_qqmm_workspace_size": (_sz, [_i] * 9),
     "mlxrocm_fp_gather_qqmm": (_i, [_p] * 8 + [_i] * 6 + [_i64] * 3 + [_i] * 2 + [_p, _sz, _p]),
     "mlxrocm_nvfp4_quantize_global": (_i, [_p] * 4 + [_sz, _i, _p]),
     "mlxrocm_nvfp4_dequantize_global": (_i, [_p] * 4 + [_sz, _i, _p]),

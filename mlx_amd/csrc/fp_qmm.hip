@@ -911,6 +911,49 @@ extern "C" size_t mlxrocm_fp_qmm_workspace_size(
 
 namespace {
 
+// A gather with one row of x per index pair and many pairs per expert is sorted
+// by expert (gather_group.hip) and multiplied by the tile kernel once per group
+// of up to 256 pairs, so that every expert's weights are read once for all the
+// rows routed to it, instead of one streaming product per pair.  The sort, the
+// scale images of the experts and the kernel's ramp cost about four products of
+// one pair per expert.  The kernel addresses x, an expert's codes and its scale
+// image with 32-bit byte offsets.
+bool fp_group_gather(
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int n_experts,
+    int x_batches,
+    int64_t x_batch_stride,
+    int mode,
+    int dtype,
+    bool transpose) {
+  if (M != 1 || !transpose || dtype == MLXROCM_FLOAT32 || K % 64 != 0 || K < 64) {
+    return false;
+  }
+  if (n_indices < 32 || static_cast<int64_t>(n_indices) < int64_t{4} * n_experts) {
+    return false;
+  }
+  const uint64_t bits = mode == MLXROCM_MXFP8 ? 8 : 4;
+  const uint64_t limit = uint64_t{1} << 32;
+  if ((static_cast<uint64_t>(x_batches) * static_cast<uint64_t>(x_batch_stride) + K) * 2 >= limit ||
+      static_cast<uint64_t>(N) * K * bits / 8 >= limit ||
+      static_cast<uint64_t>(N) * (K / 32) * 4 >= limit) {
+    return false;
+  }
+  if (gather_group_max_tiles(n_indices, n_experts, kGroupLargeTile) > 65535 || n_experts > 65535) {
+    return false;
+  }
+  return gather_group_workspace_bytes(n_indices, n_experts) > 0;
+}
+
+// Grouping tables, then the scale images of the experts (one when they share
+// their scales).
+size_t fp_group_gather_bytes(int N, int K, int n_indices, int n_experts, int images) {
+  return gather_group_workspace_bytes(n_indices, n_experts) + fp_image_bytes(N, K, images);
+}
+
 int fp_gather_entry(
     const void* x,
     const uint32_t* wq,
@@ -930,6 +973,8 @@ int fp_gather_entry(
     int mode,
     int dtype,
     int transpose,
+    void* workspace,
+    size_t workspace_bytes,
     mlxrocm_stream_t stream,
     const float* out_scale) {
   int rc = fp_check("gather_qmm", M, N, K, n_indices, mode, dtype, transpose);
@@ -954,6 +999,44 @@ int fp_gather_entry(
   if (!aligned16(x) || !aligned16(wq) || !aligned16(out) || x_batch_stride % x_vec != 0 ||
       w_expert_stride % 4 != 0) {
     return fail(MLXROCM_UNSUPPORTED, "[gather_qmm] operands must keep 16-byte alignment");
+  }
+  const int images = scales_expert_stride != 0 ? n_experts : 1;
+  if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0 &&
+      fp_group_gather(
+          M, N, K, n_indices, n_experts, x_batches, x_batch_stride, mode, dtype, transpose != 0) &&
+      workspace_bytes >= fp_group_gather_bytes(N, K, n_indices, n_experts, images)) {
+    QmmArgs a{};
+    a.x = x;
+    a.w = wq;
+    a.out = out;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.L = n_indices;
+    a.x_batch_stride = x_batch_stride;
+    a.w_batch_stride = w_expert_stride;
+    a.lhs_indices = lhs_indices;
+    a.rhs_indices = rhs_indices;
+    a.x_batches = x_batches;
+    a.n_experts = n_experts;
+    a.out_scale = out_scale;
+    // pairs with an index out of range are zero-filled by the grouping kernels
+    rc = launch_gather_group(a, dtype, kGroupLargeTile, workspace, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    void* image = static_cast<char*>(workspace) + gather_group_workspace_bytes(n_indices, n_experts);
+    rc = fp_scale_image_for_qmm_t(
+        scales, image, N, K, images, scales_expert_stride, mode, dtype, s);
+    if (rc != MLXROCM_OK) {
+      return rc;
+    }
+    a.scales = image;
+    a.biases = image;
+    a.sb_transposed = 2;
+    // elements of T between the images of two experts
+    a.sb_batch_stride = images > 1 ? static_cast<int64_t>(N) * (K / 32) * 2 : 0;
+    return launch_qmm_mfma_fp_grouped(a, mode, dtype, s);
   }
   constexpr int kMaxZ = 65535;
   for (int first = 0; first < n_indices; first += kMaxZ) {
@@ -1020,19 +1103,47 @@ extern "C" int mlxrocm_fp_gather_qmm(
     int mode,
     int dtype,
     int transpose,
+    void* workspace,
+    size_t workspace_bytes,
     mlxrocm_stream_t stream) {
   mlxrocm::ApiRange api_range("mlxrocm_fp_gather_qmm");
   return fp_gather_entry(
       x, wq, scales, lhs_indices, rhs_indices, out, M, N, K, n_indices, x_batches, n_experts,
-      x_batch_stride, w_expert_stride, scales_expert_stride, mode, dtype, transpose, stream,
-      nullptr);
+      x_batch_stride, w_expert_stride, scales_expert_stride, mode, dtype, transpose, workspace,
+      workspace_bytes, stream, nullptr);
 }
 
-extern "C" size_t mlxrocm_fp_gather_qqmm_workspace_size(int M, int K, int x_batches, int dtype) {
+extern "C" size_t mlxrocm_fp_gather_qmm_workspace_size(
+    int M,
+    int N,
+    int K,
+    int n_indices,
+    int n_experts,
+    int batched_scales,
+    int mode,
+    int dtype,
+    int transpose) {
+  if (fp_check("gather_qmm", M, N, K, n_indices, mode, dtype, transpose) != MLXROCM_OK ||
+      n_experts <= 0) {
+    return 0;
+  }
+  // x is assumed to be within reach of 32-bit offsets; a call whose x is not
+  // leaves the workspace unused
+  if (!fp_group_gather(M, N, K, n_indices, n_experts, 1, 0, mode, dtype, transpose != 0)) {
+    return 0;
+  }
+  return fp_group_gather_bytes(N, K, n_indices, n_experts, batched_scales ? n_experts : 1);
+}
+
+extern "C" size_t mlxrocm_fp_gather_qqmm_workspace_size(
+    int M, int N, int K, int n_indices, int x_batches, int n_experts, int batched_scales, int mode,
+    int dtype) {
   if (!valid_dtype(dtype) || M <= 0 || K <= 0 || x_batches <= 0) {
     return 0;
   }
-  return round256(static_cast<size_t>(x_batches) * M * K * dtype_size(dtype));
+  return round256(static_cast<size_t>(x_batches) * M * K * dtype_size(dtype)) +
+      mlxrocm_fp_gather_qmm_workspace_size(
+             M, N, K, n_indices, n_experts, batched_scales, mode, dtype, 1);
 }
 
 extern "C" int mlxrocm_fp_gather_qqmm(
@@ -1082,7 +1193,9 @@ extern "C" int mlxrocm_fp_gather_qqmm(
   if (x_batches <= 0 || x_batch_stride < rows_elems) {
     return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qqmm] invalid batch description");
   }
-  const size_t need = mlxrocm_fp_gather_qqmm_workspace_size(M, K, x_batches, dtype);
+  const size_t xhat_bytes = round256(static_cast<size_t>(x_batches) * M * K * dtype_size(dtype));
+  const size_t need = mlxrocm_fp_gather_qqmm_workspace_size(
+      M, N, K, n_indices, x_batches, n_experts, scales_expert_stride != 0, mode, dtype);
   if (workspace == nullptr || workspace_bytes < need ||
       (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) {
     return fail(
@@ -1108,7 +1221,8 @@ extern "C" int mlxrocm_fp_gather_qqmm(
   }
   return fp_gather_entry(
       workspace, wq, scales, lhs_indices, rhs_indices, out, M, N, K, n_indices, x_batches,
-      n_experts, rows_elems, w_expert_stride, scales_expert_stride, mode, dtype, 1, stream,
+      n_experts, rows_elems, w_expert_stride, scales_expert_stride, mode, dtype, 1,
+      static_cast<char*>(workspace) + xhat_bytes, workspace_bytes - xhat_bytes, stream,
       global_scale_w);
 }
 

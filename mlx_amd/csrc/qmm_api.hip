@@ -1353,7 +1353,8 @@ bool group_gather(
       (n_indices < 32 || static_cast<int64_t>(n_indices) < static_cast<int64_t>(n_experts))) {
     return false;
   }
-  if (static_cast<int64_t>(x_batches) * x_batch_stride + K >= (int64_t(1) << 32)) {
+  // the grouped kernels reach x through 32-bit byte offsets (16-bit elements)
+  if ((static_cast<int64_t>(x_batches) * x_batch_stride + K) * 2 >= (int64_t(1) << 32)) {
     return false;
   }
   if (gather_group_max_tiles(n_indices, n_experts, kGroupSmallTile) > 65535) {
@@ -1392,7 +1393,8 @@ bool group_gather_n(
   if (n_indices < 4) {
     return false;
   }
-  if (static_cast<int64_t>(x_batches) * x_batch_stride + K >= (int64_t(1) << 32)) {
+  // the grouped kernels reach x through 32-bit byte offsets (16-bit elements)
+  if ((static_cast<int64_t>(x_batches) * x_batch_stride + K) * 2 >= (int64_t(1) << 32)) {
     return false;
   }
   if (gather_group_max_tiles(n_indices, n_experts, kGroupLargeTile) > 65535) {

@@ -135,6 +135,9 @@ int fp_scale_image_for_qmm_t(
     int dtype,
     hipStream_t s);
 int launch_qmm_mfma_fp(const QmmArgs& a, int mode, int dtype, int k_splits, hipStream_t s);
+// The same kernel on a gather grouped by expert (launch_gather_group's tables in
+// `a`, one scale image per expert).
+int launch_qmm_mfma_fp_grouped(const QmmArgs& a, int mode, int dtype, hipStream_t s);
 
 // qqmm in the MX modes on the block-scaled matrix instruction (qq_mfma.hip):
 // x as codes and scale bytes (fp_quantize_activations, fp_quantize.hip) times

@@ -153,4 +153,27 @@ int launch_qmm_mfma_fp(const QmmArgs& a, int mode, int dtype, int k_splits, hipS
   return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
 }
 
+// Gather grouped by expert (M == 1 per index pair): `a` carries the tile list of
+// launch_gather_group and the scale images of all experts (a.sb_batch_stride
+// elements apart, 0 when the experts share one); one grid row per possible tile,
+// rows past the device-side tile count exit at once.
+int launch_qmm_mfma_fp_grouped(const QmmArgs& a, int mode, int dtype, hipStream_t s) {
+  MLXROCM_REHEARSE("fp_qmm_t_tile_grouped");
+  constexpr int kNT = 7;
+  const dim3 grid(
+      (a.N + 32 * kNT - 1) / (32 * kNT), gather_group_max_tiles(a.L, a.n_experts, kGroupLargeTile), 1);
+  auto run = [&](auto tval) -> int {
+    using T = decltype(tval);
+    switch (mode) {
+      case MLXROCM_MXFP4:
+        return launch_variant<T, T, T, 4, kNT, true, false, true, 1>(a, 5, grid, s);
+      case MLXROCM_MXFP8:
+        return launch_variant<T, T, T, 8, kNT, true, false, true, 2>(a, 5, grid, s);
+      default:
+        return launch_variant<T, T, T, 4, kNT, true, false, true, 3>(a, 5, grid, s);
+    }
+  };
+  return dtype == MLXROCM_BFLOAT16 ? run(bf16_t{}) : run(f16_t{});
+}
+
 } // namespace mlxrocm

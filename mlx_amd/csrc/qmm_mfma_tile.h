@@ -114,7 +114,9 @@ __global__ __launch_bounds__(kThreads) void qmm_t_mfma_kernel(
   static_assert(!(kSplit && GROUPED), "the grouped gather runs on 16-bit types only");
   static_assert(!(WN && kSplit), "[K, N] weights: 16-bit problems only");
   static_assert(!WN || BITS == 4 || BITS == 8, "[K, N] weights: 4- and 8-bit codes");
-  static_assert(!SBI || (!WN && !GROUPED && !kSplit && sizeof(TS) == 2), "pair image: plain 16-bit launches");
+  static_assert(
+      !SBI || (!WN && !kSplit && sizeof(TS) == 2 && (!GROUPED || FP != 0)),
+      "pair image: plain 16-bit launches, and the grouped gather of the fp modes");
   static_assert(FP == 0 || (SBI && BITS == (FP == 2 ? 8 : 4)), "fp codes: pair image, 4 or 8 bits");
   using DQ = std::conditional_t<FP != 0, FpPairDequant<T, (FP != 0 ? FP : 1)>, PairDequant<T, BITS>>;
   constexpr int kBN = 32 * NT;

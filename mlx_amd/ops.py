@@ -715,13 +715,19 @@ def gather_qmm(
             lhs_u = _as_uint32(lhs) if n_idx else lhs.reshape(-1)
         rhs_u = _as_uint32(rhs) if n_idx else rhs.reshape(-1)
         out = torch.empty(tuple(rhs.shape) + (M, w_outer), dtype=out_type, device=x.device)
+        ws_bytes = lib.mlxrocm_fp_gather_qmm_workspace_size(
+            M, w_outer, K, n_idx, wb.shape[0], int(sb_stride != 0), _MODE_CODE[mode],
+            _DTYPE_CODE[out_type], int(bool(transpose)),
+        )
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
         _lib.check(
             lib.mlxrocm_fp_gather_qmm(
                 xb.data_ptr(), wb.data_ptr(), sb.data_ptr(),
                 lhs_u.data_ptr() if n_idx else None, rhs_u.data_ptr() if n_idx else None,
                 out.data_ptr(), M, w_outer, K, n_idx, xb.shape[0], wb.shape[0],
                 M * K, w_stride, sb_stride, _MODE_CODE[mode], _DTYPE_CODE[out_type],
-                int(bool(transpose)), _stream_ptr(x),
+                int(bool(transpose)), ws.data_ptr() if ws is not None else None, ws_bytes,
+                _stream_ptr(x),
             )
         )
         return out
@@ -941,7 +947,9 @@ def gather_qqmm(
     rhs_u = _as_uint32(rhs) if n_idx else rhs.reshape(-1)
     out = torch.empty(tuple(rhs.shape) + (M, w_outer), dtype=x.dtype, device=x.device)
     code = _DTYPE_CODE[x.dtype]
-    ws_bytes = lib.mlxrocm_fp_gather_qqmm_workspace_size(M, K, xb.shape[0], code)
+    ws_bytes = lib.mlxrocm_fp_gather_qqmm_workspace_size(
+        M, w_outer, K, n_idx, xb.shape[0], wb.shape[0], int(sb_stride != 0), _MODE_CODE[mode], code
+    )
     ws = torch.empty(max(int(ws_bytes), 256), dtype=torch.uint8, device=x.device)
     _lib.check(
         lib.mlxrocm_fp_gather_qqmm(

@@ -399,7 +399,8 @@ void GatherQQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
   const int n_experts = (N == 0 || w.shape(-1) == 0)
       ? 0
       : static_cast<int>(w.size() / (size_t(w.shape(-1)) * w.shape(-2)));
-  const size_t ws_bytes = mlxrocm_fp_gather_qqmm_workspace_size(M, K, x_batches, dt);
+  const size_t ws_bytes = mlxrocm_fp_gather_qqmm_workspace_size(
+      M, N, K, n_idx, x_batches, n_experts, 1, mode, dt);
   void* ws_ptr = nullptr;
   if (ws_bytes > 0) {
     array ws = workspace_array(ws_bytes);
@@ -467,6 +468,15 @@ void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
   const int dt = dtype_code(x.dtype(), "gather_qmm");
 
   if (!affine) {
+    const int64_t scales_stride = scales.ndim() > 2 ? matrix_stride(scales) : 0;
+    const size_t fp_ws_bytes = mlxrocm_fp_gather_qmm_workspace_size(
+        M, N, K, n_idx, n_experts, scales_stride != 0, fp_mode_code(mode_), dt, transpose_ ? 1 : 0);
+    void* fp_ws = nullptr;
+    if (fp_ws_bytes > 0) {
+      array ws = workspace_array(fp_ws_bytes);
+      enc.add_temporary(ws);
+      fp_ws = rocm::gpu_ptr<void>(ws, enc.stream());
+    }
     rocm::check(mlxrocm_fp_gather_qmm(
         rocm::gpu_ptr<void>(x, enc.stream()),
         rocm::gpu_ptr<uint32_t>(w, enc.stream()),
@@ -482,10 +492,12 @@ void GatherQMM::eval_gpu(const std::vector<array>& inputs, array& out) {
         n_experts,
         int64_t(M) * K,
         w.ndim() > 2 ? matrix_stride(w) : 0,
-        scales.ndim() > 2 ? matrix_stride(scales) : 0,
+        scales_stride,
         fp_mode_code(mode_),
         dt,
         transpose_ ? 1 : 0,
+        fp_ws,
+        fp_ws_bytes,
         enc.stream()));
     return;
   }

@@ -330,7 +330,7 @@ def test_fp_gather_qmm_many_pairs_bad_indices_and_no_pairs(fp_oracle, gpu, mode)
     _lib.check(lib.mlxrocm_fp_gather_qmm(
         xg.data_ptr(), wq.data_ptr(), scales.data_ptr(), lhs_u.data_ptr(), rhs_u.data_ptr(),
         out.data_ptr(), 1, N, K, 3, 7, E, K, wq.stride(0), scales.stride(0), _MODE_CODE[mode],
-        _lib.FLOAT16, 1, torch.cuda.current_stream().cuda_stream))
+        _lib.FLOAT16, 1, None, 0, torch.cuda.current_stream().cuda_stream))
     assert float(out[1].abs().max()) == 0.0
     assert float(out[0].abs().max()) > 0.0 and float(out[2].abs().max()) > 0.0
     # no pairs
@@ -688,7 +688,8 @@ def test_global_scale_abi_rejects_bad_arguments(gpu):
         == _lib.INVALID_ARGUMENT
     assert lib.mlxrocm_fp_gather_qqmm(p, p, p, p, p, None, None, p, *args, _lib.MXFP4, 0, p, 16, None) \
         == _lib.INVALID_ARGUMENT
-    assert lib.mlxrocm_fp_gather_qqmm_workspace_size(2, 64, 3, 0) == 2 * 64 * 3 * 4
+    assert lib.mlxrocm_fp_gather_qqmm_workspace_size(2, 8, 64, 1, 3, 1, 0, _lib.MXFP4, 0) \
+        == 2 * 64 * 3 * 4
     # nothing to do
     assert lib.mlxrocm_nvfp4_quantize_global(None, p, None, None, 0, 0, None) == _lib.OK
 
@@ -778,3 +779,99 @@ def test_fp_quantize_dequantize_scales_next_to_a_tie_bit_for_bit(fp_oracle, gpu,
     w_hat = fp_qref.exact_fp_weights(wq.cpu(), scales.cpu(), mode)
     want = (fp_oracle.quantize_dequantize(x2, mode).double() @ w_hat.T).to(dtype)
     assert _equal_bits(y.cpu(), want), mode
+
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16), ids=str)
+@pytest.mark.parametrize("mode", MODES)
+def test_fp_gather_grouped_by_expert(gpu, mode, dtype):
+    """One row of x per pair and many pairs per expert: the pairs are sorted by
+    expert and every expert multiplied once on the matrix cores.  Every pair
+    against float64; an expert with no pair, one with more than a tile of 256,
+    pairs with an index out of range (zeros), ragged N, a sliced expert stack;
+    and the same call without a workspace (one product per pair)."""
+    from mlx_amd import _lib
+    from mlx_amd.ops import _DTYPE_CODE, _MODE_CODE
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(91)
+    E, N, K, T = 8, 300, 256, 40
+    w = torch.randn((E + 1, N, K), generator=g).to(dtype)
+    x = torch.randn((T, 1, K), generator=g).to(dtype)
+    wq_all, sc_all = mlx_amd.quantize(w.to(gpu), mode=mode)
+    wq, scales = wq_all[1:], sc_all[1:]  # a view that starts at the second expert
+    n_pairs = 900
+    lhs = torch.randint(0, T, (n_pairs,), generator=g, dtype=torch.int32)
+    # expert 3 gets no pair, expert 5 about 400 of them
+    rhs = torch.tensor([0, 1, 2, 4, 6, 7], dtype=torch.int32)[
+        torch.randint(0, 6, (n_pairs,), generator=g)]
+    rhs[::2][:400] = 5
+    lhs[17], rhs[18] = T + 3, E  # out of range
+    assert lib.mlxrocm_fp_gather_qmm_workspace_size(
+        1, N, K, n_pairs, E, 1, _MODE_CODE[mode], _DTYPE_CODE[dtype], 1) > 0
+    got = mlx_amd.gather_qmm(x.to(gpu), wq, scales, None, lhs.to(gpu), rhs.to(gpu), mode=mode)
+    assert got.shape == (n_pairs, 1, N) and got.dtype == dtype
+    assert float(got[17].abs().max()) == 0.0 and float(got[18].abs().max()) == 0.0
+    w_hat = fp_qref.exact_fp_weights(wq.cpu(), scales.cpu(), mode)  # [E, N, K]
+    ok = torch.ones(n_pairs, dtype=torch.bool)
+    ok[17] = ok[18] = False
+    li, ri = lhs[ok].long(), rhs[ok].long()
+    want = torch.einsum("pk,pnk->pn", x[li, 0].double(), w_hat[ri])
+    mag = torch.einsum("pk,pnk->pn", x[li, 0].double().abs(), w_hat[ri].abs()) + 1e-30
+    half_ulp = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    err = ((got[ok, 0].cpu().double() - want).abs() / mag).max().item()
+    assert err <= ACC_TOL[dtype] + half_ulp, (mode, dtype, err)
+    # the same pairs without a workspace: one streaming product per pair
+    xg, out = x.to(gpu).contiguous(), torch.empty((n_pairs, 1, N), dtype=dtype, device=gpu)
+    lhs_u, rhs_u = lhs.to(gpu).view(torch.uint32), rhs.to(gpu).view(torch.uint32)
+    _lib.check(lib.mlxrocm_fp_gather_qmm(
+        xg.data_ptr(), wq.data_ptr(), scales.data_ptr(), lhs_u.data_ptr(), rhs_u.data_ptr(),
+        out.data_ptr(), 1, N, K, n_pairs, T, E, K, wq.stride(0), scales.stride(0),
+        _MODE_CODE[mode], _DTYPE_CODE[dtype], 1, None, 0, torch.cuda.current_stream().cuda_stream))
+    perr = ((out[ok, 0].cpu().double() - got[ok, 0].cpu().double()).abs() / mag).max().item()
+    assert perr <= 2 * (ACC_TOL[dtype] + half_ulp), (mode, dtype, perr)
+    assert float(out[17].abs().max()) == 0.0 and float(out[18].abs().max()) == 0.0
+    # sorted indices, and fewer pairs than the rule asks for (not grouped): same answers
+    order = torch.argsort(rhs.long() * T + lhs.long())
+    got_sorted = mlx_amd.gather_qmm(x.to(gpu), wq, scales, None, lhs[order].to(gpu),
+                                    rhs[order].to(gpu), mode=mode, sorted_indices=True)
+    assert torch.equal(got_sorted, got[order.to(gpu)])
+    assert lib.mlxrocm_fp_gather_qmm_workspace_size(
+        1, N, K, 24, E, 1, _MODE_CODE[mode], _DTYPE_CODE[dtype], 1) == 0
+    few = mlx_amd.gather_qmm(x.to(gpu), wq, scales, None, lhs[:24].to(gpu), rhs[:24].to(gpu), mode=mode)
+    ferr = ((few[ok[:24], 0].cpu().double() - got[:24][ok[:24], 0].cpu().double()).abs()
+            / mag[: int(ok[:24].sum())]).max().item()
+    assert ferr <= 2 * (ACC_TOL[dtype] + half_ulp), (mode, dtype, ferr)
+
+
+@pytest.mark.parametrize("mode", ("mxfp4", "nvfp4"))
+def test_gather_qqmm_grouped_by_expert(fp_oracle, gpu, mode):
+    """gather_qqmm with enough pairs for the grouped route (nvfp4 with both
+    tensor-wide scales): every pair against float64 of x_hat times the decoded
+    expert."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(92)
+    E, N, K, T = 4, 96, 128, 64
+    w = torch.randn((E, N, K), generator=g).to(dtype)
+    x = torch.randn((T, 1, K), generator=g).to(dtype)
+    use_global = mode == "nvfp4"
+    gx = x.float().abs().max() if use_global else None
+    gw = w.float().abs().max() if use_global else None
+    wq, scales = mlx_amd.quantize(w.to(gpu), mode=mode,
+                                  **(dict(global_scale=gw.to(gpu)) if use_global else {}))
+    lhs = torch.arange(T, dtype=torch.int32).repeat_interleave(2)
+    rhs = torch.randint(0, E, (2 * T,), generator=g, dtype=torch.int32)
+    kw = dict(global_scale_x=gx.to(gpu), global_scale_w=gw.to(gpu)) if use_global else {}
+    got = mlx_amd.gather_qqmm(x.to(gpu), wq, scales, lhs.to(gpu), rhs.to(gpu), mode=mode, **kw)
+    assert got.shape == (2 * T, 1, N) and got.dtype == dtype
+    for i in range(2 * T):
+        xi, e = x[int(lhs[i])], int(rhs[i])
+        if use_global:
+            want, mag = fp_qref.nvfp4_global_qqmm_f64(xi, wq[e].cpu(), scales[e].cpu(),
+                                                      float(gx), float(gw))
+        else:
+            x_hat = fp_oracle.quantize_dequantize(xi, mode).double()
+            w_hat = fp_qref.exact_fp_weights(wq[e].cpu(), scales[e].cpu(), mode)
+            want, mag = x_hat @ w_hat.T, x_hat.abs() @ w_hat.abs().T
+        err = ((got[i].cpu().double() - want).abs() / (mag + 1e-30)).max().item()
+        assert err <= ACC_TOL[dtype] + 2.0 ** -8, (mode, i, err)
