@@ -524,16 +524,20 @@ def sweep(torch, mlx_amd, dev) -> list:
         add("f4", f"qqmm nvfp4 with global scales: x bfloat16 [{M},4096] W [14336,4096]", ms,
             flops=2.0 * M * 14336 * 4096)
     for mode in ("mxfp4", "nvfp4"):
-        E, T, topk = 8, 64, 2
+        E, topk = 8, 2
         w = (torch.randn((E, 14336, 4096), generator=g, dtype=torch.float32)).to(bf16).to(dev)
         q = mlx_amd.quantize(w, mode=mode)
         del w
-        x = torch.randn((T, 1, 4096), generator=g, dtype=torch.float32).to(bf16).to(dev)
-        lhs = torch.arange(T, dtype=torch.int32, device=dev).repeat_interleave(topk)
-        rhs = torch.randint(0, E, (T * topk,), generator=g, dtype=torch.int32).to(dev)
-        ms = timed(lambda i: mlx_amd.gather_qqmm(x, *q, lhs, rhs, mode=mode))
-        add("f4", f"gather_qqmm {mode}: T={T} top-{topk} of {E}, x bfloat16 [{T},1,4096] "
-            f"W [{E},14336,4096]", ms, flops=2.0 * T * topk * 14336 * 4096)
+        for T in (8, 64, 2048):
+            x = torch.randn((T, 1, 4096), generator=g, dtype=torch.float32).to(bf16).to(dev)
+            lhs = torch.arange(T, dtype=torch.int32, device=dev).repeat_interleave(topk)
+            rhs = torch.randint(0, E, (T * topk,), generator=g, dtype=torch.int32).to(dev)
+            ms = timed(lambda i: mlx_amd.gather_qmm(x, *q, None, lhs, rhs, mode=mode))
+            add("f4", f"gather_qmm {mode}: T={T} top-{topk} of {E}, x bfloat16 [{T},1,4096] "
+                f"W [{E},14336,4096]", ms, flops=2.0 * T * topk * 14336 * 4096)
+            ms = timed(lambda i: mlx_amd.gather_qqmm(x, *q, lhs, rhs, mode=mode))
+            add("f4", f"gather_qqmm {mode}: T={T} top-{topk} of {E}, x bfloat16 [{T},1,4096] "
+                f"W [{E},14336,4096]", ms, flops=2.0 * T * topk * 14336 * 4096)
         del q
 
     for mode in ("mxfp4", "mxfp8", "nvfp4"):
