@@ -875,3 +875,40 @@ def test_gather_qqmm_grouped_by_expert(fp_oracle, gpu, mode):
             want, mag = x_hat @ w_hat.T, x_hat.abs() @ w_hat.abs().T
         err = ((got[i].cpu().double() - want).abs() / (mag + 1e-30)).max().item()
         assert err <= ACC_TOL[dtype] + 2.0 ** -8, (mode, i, err)
+
+
+def test_fp_gather_full_size_moe_prefill(gpu):
+    """The expert-routed prefill at full size in mxfp4: 8 experts of
+    [14336, 4096], 2048 tokens, top-2 (4096 pairs, grouped by expert).  Every
+    pair against float64 on a spread of 384 output columns per expert, and
+    invariance under a permutation of the pairs."""
+    mode, dtype = "mxfp4", torch.bfloat16
+    g = torch.Generator().manual_seed(93)
+    E, N, K, T = 8, 14336, 4096, 2048
+    wq = torch.empty((E, N, K // 8), dtype=torch.uint32, device=gpu)
+    scales = torch.empty((E, N, K // 32), dtype=torch.uint8, device=gpu)
+    for e in range(E):  # one expert at a time: the unquantized stack would be 940 MB
+        w = (torch.randn((N, K), generator=g) * 0.05).to(dtype).to(gpu)
+        wq[e], scales[e] = mlx_amd.quantize(w, mode=mode)
+        del w
+    x = torch.randn((T, 1, K), generator=g).to(dtype)
+    lhs = torch.arange(T, dtype=torch.int32).repeat_interleave(2)
+    rhs = torch.stack([torch.randperm(E, generator=g)[:2] for _ in range(T)]).reshape(-1).to(torch.int32)
+    got = mlx_amd.gather_qmm(x.to(gpu), wq, scales, None, lhs.to(gpu), rhs.to(gpu), mode=mode)
+    assert got.shape == (2 * T, 1, N) and got.dtype == dtype
+    cols = torch.cat([torch.arange(0, 128), torch.arange(7000, 7128), torch.arange(N - 128, N)])
+    xd = x[:, 0].double()
+    for e in range(E):
+        wq_e = wq[e].view(torch.int32)[cols.to(gpu)].cpu().view(torch.uint32)
+        w_hat = fp_qref.exact_fp_weights(wq_e, scales[e][cols.to(gpu)].cpu(), mode)
+        pairs = torch.nonzero(rhs == e).flatten()
+        assert pairs.numel() > 256  # more than one tile of the grouped kernel
+        xe = xd[lhs[pairs].long()]
+        want = xe @ w_hat.T
+        mag = xe.abs() @ w_hat.abs().T + 1e-30
+        have = got[pairs.to(gpu), 0][:, cols.to(gpu)].cpu().double()
+        err = ((have - want).abs() / mag).max().item()
+        assert err <= ACC_TOL[dtype] + 2.0 ** -8, (e, err)
+    perm = torch.randperm(2 * T, generator=g)
+    again = mlx_amd.gather_qmm(x.to(gpu), wq, scales, None, lhs[perm].to(gpu), rhs[perm].to(gpu), mode=mode)
+    assert torch.equal(again, got[perm.to(gpu)])
