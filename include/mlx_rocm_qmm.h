@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MLXROCM_ABI_VERSION 3
+#define MLXROCM_ABI_VERSION 4
 
 typedef enum {
   MLXROCM_OK = 0,

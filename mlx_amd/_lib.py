@@ -135,7 +135,7 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
-    if lib.mlxrocm_abi_version() != 3:
+    if lib.mlxrocm_abi_version() != 4:
         raise ImportError("libmlx_rocm_qmm.so ABI version mismatch")
     _lib = lib
     return lib

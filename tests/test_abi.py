@@ -35,7 +35,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 
 def test_abi_version(lib):
-    assert lib.mlxrocm_abi_version() == 3
+    assert lib.mlxrocm_abi_version() == 4
 
 
 def test_invalid_arguments_are_reported_not_thrown(lib):
