@@ -311,8 +311,26 @@ __global__ __launch_bounds__(64 * kFp16Waves) void fp_qmv16_kernel(const QmmArgs
     wrow[r] = p.w + static_cast<size_t>(n) * row_bytes;
     srow[r] = p.scales + static_cast<size_t>(n) * groups;
   }
-  // every lane takes every step (the staged form has barriers inside): a lane
-  // whose codes lie past K multiplies zero codes
+  // The codes and scale bytes of a step are fetched one step ahead of their use,
+  // so that a wavefront always has two steps' loads in flight.  A lane whose
+  // codes lie past K fetches nothing and multiplies zero codes.
+  uint4 wv_next[RPW];
+  uint32_t sb_next[RPW][kGroups];
+  auto fetch_w = [&](int kb) {
+    const int kf = kb + lane * kCodes;
+    const bool in_range = kf < K;
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      wv_next[r] = in_range ? load_once(wrow[r] + static_cast<size_t>(kf) * BITS / 8)
+                            : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int g = 0; g < kGroups; ++g) {
+        sb_next[r][g] = in_range ? srow[r][kf / GS + g] : 0x7fu;
+      }
+    }
+  };
+  fetch_w(0);
+  // every lane takes every step (the staged form has barriers inside)
   for (int kbase = 0; kbase < K; kbase += 64 * kCodes) {
     const int k0 = kbase + lane * kCodes;
     const bool live = k0 < K;
@@ -325,12 +343,13 @@ __global__ __launch_bounds__(64 * kFp16Waves) void fp_qmv16_kernel(const QmmArgs
     uint32_t sb[RPW][kGroups];
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
-      wv[r] = live ? load_once(wrow[r] + static_cast<size_t>(k0) * BITS / 8) : make_uint4(0, 0, 0, 0);
+      wv[r] = wv_next[r];
 #pragma unroll
       for (int g = 0; g < kGroups; ++g) {
-        sb[r][g] = live ? srow[r][k0 / GS + g] : 0x7fu;
+        sb[r][g] = sb_next[r][g];
       }
     }
+    fetch_w(kbase + 64 * kCodes);
     // this lane's slice of the rows of x, as pairs
     uint32_t xr[MB][kPairs];
     if constexpr (XL) {
