@@ -67,6 +67,52 @@ __global__ __launch_bounds__(256) void fp_scale_image_kernel(
   }
 }
 
+// The same image four scale bytes per load: a workgroup takes 32 rows x 128
+// bytes of scales (128 groups, or 64 with two scales per 32 codes) through LDS.
+// Rows of scales must be whole dwords (G * PER % 4 == 0) and 4-byte aligned.
+template <typename T, int PER>
+__global__ __launch_bounds__(256) void fp_scale_image_wide_kernel(
+    const uint8_t* scales, uint32_t* out, int N, int G, int64_t src_stride) {
+  constexpr int kGroups = 128 / PER; // groups per workgroup
+  __shared__ uint32_t tile[32][kGroups + 1];
+  const int l = blockIdx.z;
+  const uint8_t* sc = scales + l * src_stride;
+  uint32_t* dst = out + static_cast<size_t>(l) * N * G;
+  const int tx = threadIdx.x & 31;
+  const int ty = threadIdx.x >> 5; // 0..7
+  const int g0 = blockIdx.x * kGroups;
+  const int n0 = blockIdx.y * 32;
+  const int row_bytes = G * PER;
+  const int c = g0 * PER + 4 * tx; // first of this thread's four bytes in a row
+#pragma unroll
+  for (int r = ty; r < 32; r += 8) {
+    const int n = n0 + r;
+    if (n < N && c < row_bytes) { // whole dwords: c + 3 < row_bytes as well
+      const uint32_t v =
+          *reinterpret_cast<const uint32_t*>(sc + static_cast<size_t>(n) * row_bytes + c);
+      if constexpr (PER == 2) {
+        tile[r][2 * tx] = scale_bits<T, true>(v & 0xffu) | (scale_bits<T, true>((v >> 8) & 0xffu) << 16);
+        tile[r][2 * tx + 1] =
+            scale_bits<T, true>((v >> 16) & 0xffu) | (scale_bits<T, true>(v >> 24) << 16);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t b = scale_bits<T, false>((v >> (8 * j)) & 0xffu);
+          tile[r][4 * tx + j] = b | (b << 16);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int r = ty; r < kGroups; r += 8) {
+    const int g = g0 + r;
+    const int n = n0 + tx;
+    if (n < N && g < G) {
+      dst[static_cast<size_t>(g) * N + n] = tile[tx][r];
+    }
+  }
+}
+
 } // namespace
 
 // `mode`: mlxrocm_fp_mode.  out: batches * (K / 32) * N dwords.
@@ -87,6 +133,27 @@ int fp_scale_image_for_qmm_t(
   }
   MLXROCM_REHEARSE("fp_scale_image");
   uint32_t* dst = static_cast<uint32_t*>(out);
+  const int per = mode == MLXROCM_NVFP4 ? 2 : 1;
+  if ((G * per) % 4 == 0 && (reinterpret_cast<uintptr_t>(scales) & 3u) == 0 && src_stride % 4 == 0) {
+    // whole dwords of scale bytes per row: four bytes per load
+    const int groups_per_block = 128 / per;
+    const dim3 wide((G + groups_per_block - 1) / groups_per_block, (N + 31) / 32, batches);
+    if (dtype == MLXROCM_BFLOAT16) {
+      if (per == 2) {
+        fp_scale_image_wide_kernel<bf16_t, 2><<<wide, 256, 0, s>>>(scales, dst, N, G, src_stride);
+      } else {
+        fp_scale_image_wide_kernel<bf16_t, 1><<<wide, 256, 0, s>>>(scales, dst, N, G, src_stride);
+      }
+    } else {
+      if (per == 2) {
+        fp_scale_image_wide_kernel<f16_t, 2><<<wide, 256, 0, s>>>(scales, dst, N, G, src_stride);
+      } else {
+        fp_scale_image_wide_kernel<f16_t, 1><<<wide, 256, 0, s>>>(scales, dst, N, G, src_stride);
+      }
+    }
+    MLXROCM_HIP_TRY(hipGetLastError());
+    return MLXROCM_OK;
+  }
   if (dtype == MLXROCM_BFLOAT16) {
     if (mode == MLXROCM_NVFP4) {
       fp_scale_image_kernel<bf16_t, 2><<<grid, 256, 0, s>>>(scales, dst, N, G, src_stride);
