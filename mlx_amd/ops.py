@@ -432,6 +432,31 @@ def quantized_swiglu(
     return out
 
 
+class _QuantizedMatmulVjp(torch.autograd.Function):
+    """The vector-Jacobian product of QuantizedMatmul with respect to x
+    (mlx/primitives.cpp:3532-3555): the cotangent times the same quantized
+    matrix with ``transpose`` flipped."""
+
+    @staticmethod
+    def forward(ctx, x, w, scales, biases, transpose, group_size, bits, mode, sb_image):
+        ctx.save_for_backward(w, scales, biases if biases is not None else scales)
+        ctx.args = (bool(transpose), group_size, bits, mode, biases is None, x.shape, x.dtype)
+        return _quantized_matmul(x, w, scales, biases, transpose, group_size, bits, mode, sb_image)
+
+    @staticmethod
+    def backward(ctx, cotangent):
+        w, scales, biases = ctx.saved_tensors
+        transpose, group_size, bits, mode, no_biases, x_shape, x_dtype = ctx.args
+        dx = _quantized_matmul(cotangent, w, scales, None if no_biases else biases,
+                               not transpose, group_size, bits, mode, None)
+        if tuple(dx.shape) != tuple(x_shape):
+            raise NotImplementedError(
+                "[QuantizedMatmul::vjp] x was broadcast against a batched weight: "
+                f"cotangent of shape {tuple(dx.shape)} for x of shape {tuple(x_shape)}"
+            )
+        return (_astype(dx, x_dtype),) + (None,) * 8
+
+
 def quantized_matmul(
     x: torch.Tensor,
     w: torch.Tensor,
@@ -447,7 +472,29 @@ def quantized_matmul(
     """``mx.quantized_matmul`` (mlx/ops.cpp:4784-4834).  ``sb_image`` (not in
     the reference): the result of :func:`quantized_matmul_sb_image` for these
     scales and biases, which saves prefill calls their transposition pre-pass;
-    results do not depend on it."""
+    results do not depend on it.  Under autograd the gradient with respect to x
+    is the reference's (QuantizedMatmul::vjp, mlx/primitives.cpp:3532-3555);
+    gradients with respect to scales and biases are not provided."""
+    if torch.is_grad_enabled():
+        wants = [t is not None and t.requires_grad for t in (scales, biases)]
+        if any(wants):
+            if mode != "affine":
+                # mlx/primitives.cpp:3562-3567
+                raise ValueError(
+                    f"[QuantizedMatmul::vjp] no gradient wrt scales in {mode} quantization."
+                )
+            raise NotImplementedError(
+                "[QuantizedMatmul::vjp] gradients wrt scales and biases are not provided "
+                "by mlx_amd (they need a dense matmul, which is outside this path)"
+            )
+        if x.requires_grad:
+            return _QuantizedMatmulVjp.apply(
+                x, w, scales, biases, transpose, group_size, bits, mode, sb_image
+            )
+    return _quantized_matmul(x, w, scales, biases, transpose, group_size, bits, mode, sb_image)
+
+
+def _quantized_matmul(x, w, scales, biases, transpose, group_size, bits, mode, sb_image):
     dtype, mode = _validate_mode_with_type("quantized_matmul", scales, biases, None, mode)
     group_size, bits = _params_from_mode(mode, group_size, bits)
     _, w_outer = _extract_dims(

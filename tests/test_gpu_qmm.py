@@ -650,3 +650,36 @@ def test_qmm_prepacked_scale_image(gpu, dtype):
     assert torch.equal(lin.prepack()(x), before)
     lin._set_quantized(w)
     assert torch.equal(lin(x), mlx_amd.quantized_matmul(x, wq, s, b, True, gs, 4))
+
+
+@pytest.mark.parametrize("dtype", (torch.float32, torch.bfloat16), ids=str)
+def test_vjp_with_respect_to_x(gpu, dtype):
+    """python/tests/test_quantized.py:480-508 (test_qmm_vjp): the gradient with
+    respect to x is the cotangent times the same quantized matrix with transpose
+    flipped; here under torch autograd, through the operator and the layer."""
+    g = torch.Generator().manual_seed(0)
+    M, N, K = 64, 1024, 512
+    c = torch.ones((2, M, N), dtype=dtype, device=gpu)
+    for transposed in (True, False):
+        w = torch.randn((N, K) if transposed else (K, N), generator=g).to(dtype).to(gpu)
+        wq, scales, biases = mlx_amd.quantize(w, 64, 8)
+        x = torch.randn((2, M, K), generator=g).to(dtype).to(gpu).requires_grad_(True)
+        y = mlx_amd.quantized_matmul(x, wq, scales, biases, transposed, 64, 8)
+        assert y.requires_grad
+        y.backward(c)
+        want = mlx_amd.quantized_matmul(c, wq, scales, biases, not transposed, 64, 8)
+        assert x.grad.shape == x.shape and x.grad.dtype == dtype
+        assert torch.equal(x.grad, want)
+    # the floating-point modes take the same route
+    wq, scales = mlx_amd.quantize(torch.randn((N, K), generator=g).to(dtype).to(gpu), mode="mxfp4")
+    x = torch.randn((3, K), generator=g).to(dtype).to(gpu).requires_grad_(True)
+    mlx_amd.quantized_matmul(x, wq, scales, mode="mxfp4").sum().backward()
+    want = mlx_amd.quantized_matmul(torch.ones((3, N), dtype=dtype, device=gpu), wq, scales,
+                                    transpose=False, mode="mxfp4")
+    assert torch.equal(x.grad, want)
+    # a frozen quantized layer between two trainable ones passes gradients through
+    lin = mlx_amd.nn.QuantizedLinear.from_linear(
+        torch.nn.Linear(K, N, bias=True).to(gpu).to(dtype), group_size=64, bits=4)
+    x = torch.randn((5, K), generator=g).to(dtype).to(gpu).requires_grad_(True)
+    lin(x).sum().backward()
+    assert x.grad is not None and float(x.grad.abs().max()) > 0

@@ -207,3 +207,23 @@ def test_fp8_conversion_errors():
         mlx_amd.to_fp8(torch.zeros(4))
     with pytest.raises(RuntimeError, match="GPU"):
         mlx_amd.from_fp8(torch.zeros(4, dtype=torch.uint8))
+
+
+def test_vjp_wrt_scales_is_refused():
+    # python/tests/test_quantized.py:1668-1694 (test_fp_vjp_scales_throws) and
+    # mlx/primitives.cpp:3556-3567
+    x = torch.zeros((2, 64))
+    wq = torch.zeros((8, 8), dtype=torch.uint32)
+    for mode, match, exc in (("mxfp4", "no gradient wrt scales in mxfp4", ValueError),
+                             ("mxfp8", "no gradient wrt scales in mxfp8", ValueError)):
+        sc = torch.zeros((8, 2), dtype=torch.float32, requires_grad=True)
+        with pytest.raises(exc, match=match):
+            mlx_amd.quantized_matmul(x, wq if mode == "mxfp4" else torch.zeros((8, 16), dtype=torch.uint32),
+                                     sc, mode=mode)
+    s = torch.zeros((8, 1), requires_grad=True)
+    b = torch.zeros((8, 1))
+    with pytest.raises(NotImplementedError, match="scales and biases"):
+        mlx_amd.quantized_matmul(x, wq, s, b)
+    with torch.no_grad():  # no graph is being recorded: the ordinary checks apply
+        with pytest.raises(RuntimeError, match="GPU"):
+            mlx_amd.quantized_matmul(x, wq, s, b)
