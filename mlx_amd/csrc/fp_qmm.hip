@@ -692,8 +692,16 @@ int fp_qmm_entry(
     return fail(MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] negative stride");
   }
   const int64_t x_vec = 16 / static_cast<int64_t>(dtype_size(dtype));
+  // [K, N] weights with a K that is not a multiple of 16 bytes: the kernel of that
+  // case reads x element by element, and a stack of such matrices cannot have an
+  // aligned stride
+  const bool x_by_elements = transpose == 0 && K % x_vec != 0;
+  // packed rows that are not whole 16-byte pieces are read by the byte
+  const int64_t row_bits = static_cast<int64_t>(transpose ? K : N) * (mode == MLXROCM_MXFP8 ? 8 : 4);
+  const bool w_by_bytes = row_bits % 128 != 0;
   if (!aligned16(x) || !aligned16(wq) || !aligned16(out) ||
-      (L > 1 && (x_batch_stride % x_vec != 0 || w_batch_stride % 4 != 0))) {
+      (L > 1 && ((!x_by_elements && x_batch_stride % x_vec != 0) ||
+                 (!w_by_bytes && w_batch_stride % 4 != 0)))) {
     return fail(MLXROCM_UNSUPPORTED, "[quantized_matmul] operands must keep 16-byte alignment");
   }
   QmmArgs a{};
@@ -1015,8 +1023,12 @@ int fp_gather_entry(
     return fail(MLXROCM_INVALID_ARGUMENT, "[gather_qmm] invalid batch description");
   }
   const int64_t x_vec = 16 / static_cast<int64_t>(dtype_size(dtype));
-  if (!aligned16(x) || !aligned16(wq) || !aligned16(out) || x_batch_stride % x_vec != 0 ||
-      w_expert_stride % 4 != 0) {
+  const bool x_by_elements = transpose == 0 && K % x_vec != 0; // as in quantized_matmul
+  const int64_t row_bits = static_cast<int64_t>(transpose ? K : N) * (mode == MLXROCM_MXFP8 ? 8 : 4);
+  const bool w_by_bytes = row_bits % 128 != 0;
+  if (!aligned16(x) || !aligned16(wq) || !aligned16(out) ||
+      (!x_by_elements && x_batch_stride % x_vec != 0) ||
+      (!w_by_bytes && w_expert_stride % 4 != 0)) {
     return fail(MLXROCM_UNSUPPORTED, "[gather_qmm] operands must keep 16-byte alignment");
   }
   const int images = scales_expert_stride != 0 ? n_experts : 1;

@@ -103,7 +103,8 @@ bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
-int check_alignment(const char* who, const QmmArgs& a, int dtype) {
+int check_alignment(
+    const char* who, const QmmArgs& a, int dtype, bool transpose = true, int bits = 0) {
   if (!aligned16(a.x) || !aligned16(a.w) || !aligned16(a.scales) ||
       !aligned16(a.biases) || !aligned16(a.out)) {
     return fail(
@@ -115,7 +116,18 @@ int check_alignment(const char* who, const QmmArgs& a, int dtype) {
   // one problem without indices never applies a batch stride (transpose=false
   // allows any K, so M * K need not be a multiple of 16 bytes there)
   const bool strided = a.L > 1 || a.lhs_indices != nullptr;
-  if (strided && (a.x_batch_stride % x_vec != 0 || a.w_batch_stride % 4 != 0)) {
+  // [K, N] weights with a K that is not a multiple of 16 bytes: the rows of x are
+  // unaligned anyway, the kernels of that case read x element by element, and a
+  // stack of such matrices (x [B, 1, 67]) cannot have an aligned stride
+  const bool x_by_elements = !transpose && a.K % x_vec != 0;
+  // likewise the packed rows: when a row is not a whole number of 16-byte pieces
+  // the kernels of that shape load words, and a stack of such matrices (three of
+  // [3, 32] at 6 bits: 18 words each) has no aligned stride either
+  const int64_t row_words = static_cast<int64_t>(transpose ? a.K : a.N) / 32 * bits;
+  const bool w_by_words = bits != 0 && row_words % 4 != 0;
+  if (strided &&
+      ((!x_by_elements && a.x_batch_stride % x_vec != 0) ||
+       (!w_by_words && a.w_batch_stride % 4 != 0))) {
     return fail(
         MLXROCM_UNSUPPORTED,
         "[%s] batch strides must keep 16-byte alignment (x stride %lld, w "
@@ -1076,7 +1088,7 @@ int qmm_entry(
       return fail(
           MLXROCM_INVALID_ARGUMENT, "[quantized_matmul] null device pointer");
     }
-    rc = check_alignment("quantized_matmul", a, dtype);
+    rc = check_alignment("quantized_matmul", a, dtype, transpose != 0, bits);
     if (rc != MLXROCM_OK) {
       return rc;
     }
@@ -1535,7 +1547,7 @@ int gather_entry(
   a.rhs_indices = rhs_indices;
   a.x_batches = x_batches;
   a.n_experts = n_experts;
-  rc = check_alignment("gather_qmm", a, dtype);
+  rc = check_alignment("gather_qmm", a, dtype, transpose != 0, bits);
   if (rc != MLXROCM_OK) {
     return rc;
   }

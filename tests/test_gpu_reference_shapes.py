@@ -1,0 +1,125 @@
+"""The shape grids of the reference's own quantized-matmul tests
+(python/tests/test_quantized.py), run the way they are written there: quantize,
+dequantize, and compare ``quantized_matmul`` with the dense product of the
+dequantized matrix under the reference's absolute tolerance.  The other GPU
+tests check the same kernels against the oracle at full sizes; these add the
+small, ragged and lopsided shapes the reference walks -- N of 3 .. 99, K of 3,
+8, 33 and 67 with ``transpose=False``, N beyond 2^15, M beyond 2^15, stacks of
+1, 3 and 8 weight matrices.  The dense product is float64 on the CPU."""
+import itertools
+
+import pytest
+import torch
+
+import mlx_amd
+
+pytestmark = pytest.mark.gpu
+
+FP_MODES = ("mxfp4", "nvfp4", "mxfp8")
+
+
+def _randn(shape, g, dtype=torch.float32, scale=1.0):
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _check(gpu, x, w, transpose, tol, group_size=None, bits=None, mode="affine"):
+    """quantized_matmul(x, quantize(w)) against x @ dequantize(quantize(w))."""
+    kw = dict(group_size=group_size, bits=bits, mode=mode)
+    q = mlx_amd.quantize(w.to(gpu), **kw)
+    if mode == "affine":
+        w_hat = mlx_amd.dequantize(*q, **kw)
+        y_q = mlx_amd.quantized_matmul(x.to(gpu), *q, transpose=transpose, **kw)
+    else:
+        w_hat = mlx_amd.dequantize(*q, **kw, dtype=torch.float32)
+        y_q = mlx_amd.quantized_matmul(x.to(gpu), *q, transpose=transpose, **kw)
+    w_hat = w_hat.cpu().double()
+    y_hat = x.double() @ (w_hat.transpose(-1, -2) if transpose else w_hat)
+    assert tuple(y_q.shape) == tuple(y_hat.shape), (x.shape, w.shape, transpose)
+    err = (y_q.cpu().double() - y_hat).abs().max().item() if y_hat.numel() else 0.0
+    assert err < tol, (tuple(x.shape), tuple(w.shape), transpose, group_size, bits, mode, err)
+
+
+def test_qmm_large_dims(gpu):
+    # :325-357 -- N beyond 2^15 and not a tile multiple; M beyond 2^15
+    g = torch.Generator().manual_seed(0)
+    K = 128
+    for M, N in ((16, 32840), (32, 32840), (33, 32840), (33000, 64)):
+        x = _randn((M, K), g, torch.float16, K ** -0.5)
+        w = _randn((N, K), g, torch.float16, K ** -0.5)
+        _check(gpu, x, w, True, 1.5e-3, 64, 4)
+
+
+def test_qmv_wide_grid(gpu):
+    # :678-753 -- 2..9 rows of x, ragged N, one and three weight matrices, every
+    # width and group size; then the fp modes; then tiny shapes
+    g = torch.Generator().manual_seed(1)
+    Ms, Ns, Bs = (2, 3, 4, 5, 6, 7, 9), (256, 67), (1, 3)
+    for gs, bits, K in itertools.product((32, 64, 128), (2, 3, 4, 5, 6, 8), (128, 512)):
+        for M, N, B in itertools.product(Ms, Ns, Bs):
+            x = _randn((M, K) if B == 1 else (B, M, K), g)
+            w = _randn((N, K) if B == 1 else (B, N, K), g)
+            _check(gpu, x, w, True, 1e-3, gs, bits)
+    for mode, K in itertools.product(FP_MODES, (128, 512)):
+        for M, N, B in itertools.product(Ms, Ns, Bs):
+            x = _randn((M, K) if B == 1 else (B, M, K), g)
+            w = _randn((N, K) if B == 1 else (B, N, K), g)
+            _check(gpu, x, w, True, 1e-3, mode=mode)
+    for M, K, N in ((2, 32, 10), (4, 32, 7), (3, 64, 5), (5, 64, 3)):
+        for bits, gs, mode in ((4, 32, "affine"), (6, 32, "affine"), (4, 16, "nvfp4")):
+            _check(gpu, _randn((M, K), g), _randn((N, K), g), True, 1e-3, gs, bits, mode)
+
+
+def test_small_matrix_and_non_multiples(gpu):
+    # :958-992 (test_small_matrix), :994-1066 (test_non_multiples)
+    g = torch.Generator().manual_seed(2)
+    for w_shape in ((8, 256), (1, 8, 256), (3, 8, 256)):
+        w = _randn(w_shape, g)
+        for x_shape in ((3, 1, 256), (3, 4, 256), (3, 10, 256)):
+            _check(gpu, _randn(x_shape, g), w, True, 1e-3)
+        for x_shape in ((3, 1, 8), (3, 10, 8)):
+            _check(gpu, _randn(x_shape, g), w, False, 1e-3)
+    for rows in (33, 3):
+        w = _randn((rows, 256), g)
+        for M in (1, 10):
+            _check(gpu, _randn((M, 256), g), w, True, 1e-3)
+            _check(gpu, _randn((M, rows), g), w, False, 1e-3)
+    _check(gpu, _randn((129, 256), g), _randn((99, 256), g), True, 1e-3)
+
+
+def test_qmv_small_non_multiples(gpu):
+    # :1068-1125 -- very small K and N, with and without a batch of weights
+    g = torch.Generator().manual_seed(3)
+    for M, K, N in ((1, 32, 3), (2, 32, 10), (1, 32, 5), (4, 32, 7)):
+        for bits, gs, mode in ((4, 32, "affine"), (6, 32, "affine"), (4, 16, "nvfp4")):
+            _check(gpu, _randn((M, K), g), _randn((N, K), g), True, 1e-3, gs, bits, mode)
+            _check(gpu, _randn((3, M, K), g), _randn((3, N, K), g), True, 1e-3, gs, bits, mode)
+
+
+def test_qvm_grid(gpu):
+    # :755-780 (test_qvm), :844-875 (test_fp_qvm): one row of x against [K, N]
+    # weights, K of 128, 256 and 67, stacks of 1, 3 and 8 matrices
+    g = torch.Generator().manual_seed(4)
+    for gs, bits, M, N, B in itertools.product(
+            (128, 64, 32), (2, 3, 4, 5, 6, 8), (32, 128, 256), (128, 256, 67), (0, 1, 3, 8)):
+        if M < gs:
+            continue
+        x = _randn((1, N) if B == 0 else (B, 1, N), g)
+        w = _randn((N, M) if B == 0 else (B, N, M), g)
+        _check(gpu, x, w, False, 1e-3, gs, bits)
+    cases = list(itertools.product((32, 128, 256), (128, 256, 67), (0, 1, 3, 8))) + [(128, 16384, 0)]
+    for (M, N, B), mode in itertools.product(cases, FP_MODES):
+        x = _randn((1, N) if B == 0 else (B, 1, N), g)
+        w = _randn((N, M) if B == 0 else (B, N, M), g)
+        _check(gpu, x, w, False, 2e-3, mode=mode)
+
+
+def test_qvm_split_k(gpu):
+    # :782-842 -- long K with transpose=False: one row and 2..3 rows of x; a 1-D x
+    g = torch.Generator().manual_seed(5)
+    for gs, bits, B in itertools.product((128, 64, 32), (2, 4, 8), (1, 3)):
+        x = _randn((B, 1, 16384), g, scale=0.1)
+        w = _randn((B, 16384, 128), g, scale=0.1)
+        _check(gpu, x, w, False, 2e-3, gs, bits)
+    _check(gpu, _randn((2048,), g, scale=0.1), _randn((2048, 2048), g, scale=0.1), False, 2e-3, 32, 8)
+    for gs, bits, K, M in itertools.product((64, 32), (4, 8), (2048, 4096), (2, 3)):
+        _check(gpu, _randn((M, K), g, scale=0.1), _randn((K, 128), g, scale=0.1), False, 2e-3, gs, bits)
