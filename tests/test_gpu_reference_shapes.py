@@ -123,3 +123,84 @@ def test_qvm_split_k(gpu):
     _check(gpu, _randn((2048,), g, scale=0.1), _randn((2048, 2048), g, scale=0.1), False, 2e-3, 32, 8)
     for gs, bits, K, M in itertools.product((64, 32), (4, 8), (2048, 4096), (2, 3)):
         _check(gpu, _randn((M, K), g, scale=0.1), _randn((K, 128), g, scale=0.1), False, 2e-3, gs, bits)
+
+
+def test_qmm_grid(gpu):
+    # :288-323 (test_qmm) -- both values of transpose, float16 as on the GPU there
+    g = torch.Generator().manual_seed(6)
+    for gs, bits, M, N, K, transposed in itertools.product(
+            (128, 64, 32), (2, 4, 8), (8, 32, 33, 64), (128, 256), (128, 256), (True, False)):
+        x = _randn((M, K), g, torch.float16, K ** -0.5)
+        w = _randn((N, K) if transposed else (K, N), g, torch.float16, K ** -0.5)
+        _check(gpu, x, w, transposed, 1.5e-3, gs, bits)
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16), ids=str)
+def test_qmm_non_transposed(gpu, dtype):
+    # :359-442 -- [K, N] weights over transformer-sized K / N and M values that
+    # leave partial tiles; affine and the fp modes; batched x; M beyond 2^15.
+    # bfloat16 results are compared at their own resolution.
+    g = torch.Generator().manual_seed(7)
+    tol = 1.5e-3 if dtype == torch.float16 else 1.2e-2
+
+    def affine(M, K, N, gs, bits, batch=()):
+        x = _randn(batch + (M, K), g, dtype, K ** -0.5)
+        _check(gpu, x, _randn((K, N), g, dtype, K ** -0.5), False, tol, gs, bits)
+
+    def fp(M, K, N, mode, batch=()):
+        x = _randn(batch + (M, K), g, dtype, K ** -0.5)
+        _check(gpu, x, _randn((K, N), g, dtype, K ** -0.5), False, tol, mode=mode)
+
+    for M in (1, 2, 31, 32, 33, 63, 64, 65, 96, 97, 100, 127, 128, 129):
+        for gs, bits in ((64, 4), (128, 4), (64, 8)):
+            affine(M, 512, 1024, gs, bits)
+        for mode in FP_MODES:
+            fp(M, 512, 1024, mode)
+    for K, N in ((2048, 2048), (512, 2048), (2048, 512), (11008, 2048)):
+        for M in (100, 256):
+            affine(M, K, N, 64, 4)
+    for batch in ((2,), (2, 3)):
+        for M in (33, 250):
+            affine(M, 512, 1024, 64, 4, batch)
+            for mode in FP_MODES:
+                fp(M, 512, 1024, mode, batch)
+    affine(33000, 128, 64, 64, 4)
+    fp(33000, 128, 64, "mxfp8")
+    for M, K in itertools.product((8, 33, 65), (64, 128, 256)):
+        for bits in (2, 4, 8):
+            affine(M, K, 128, 32, bits)
+        for mode in FP_MODES:
+            fp(M, K, 128, mode)
+
+
+def test_qmm_small_m_block_and_shapes(gpu):
+    # :444-478 (batched weights / an fp mode at 14 rows), :540-563 (test_qmm_shapes)
+    g = torch.Generator().manual_seed(8)
+    K = 1024
+    x = _randn((2, 14, K), g, torch.float16, K ** -0.5)
+    _check(gpu, x, _randn((2, 8256, K), g, torch.float16, K ** -0.5), True, 1e-3, 64, 4)
+    x = _randn((14, K), g, torch.bfloat16, K ** -0.5)
+    _check(gpu, x, _randn((8256, K), g, torch.bfloat16, K ** -0.5), True, 8e-3, mode="mxfp4")
+    for w_shape, transposed in (((32, 256), True), ((256, 256), False)):
+        w = _randn(w_shape, g)
+        for s in ((3, 256), (2, 1, 7, 256)):
+            _check(gpu, _randn(s, g), w, transposed, 1e-3, 64, 4)
+
+
+def test_qmv_grid(gpu):
+    # :565-590 (test_qmv), :592-641 (test_fp_qmv): one row of x per matrix, N of
+    # 256, 512, 67, 5 and 7, stacks of 1, 3 and 8 matrices, every width
+    g = torch.Generator().manual_seed(9)
+    for gs, bits, M, N, B in itertools.product(
+            (128, 64, 32), (2, 3, 4, 5, 6, 8), (256, 512, 67), (64, 256), (0, 1, 3, 8)):
+        if gs > N:
+            continue
+        x = _randn((3, 1, N) if B == 0 else (B, 1, N), g, scale=N ** -0.5)
+        w = _randn((M, N) if B == 0 else (B, M, N), g, scale=N ** -0.5)
+        _check(gpu, x, w, True, 1e-3, gs, bits)
+    for (M, N, B), mode in itertools.product(
+            itertools.product((256, 512, 67, 5, 7), (64, 256), (0, 1, 3, 8)), FP_MODES):
+        x = _randn((3, 1, N) if B == 0 else (B, 1, N), g)
+        w = _randn((M, N) if B == 0 else (B, M, N), g)
+        _check(gpu, x, w, True, 1e-3, mode=mode)
+    _check(gpu, _randn((1, 48), g), _randn((128, 48), g), True, 1e-3, mode="nvfp4")
