@@ -204,3 +204,29 @@ def test_qmv_grid(gpu):
         w = _randn((M, N) if B == 0 else (B, M, N), g)
         _check(gpu, x, w, True, 1e-3, mode=mode)
     _check(gpu, _randn((1, 48), g), _randn((128, 48), g), True, 1e-3, mode="nvfp4")
+
+
+def test_qmm_fp_type_and_strided_scales(gpu):
+    # :1362-1379 (test_qmm_fp_type): the result has the type of x, also through
+    # gather_qmm with a 2-D x and [3, 1] expert indices; :1696-1706
+    # (test_quantize_strided): scales that are a broadcast view
+    g = torch.Generator().manual_seed(10)
+    indices = torch.tensor([[2], [0], [1]], dtype=torch.int32, device=gpu)
+    for mode in ("mxfp8", "mxfp4"):
+        for t in (torch.bfloat16, torch.float16, torch.float32):
+            x = _randn((32, 256), g, t).to(gpu)
+            wq, s = mlx_amd.quantize(_randn((32, 256), g).to(gpu), mode=mode)
+            assert mlx_amd.quantized_matmul(x, wq, s, mode=mode).dtype == t
+            wq, s = mlx_amd.quantize(_randn((4, 32, 256), g).to(gpu), mode=mode)
+            out = mlx_amd.gather_qmm(x, wq, s, rhs_indices=indices, mode=mode)
+            assert out.dtype == t and tuple(out.shape) == (3, 1, 32, 32)
+            w_hat = mlx_amd.dequantize(wq, s, mode=mode, dtype=torch.float32).cpu().double()
+            for i, e in enumerate((2, 0, 1)):
+                want = x.cpu().double() @ w_hat[e].T
+                tol = {torch.float32: 1e-3, torch.float16: 3e-2, torch.bfloat16: 2.5e-1}[t]
+                assert (out[i, 0].cpu().double() - want).abs().max().item() < tol, (mode, t, i)
+    w_q, scales = mlx_amd.quantize(_randn((64, 64), g).to(gpu), mode="nvfp4")
+    flat = torch.tensor(56, dtype=torch.uint8, device=gpu).expand(scales.shape)
+    w_hat = mlx_amd.dequantize(w_q, flat, mode="nvfp4")
+    expected = mlx_amd.dequantize(w_q, flat.contiguous(), mode="nvfp4")
+    assert torch.equal(w_hat, expected)
