@@ -595,7 +595,31 @@ size_t fp_tile_workspace(int M, int N, int K, int L, int batches) {
 
 // L problems (batch entries or index pairs), at most 65535 per launch.
 int fp_launch(const QmmArgs& a, int mode, int dtype, bool transpose, hipStream_t s) {
-  if (a.L > 65535 || a.M > 65535 * kFpRowBlock) {
+  constexpr int kMaxRows = 65535; // the kernels below use up to one grid row per row of x
+  if (a.M > kMaxRows && a.lhs_indices == nullptr && a.L <= 65535) {
+    // more rows of x than a grid is deep: one problem at a time, in slices of rows
+    const size_t esize = dtype_size(dtype);
+    for (int l = 0; l < a.L; ++l) {
+      for (int m0 = 0; m0 < a.M; m0 += kMaxRows) {
+        QmmArgs part = a;
+        part.L = 1;
+        part.M = a.M - m0 < kMaxRows ? a.M - m0 : kMaxRows;
+        part.x = static_cast<const char*>(a.x) +
+            (static_cast<size_t>(l) * a.x_batch_stride + static_cast<size_t>(m0) * a.K) * esize;
+        part.w = a.w + static_cast<size_t>(l) * a.w_batch_stride;
+        part.scales = static_cast<const uint8_t*>(a.scales) +
+            static_cast<size_t>(l) * a.sb_batch_stride;
+        part.out = static_cast<char*>(a.out) +
+            (static_cast<size_t>(l) * a.M + m0) * static_cast<size_t>(a.N) * esize;
+        const int rc = fp_launch(part, mode, dtype, transpose, s);
+        if (rc != MLXROCM_OK) {
+          return rc;
+        }
+      }
+    }
+    return MLXROCM_OK;
+  }
+  if (a.L > 65535 || a.M > kMaxRows) {
     return fail(MLXROCM_UNSUPPORTED, "[quantized_matmul] M=%d or batch=%d exceed the grid", a.M, a.L);
   }
   return dispatch_dtype(dtype, [&](auto tval) {

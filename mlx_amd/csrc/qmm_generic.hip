@@ -210,6 +210,32 @@ int launch_qmm_naive(
     int dtype,
     bool transpose,
     hipStream_t s) {
+  constexpr int kMaxRows = 65535; // one grid row per row of x
+  if (a.M > kMaxRows && a.lhs_indices == nullptr && a.L <= kMaxRows) {
+    // more rows of x than a grid is deep: one problem at a time, in slices of rows
+    const size_t esize = dtype_size(dtype);
+    for (int l = 0; l < a.L; ++l) {
+      for (int m0 = 0; m0 < a.M; m0 += kMaxRows) {
+        QmmArgs part = a;
+        part.L = 1;
+        part.M = a.M - m0 < kMaxRows ? a.M - m0 : kMaxRows;
+        part.x = static_cast<const char*>(a.x) +
+            (static_cast<size_t>(l) * a.x_batch_stride + static_cast<size_t>(m0) * a.K) * esize;
+        part.w = a.w + static_cast<size_t>(l) * a.w_batch_stride;
+        part.scales = static_cast<const char*>(a.scales) +
+            static_cast<size_t>(l) * a.sb_batch_stride * esize;
+        part.biases = static_cast<const char*>(a.biases) +
+            static_cast<size_t>(l) * a.sb_batch_stride * esize;
+        part.out = static_cast<char*>(a.out) +
+            (static_cast<size_t>(l) * a.M + m0) * static_cast<size_t>(a.N) * esize;
+        const int rc = launch_qmm_naive(part, gs, bits, dtype, transpose, s);
+        if (rc != MLXROCM_OK) {
+          return rc;
+        }
+      }
+    }
+    return MLXROCM_OK;
+  }
   const int cols = transpose ? a.N : a.N / 8;
   const dim3 grid((cols + 255) / 256, a.M, a.L);
   if (grid.y > 65535u || grid.z > 65535u) {

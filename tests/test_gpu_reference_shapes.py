@@ -230,3 +230,19 @@ def test_qmm_fp_type_and_strided_scales(gpu):
     w_hat = mlx_amd.dequantize(w_q, flat, mode="nvfp4")
     expected = mlx_amd.dequantize(w_q, flat.contiguous(), mode="nvfp4")
     assert torch.equal(w_hat, expected)
+
+
+def test_more_rows_of_x_than_a_grid_is_deep(gpu):
+    """70,000 rows of x through the kernels that use one grid row per row of x
+    (K not a multiple of 64, [K, N] weights with an odd K, the fp modes' streaming
+    kernels): the launches are cut into slices of rows on the host."""
+    g = torch.Generator().manual_seed(11)
+    M = 70000
+    _check(gpu, _randn((M, 32), g), _randn((40, 32), g), True, 1e-3, 32, 4)
+    _check(gpu, _randn((M, 5), g), _randn((5, 64), g), False, 1e-3, 32, 4)
+    _check(gpu, _randn((2, M, 5), g), _randn((2, 5, 64), g), False, 1e-3, 32, 8)
+    _check(gpu, _randn((M, 64), g), _randn((24, 64), g), True, 1e-3, mode="mxfp4")
+    _check(gpu, _randn((M, 48), g), _randn((24, 48), g), True, 1e-3, mode="nvfp4")
+    _check(gpu, _randn((M, 7), g), _randn((7, 64), g), False, 1e-3, mode="mxfp8")
+    _check(gpu, _randn((M, 64), g, torch.bfloat16), _randn((24, 64), g, torch.bfloat16), True, 0.15,
+           mode="mxfp8")
