@@ -193,3 +193,49 @@ def test_fp_qmm_workspace_size_is_exact_and_plans_name_the_kernels():
     assert _lib.fp_qqmm_plan(64, 128, 96, _lib.MXFP4, bf16)[1].startswith("fp_quantize_dequantize+")
     assert _lib.fp_qqmm_plan(8192, 14336, 4096, _lib.NVFP4, bf16)[1] == \
         "fp_quantize_dequantize+fp_scale_image+fp_qmm_t_tile(nt=7)"
+
+
+def test_no_valid_shape_is_refused():
+    """A seeded random walk over valid shapes -- rows of x from 1 to 300,000, N from
+    1 to 70,001, ragged K with [K, N] weights, stacks of matrices, every width,
+    group size, element type and fp mode -- through the rehearsal of the entry
+    points: every call is accepted (shapes the kernels cannot take in one launch
+    are cut up on the host, never refused)."""
+    import random
+
+    from mlx_amd import _lib
+
+    rnd = random.Random(1)
+    rows = (1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 255,
+            256, 257, 500, 1000, 2048, 4097, 70000, 300000)
+    outer = (1, 2, 3, 5, 7, 8, 9, 31, 32, 33, 64, 67, 100, 127, 128, 255, 256, 1000, 4096, 11008,
+             32840, 70001)
+    inner = (1, 2, 3, 5, 7, 8, 9, 31, 32, 33, 64, 67, 100, 127, 128, 255, 256, 1000, 4096, 11008)
+
+    def quantized_dim(gs):
+        return gs * rnd.randint(1, max(1, rnd.choice((128, 512, 4096, 16384)) // gs))
+
+    refused = []
+    for _ in range(6000):
+        transpose = rnd.random() < 0.6
+        M, L = rnd.choice(rows), rnd.choice((1, 1, 1, 2, 3, 8))
+        batched = L > 1 and rnd.random() < 0.5
+        dtype = rnd.choice((_lib.FLOAT32, _lib.FLOAT16, _lib.BFLOAT16))
+        if rnd.random() < 0.6:
+            gs, bits = rnd.choice((32, 64, 128)), rnd.choice((2, 3, 4, 5, 6, 8))
+            N, K = (rnd.choice(outer), quantized_dim(gs)) if transpose else \
+                (quantized_dim(gs), rnd.choice(inner))
+            rc, _ = _lib.qmm_plan(M, N, K, L, batched, gs, bits, dtype, transpose)
+            case = ("affine", M, N, K, L, batched, gs, bits, dtype, transpose)
+        else:
+            mode = rnd.choice((_lib.MXFP4, _lib.MXFP8, _lib.NVFP4))
+            gs = 16 if mode == _lib.NVFP4 else 32
+            N, K = (rnd.choice(outer), quantized_dim(gs)) if transpose else \
+                (quantized_dim(gs), rnd.choice(inner))
+            rc, _ = _lib.fp_qmm_plan(M, N, K, L, batched, mode, dtype, transpose)
+            case = ("fp", M, N, K, L, batched, mode, dtype, transpose)
+            if rc == 0 and transpose and L == 1:
+                rc, _ = _lib.fp_qqmm_plan(M, N, K, mode, dtype)
+        if rc != 0:
+            refused.append((case, _lib.last_error()))
+    assert not refused, refused[:5]
