@@ -246,3 +246,21 @@ def test_more_rows_of_x_than_a_grid_is_deep(gpu):
     _check(gpu, _randn((M, 7), g), _randn((7, 64), g), False, 1e-3, mode="mxfp8")
     _check(gpu, _randn((M, 64), g, torch.bfloat16), _randn((24, 64), g, torch.bfloat16), True, 0.15,
            mode="mxfp8")
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16), ids=str)
+def test_stacks_with_unaligned_rows_sixteen_bit(gpu, dtype):
+    """Stacks of [K, N] weights with K = 67 and of x [B, M, 67] in the 16-bit
+    types (batch strides of 134 and 1340 bytes), and stacks of tiny packed
+    matrices (18 words each): accepted and right."""
+    g = torch.Generator().manual_seed(12)
+    tol = 4e-3 if dtype == torch.float16 else 3e-2  # results of magnitude ~1 at their own resolution
+    for M in (1, 3, 10):
+        def x_of(K):
+            return _randn((3, M, K), g, dtype, K ** -0.5)
+
+        for bits, gs in ((4, 64), (3, 32), (8, 128)):
+            _check(gpu, x_of(67), _randn((3, 67, 128), g, dtype), False, tol, gs, bits)
+        _check(gpu, x_of(67), _randn((3, 67, 128), g, dtype), False, tol, mode="mxfp4")
+        _check(gpu, x_of(32), _randn((3, 3, 32), g, dtype), True, tol, 32, 6)
+        _check(gpu, x_of(48), _randn((3, 5, 48), g, dtype), True, tol, mode="nvfp4")
